@@ -1,0 +1,631 @@
+// Neighbor-partitioned aggregation (SpMM) for gfx950, wave64.
+//
+// Work decomposition
+//   partition  <= ps neighbors of one destination row (MGG's neighbor partition)
+//   slot       LPR adjacent lanes of a wavefront that together hold one feature
+//              row (16 bytes per lane on the vector paths); a slot sums one
+//              partition per round, so a wavefront sums S = 64/LPR partitions
+//              at once and every gather instruction touches S feature rows
+//   round      the S partitions a wavefront works on together; a wavefront
+//              runs `dist` consecutive rounds (MGG's interleaved_dist)
+//   workgroup  wpb wavefronts = wpb*S*dist consecutive partitions
+// Partitions are laid out row-major (a row's local partitions, then its remote
+// ones), so the partitions of one row are adjacent and every level combines
+// neighbors only:
+//   slots      segmented scan over the slots of a round (cross-lane moves)
+//   rounds     a wavefront carries its open row from round to round in registers
+//   wavefronts a row that crosses wavefronts is finished through LDS
+//   workgroups a row that crosses workgroups leaves two partial rows in a
+//              carry buffer; a small second kernel sums them in a fixed order
+// No atomics anywhere; the summation order depends only on (ps, wpb, dist, dim).
+#include <type_traits>
+
+#include "mggx_dev.h"
+
+namespace mggx {
+namespace {
+
+constexpr int HDR_VALID = 1;   // entry holds a partial row
+constexpr int HDR_ENDS = 2;    // head entry: the row ends inside this unit
+constexpr int HDR_STARTS = 4;  // tail entry: the row started inside this unit
+
+constexpr int MODE_F32_VEC4 = 0;     // fp32 rows, one 16-byte load per lane
+constexpr int MODE_F32_STRIDED = 1;  // fp32 rows of any width/alignment, dword loads, lane-strided
+constexpr int MODE_BF16_VEC8 = 2;    // bf16 rows, one 16-byte load (8 values) per lane, fp32 accumulation
+
+struct AggArgs {
+    float *out;
+    const void *in_l;
+    const void *in_r;
+    const int *col_l;
+    const int *col_r;
+    const int4 *desc;
+    const int *off;
+    const float *rs_out;
+    int2 *c_hdr;   // [2 * workgroups]: head, tail
+    float *c_val;  // [2 * workgroups][cpad]
+    long long ld_in, ld_out;
+    int num_parts;
+    int nnz_l, nnz_r;
+    int lb, dim, ps, dist, cpad;
+    int parts_per_wg;
+    unsigned flags;
+    float eps;
+    int in_is_bf16;
+};
+
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+__device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & 63u); }
+
+// value of lane `src` (any lane of the wavefront)
+__device__ __forceinline__ int lane_read(int v, int src) { return __builtin_amdgcn_ds_bpermute(src << 2, v); }
+__device__ __forceinline__ float lane_read(float v, int src)
+{
+    return __int_as_float(__builtin_amdgcn_ds_bpermute(src << 2, __float_as_int(v)));
+}
+
+// Broadcast the value held by lane SRC of each slot to the whole slot.
+template <int LPR, int SRC>
+__device__ __forceinline__ int slot_bcast(int v, int slot_base)
+{
+    if constexpr (LPR == 1) {
+        return v;
+    } else if constexpr (LPR == 2) {
+        return __builtin_amdgcn_update_dpp(0, v, SRC | (SRC << 2) | ((2 + SRC) << 4) | ((2 + SRC) << 6), 0xf, 0xf, false);
+    } else if constexpr (LPR == 4) {
+        return __builtin_amdgcn_update_dpp(0, v, SRC | (SRC << 2) | (SRC << 4) | (SRC << 6), 0xf, 0xf, false);
+    } else if constexpr (LPR == 64) {
+        return __builtin_amdgcn_readlane(v, SRC);
+    } else {
+        return lane_read(v, slot_base + SRC);
+    }
+}
+
+template <int MODE>
+struct ModeTraits {
+    static constexpr int NV = MODE == MODE_BF16_VEC8 ? 8 : 4;
+};
+
+// feature index of value i held by lane l of a slot
+template <int LPR, int MODE>
+__device__ __forceinline__ int elem_of(int l, int i)
+{
+    if constexpr (MODE == MODE_F32_STRIDED) return l + i * LPR;
+    else return ModeTraits<MODE>::NV * l + i;
+}
+
+// Unconditional load of this lane's share of table row `r`; lanes past the row
+// width read lane 0's share instead (their values are never used).
+template <int LPR, int MODE>
+__device__ __forceinline__ void gather_row(float (&v)[ModeTraits<MODE>::NV], const void *tbl, long long r, long long ld,
+                                           int l, int dim)
+{
+    constexpr int NV = ModeTraits<MODE>::NV;
+    if constexpr (MODE == MODE_F32_VEC4) {
+        const int le = (NV * l < dim) ? l : 0;
+        const float4 t = *reinterpret_cast<const float4 *>(static_cast<const float *>(tbl) + r * ld + 4 * le);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    } else if constexpr (MODE == MODE_F32_STRIDED) {
+        const float *p = static_cast<const float *>(tbl) + r * ld;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int d = l + i * LPR;
+            v[i] = p[d < dim ? d : 0];
+        }
+    } else {
+        const int le = (NV * l < dim) ? l : 0;
+        const uint4 t = *reinterpret_cast<const uint4 *>(static_cast<const unsigned short *>(tbl) + r * ld + 8 * le);
+        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xFFFF0000u);
+        v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xFFFF0000u);
+        v[4] = __uint_as_float(t.z << 16); v[5] = __uint_as_float(t.z & 0xFFFF0000u);
+        v[6] = __uint_as_float(t.w << 16); v[7] = __uint_as_float(t.w & 0xFFFF0000u);
+    }
+}
+
+__device__ __forceinline__ float load_self(const AggArgs &a, int row, int d)
+{
+    if (a.in_is_bf16) {
+        const unsigned short h = static_cast<const unsigned short *>(a.in_l)[(long long)row * a.ld_in + d];
+        return __uint_as_float((unsigned)h << 16);
+    }
+    return static_cast<const float *>(a.in_l)[(long long)row * a.ld_in + d];
+}
+
+// Finishes one output element: scale, GIN self term, accumulate, ReLU, store.
+__device__ __forceinline__ void finish_elem(const AggArgs &a, int row, int d, float sum)
+{
+    float v = a.rs_out ? sum * a.rs_out[row] : sum;
+    if (a.flags & MGGX_AGG_GIN) v += (1.0f + a.eps) * load_self(a, row, d);
+    float *o = a.out + (long long)row * a.ld_out + d;
+    if (a.flags & MGGX_AGG_ACCUMULATE) v += *o;
+    if (a.flags & MGGX_AGG_RELU) v = fmaxf(v, 0.0f);
+    *o = v;
+}
+
+// Finishes this lane's NV elements of a complete row held in registers.
+template <int LPR, int MODE>
+__device__ __forceinline__ void finish_row(const AggArgs &a, int row, int l, const float (&acc)[ModeTraits<MODE>::NV])
+{
+    constexpr int NV = ModeTraits<MODE>::NV;
+    if constexpr (MODE == MODE_F32_VEC4) {
+        if (a.flags == 0 && a.rs_out == nullptr) {
+            if (NV * l < a.dim)
+                *reinterpret_cast<float4 *>(a.out + (long long)row * a.ld_out + 4 * l) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+            return;
+        }
+    }
+    if constexpr (MODE == MODE_BF16_VEC8) {
+        if (a.flags == 0 && a.rs_out == nullptr) {
+            if (NV * l < a.dim) {
+                float4 *o = reinterpret_cast<float4 *>(a.out + (long long)row * a.ld_out + 8 * l);
+                o[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+                o[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+            }
+            return;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int d = elem_of<LPR, MODE>(l, i);
+        if (d < a.dim) finish_elem(a, row, d, acc[i]);
+    }
+}
+
+// One wavefront-wide aggregation kernel; see the file header for the scheme.
+// Dynamic LDS: int2 hdr[2*wpb] (head, tail per wavefront), then float vals[2*wpb][cpad].
+template <int LPR, int MODE>
+__global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
+{
+    constexpr int NV = ModeTraits<MODE>::NV;
+    constexpr int S = 64 / LPR;
+    constexpr int CH = LPR > 16 ? LPR : 16;  // neighbor ids fetched per slot per chunk
+    constexpr int IPL = CH / LPR;            // ids fetched per lane
+    constexpr int BATCH = 8;                 // gathers issued back to back
+    extern __shared__ float lds[];
+
+    const int lane = lane_id();
+    const int wave = (int)(threadIdx.x >> 6);
+    const int wpb = (int)(blockDim.x >> 6);
+    const int slot = lane / LPR;
+    const int l = lane % LPR;
+    const int slot_base = slot * LPR;
+
+    int2 *hdr = reinterpret_cast<int2 *>(lds);
+    float *vals = lds + 4 * wpb;
+    if (lane == 0) {
+        hdr[2 * wave] = make_int2(-1, 0);
+        hdr[2 * wave + 1] = make_int2(-1, 0);
+    }
+
+    const long long q_wave = ((long long)blockIdx.x * wpb + wave) * ((long long)S * a.dist);
+
+    float acc[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) acc[i] = 0.0f;
+    int has_first = 0;    // the open run includes its row's first partition
+    bool c_open = false;  // wavefront-uniform: slot S-1 holds a row that continues in the next round
+
+    for (int j = 0; j < a.dist; ++j) {
+        const long long q0 = q_wave + (long long)j * S;
+        if (q0 >= a.num_parts) break;
+        const long long q = q0 + slot;
+        const bool pv = q < a.num_parts;
+        int4 d = make_int4(0, -1, 0, 0);
+        if (pv) d = a.desc[q];
+
+        // carried partial row of the previous round: slot S-1 -> slot 0
+        float cv[NV];
+        int c_first = 0;
+        if (c_open) {
+            const int src = (lane + 64 - LPR) & 63;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) cv[i] = lane_read(acc[i], src);
+            c_first = lane_read(has_first, src);
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) acc[i] = 0.0f;
+
+        const int row = d.y;
+        const int len = (int)((unsigned)d.z & DESC_LEN_MASK);
+        const bool remote = d.x < 0;
+        const long long start = (long long)((unsigned)d.x & 0x7FFFFFFFu);
+        const void *tbl = remote ? a.in_r : a.in_l;
+        const int *col = remote ? a.col_r : a.col_l;
+        const int idbase = remote ? 0 : a.lb;
+        const int nnz_side = remote ? a.nnz_r : a.nnz_l;
+
+        for (int k0 = 0; k0 < a.ps; k0 += CH) {
+            if (!__any(len > k0)) break;
+            // this lane's IPL neighbor ids of the chunk (-1 past the partition's end)
+            int ids[IPL];
+            {
+                const int kk = k0 + l * IPL;
+                const long long e0 = start + kk;
+#pragma unroll
+                for (int t = 0; t < IPL; ++t) ids[t] = -1;
+                if (kk < len) {
+                    if constexpr (IPL == 4) {
+                        if (e0 + 4 <= nnz_side) {
+                            int4 t4;
+                            __builtin_memcpy(&t4, col + e0, 16);
+                            ids[0] = t4.x; ids[1] = t4.y; ids[2] = t4.z; ids[3] = t4.w;
+                        } else {
+#pragma unroll
+                            for (int t = 0; t < IPL; ++t)
+                                if (kk + t < len) ids[t] = col[e0 + t];
+                        }
+                    } else {
+#pragma unroll
+                        for (int t = 0; t < IPL; ++t)
+                            if (kk + t < len) ids[t] = col[e0 + t];
+                    }
+#pragma unroll
+                    for (int t = 0; t < IPL; ++t)
+                        if (kk + t >= len) ids[t] = -1;
+                }
+            }
+            static_for<0, CH / BATCH>([&](auto bb) {
+                constexpr int b = decltype(bb)::value;
+                if (__any(len > k0 + b * BATCH)) {
+                    float v[BATCH][NV];
+                    bool ok[BATCH];
+                    static_for<0, BATCH>([&](auto tt) {
+                        constexpr int t = decltype(tt)::value;
+                        constexpr int k = b * BATCH + t;
+                        const int id = slot_bcast<LPR, k / IPL>(ids[k % IPL], slot_base);
+                        ok[t] = id >= 0;
+                        const long long r = ok[t] ? (long long)(id - idbase) : 0;
+                        gather_row<LPR, MODE>(v[t], tbl, r, a.ld_in, l, a.dim);
+                    });
+                    static_for<0, BATCH>([&](auto tt) {
+                        constexpr int t = decltype(tt)::value;
+#pragma unroll
+                        for (int i = 0; i < NV; ++i) acc[i] += ok[t] ? v[t][i] : 0.0f;
+                    });
+                }
+            });
+        }
+
+        // ---- combine the slots of this round ----
+        has_first = ((unsigned)d.z & DESC_FIRST) ? 1 : 0;
+        if (c_open && slot == 0) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) acc[i] += cv[i];
+            has_first |= c_first;
+        }
+        // segmented inclusive scan over slots, keyed by row (equal rows are adjacent)
+        static_for<0, 6>([&](auto oo) {
+            constexpr int o = 1 << decltype(oo)::value;
+            if constexpr (o < S) {
+                constexpr int SH = o * LPR;
+                const int src = lane >= SH ? lane - SH : lane;
+                const int prow = lane_read(row, src);
+                const bool take = lane >= SH && prow == row && row >= 0;
+                if (__any(take)) {
+                    const int pf = lane_read(has_first, src);
+                    has_first |= take ? pf : 0;
+#pragma unroll
+                    for (int i = 0; i < NV; ++i) {
+                        const float pvv = lane_read(acc[i], src);
+                        acc[i] += take ? pvv : 0.0f;
+                    }
+                }
+            }
+        });
+        // the last slot of each run now holds the run's sum
+        int nrow = -2;
+        if constexpr (S > 1) {
+            const int src = lane + LPR < 64 ? lane + LPR : lane;
+            nrow = lane_read(row, src);
+            if (slot == S - 1) nrow = -2;
+        }
+        const bool run_last = pv && nrow != row;
+        const bool row_done = ((unsigned)d.z & DESC_LAST) != 0;
+        const bool last_round = (j == a.dist - 1) || (q0 + S >= a.num_parts);
+        bool keep_open = false;
+        if (run_last) {
+            if (row_done && has_first) {
+                finish_row<LPR, MODE>(a, row, l, acc);
+            } else if (!row_done && !last_round) {
+                keep_open = true;  // slot S-1 only: continues in the next round
+            } else {
+                // partial row leaving this wavefront: head (started earlier) or tail (continues later)
+                const int e = has_first ? 2 * wave + 1 : 2 * wave;
+                const int f = HDR_VALID | (has_first ? HDR_STARTS : 0) | (row_done ? HDR_ENDS : 0);
+                if (l == 0) hdr[e] = make_int2(row, f);
+                float *dst = vals + (size_t)e * a.cpad;
+#pragma unroll
+                for (int i = 0; i < NV; ++i) {
+                    const int dd = elem_of<LPR, MODE>(l, i);
+                    if (dd < a.dim) dst[dd] = acc[i];
+                }
+            }
+        }
+        c_open = __any(keep_open);
+    }
+
+    __syncthreads();
+    if (wave != 0) return;
+
+    // ---- combine the wavefronts of this workgroup (wavefront 0; lane = feature index mod 64) ----
+    const int wg = (int)blockIdx.x;
+    if (lane == 0) {
+        a.c_hdr[2 * wg] = make_int2(-1, 0);
+        a.c_hdr[2 * wg + 1] = make_int2(-1, 0);
+    }
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    bool open = false, started = false;
+    int orow = -1;
+    auto emit = [&](bool ends) {
+        if (started && ends) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int dd = lane + 64 * i;
+                if (dd < a.dim) finish_elem(a, orow, dd, s[i]);
+            }
+        } else {
+            const int e = started ? 2 * wg + 1 : 2 * wg;
+            if (lane == 0) a.c_hdr[e] = make_int2(orow, HDR_VALID | (started ? HDR_STARTS : 0) | (ends ? HDR_ENDS : 0));
+            float *dst = a.c_val + (size_t)e * a.cpad;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int dd = lane + 64 * i;
+                if (dd < a.dim) dst[dd] = s[i];
+            }
+        }
+    };
+    for (int w = 0; w < wpb; ++w) {
+        const int2 h = hdr[2 * w];
+        if (h.y & HDR_VALID) {
+            if (!open) {
+                open = true;
+                started = false;
+                orow = h.x;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) s[i] = 0.f;
+            }
+            const float *src = vals + (size_t)(2 * w) * a.cpad;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int dd = lane + 64 * i;
+                if (dd < a.dim) s[i] += src[dd];
+            }
+            if (h.y & HDR_ENDS) {
+                emit(true);
+                open = false;
+            }
+        }
+        const int2 t = hdr[2 * w + 1];
+        if (t.y & HDR_VALID) {
+            open = true;
+            started = true;
+            orow = t.x;
+            const float *src = vals + (size_t)(2 * w + 1) * a.cpad;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int dd = lane + 64 * i;
+                s[i] = dd < a.dim ? src[dd] : 0.f;
+            }
+        }
+    }
+    if (open) emit(false);
+}
+
+// Rows that cross workgroups: the workgroup where the row starts left a tail
+// entry; every later workgroup up to the one where it ends left a head entry.
+// One block per workgroup slot; it acts only when that slot's tail is valid.
+__global__ void __launch_bounds__(256) k_agg_fixup(const AggArgs a, int num_wg, int comp_lanes)
+{
+    __shared__ float red[256];
+    const int b = (int)blockIdx.x;
+    const int2 t = a.c_hdr[2 * b + 1];
+    if (!(t.y & HDR_VALID)) return;
+    const int row = t.x;
+    const int last_wg = (a.off[row + 1] - 1) / a.parts_per_wg;
+    const int n = last_wg - b;  // head entries of workgroups b+1 .. last_wg
+    const int c = (int)threadIdx.x % comp_lanes;
+    const int walker = (int)threadIdx.x / comp_lanes;
+    const int walkers = 256 / comp_lanes;
+    float s = 0.f;
+    if (c < a.dim)
+        for (int k = walker; k < n; k += walkers) s += a.c_val[(size_t)(2 * (b + 1 + k)) * a.cpad + c];
+    red[threadIdx.x] = s;
+    __syncthreads();
+    if (walker == 0 && c < a.dim) {
+        float total = a.c_val[(size_t)(2 * b + 1) * a.cpad + c];
+        for (int w = 0; w < walkers; ++w) total += red[w * comp_lanes + c];
+        finish_elem(a, row, c, total);
+    }
+    (void)num_wg;
+}
+
+// Rows with no neighbor at all: the sum is zero.
+__global__ void __launch_bounds__(256) k_agg_empty_rows(const AggArgs a, const int *__restrict__ rows, int n_rows)
+{
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long long)n_rows * a.dim) return;
+    const int r = rows[idx / a.dim];
+    const int d = (int)(idx % a.dim);
+    finish_elem(a, r, d, 0.0f);
+}
+
+int pow2_ceil(int x)
+{
+    int p = 1;
+    while (p < x) p <<= 1;
+    return p;
+}
+
+template <int MODE>
+int launch_agg(int lpr, dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream, const AggArgs &a)
+{
+    switch (lpr) {
+#define MGGX_CASE(L)                                                      \
+    case L:                                                               \
+        k_agg<L, MODE><<<grid, block, lds_bytes, stream>>>(a);            \
+        break;
+        MGGX_CASE(1)
+        MGGX_CASE(2)
+        MGGX_CASE(4)
+        MGGX_CASE(8)
+        MGGX_CASE(16)
+        MGGX_CASE(32)
+        MGGX_CASE(64)
+#undef MGGX_CASE
+        default:
+            return fail(MGGX_EINVAL, "aggregation: no kernel for %d lanes per row", lpr);
+    }
+    return MGGX_OK;
+}
+
+int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, const int *d_col_l, const int *d_col_r,
+            int lb, int dim, int wpb, int dist, const mggx_agg_opts &o)
+{
+    State &st = state();
+    if (dim < 1 || dim > 256) return fail(MGGX_ELIMIT, "aggregation: dim %d outside 1..256", dim);
+    if (wpb < 1 || wpb > 16) return fail(MGGX_EINVAL, "aggregation: wpb %d outside 1..16", wpb);
+    if (dist < 1) return fail(MGGX_EINVAL, "aggregation: dist %d must be positive", dist);
+    const long long ld_in = o.ld_in ? o.ld_in : dim, ld_out = o.ld_out ? o.ld_out : dim;
+    if (ld_in < dim || ld_out < dim) return fail(MGGX_EINVAL, "aggregation: row stride smaller than dim");
+    if (plan->rows == 0) return MGGX_OK;
+    if (!d_out || !d_in_l) return fail(MGGX_EINVAL, "aggregation: NULL feature pointer");
+    if (plan->nnz_r > 0 && (!d_in_r || !d_col_r)) return fail(MGGX_EINVAL, "aggregation: remote edges but no remote table");
+    if (plan->nnz_l > 0 && !d_col_l) return fail(MGGX_EINVAL, "aggregation: local edges but no column array");
+
+    int mode, lpr;
+    const auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+    if (o.in_dtype == MGGX_BF16) {
+        if (dim % 8 || ld_in % 8 || ld_out % 4 || !aligned16(d_in_l) || (d_in_r && !aligned16(d_in_r)) || !aligned16(d_out))
+            return fail(MGGX_EINVAL, "aggregation: bf16 tables need dim %% 8 == 0, ld_in %% 8 == 0 and 16-byte alignment");
+        mode = MODE_BF16_VEC8;
+        lpr = pow2_ceil(dim / 8);
+    } else if (o.in_dtype == MGGX_F32) {
+        const bool vec = dim % 4 == 0 && ld_in % 4 == 0 && ld_out % 4 == 0 && aligned16(d_in_l) &&
+                         (!d_in_r || aligned16(d_in_r)) && aligned16(d_out);
+        mode = vec ? MODE_F32_VEC4 : MODE_F32_STRIDED;
+        lpr = pow2_ceil((dim + 3) / 4);
+    } else {
+        return fail(MGGX_EINVAL, "aggregation: unknown input dtype %d", o.in_dtype);
+    }
+    const int slots = 64 / lpr;
+    const long long parts_per_wg = (long long)wpb * slots * dist;
+    if (parts_per_wg > 0x3fffffffLL) return fail(MGGX_ELIMIT, "aggregation: wpb*dist too large");
+    const long long num_wg = (plan->num_parts + parts_per_wg - 1) / parts_per_wg;
+    if (num_wg > 0x7fffffffLL) return fail(MGGX_ELIMIT, "aggregation: too many workgroups");
+    const int cpad = (dim + 3) & ~3;
+
+    AggArgs a{};
+    a.out = d_out;
+    a.in_l = d_in_l;
+    a.in_r = d_in_r ? d_in_r : d_in_l;
+    a.col_l = d_col_l;
+    a.col_r = d_col_r;
+    a.desc = plan->d_desc;
+    a.off = plan->d_off;
+    a.rs_out = o.d_row_scale_out;
+    a.ld_in = ld_in;
+    a.ld_out = ld_out;
+    a.num_parts = plan->num_parts;
+    a.nnz_l = (int)plan->nnz_l;
+    a.nnz_r = (int)plan->nnz_r;
+    a.lb = lb;
+    a.dim = dim;
+    a.ps = plan->ps;
+    a.dist = dist;
+    a.cpad = cpad;
+    a.parts_per_wg = (int)parts_per_wg;
+    a.flags = o.flags;
+    a.eps = o.eps;
+    a.in_is_bf16 = o.in_dtype == MGGX_BF16;
+
+    if (num_wg > 0) {
+        const size_t hdr_bytes = (size_t)num_wg * 2 * sizeof(int2);
+        const size_t hdr_pad = (hdr_bytes + 255) & ~(size_t)255;
+        void *ws = nullptr;
+        int rc = workspace(hdr_pad + (size_t)num_wg * 2 * cpad * sizeof(float), &ws);
+        if (rc) return rc;
+        a.c_hdr = static_cast<int2 *>(ws);
+        a.c_val = reinterpret_cast<float *>(static_cast<char *>(ws) + hdr_pad);
+        const size_t lds_bytes = (size_t)wpb * 2 * sizeof(int2) + (size_t)wpb * 2 * cpad * sizeof(float);
+        const dim3 grid((unsigned)num_wg), block((unsigned)(64 * wpb));
+        if (mode == MODE_F32_VEC4) rc = launch_agg<MODE_F32_VEC4>(lpr, grid, block, lds_bytes, st.stream, a);
+        else if (mode == MODE_F32_STRIDED) rc = launch_agg<MODE_F32_STRIDED>(lpr, grid, block, lds_bytes, st.stream, a);
+        else rc = launch_agg<MODE_BF16_VEC8>(lpr, grid, block, lds_bytes, st.stream, a);
+        if (rc) return rc;
+        MGGX_LAUNCH_CHECK("k_agg");
+        if (num_wg > 1) {
+            const int comp_lanes = pow2_ceil(dim);
+            k_agg_fixup<<<dim3((unsigned)(num_wg - 1)), dim3(256), 0, st.stream>>>(a, (int)num_wg, comp_lanes);
+            MGGX_LAUNCH_CHECK("k_agg_fixup");
+        }
+    }
+    const bool touch_empty = !(o.flags & MGGX_AGG_ACCUMULATE) || (o.flags & (MGGX_AGG_GIN | MGGX_AGG_RELU));
+    if (plan->num_empty > 0 && touch_empty) {
+        const long long n = (long long)plan->num_empty * dim;
+        k_agg_empty_rows<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(a, plan->d_empty_rows, plan->num_empty);
+        MGGX_LAUNCH_CHECK("k_agg_empty_rows");
+    }
+    snprintf(st.last_kernel, sizeof(st.last_kernel), "k_agg<%d,%d> grid=%lld block=%d parts=%d", lpr, mode, num_wg, 64 * wpb,
+             plan->num_parts);
+    return MGGX_OK;
+}
+
+}  // namespace
+}  // namespace mggx
+
+using mggx::fail;
+
+MGGX_EXPORT int mggx_sag_np_div(float *d_out, const void *d_in_local, const void *d_in_remote, const int *d_ptr_l,
+                                const int *d_col_l, const int *d_ptr_r, const int *d_col_r, int lb, int ub, int dim,
+                                int nodes_per_pe, int ps, int wpb, int dist, const mggx_agg_opts *opts)
+{
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    if (ub < lb || !d_ptr_l) return fail(MGGX_EINVAL, "sag_np_div: bad row range [%d,%d) or NULL row pointers", lb, ub);
+    if (ps < 1) return fail(MGGX_EINVAL, "sag_np_div: ps %d must be positive", ps);
+    if (nodes_per_pe < ub - lb) return fail(MGGX_EINVAL, "sag_np_div: nodes_per_pe %d smaller than the row range", nodes_per_pe);
+    mggx_agg_opts o{};
+    if (opts) o = *opts;
+    mggx::Plan *plan = nullptr;
+    rc = mggx::plan_get(d_ptr_l, d_ptr_r, ub - lb, ps, &plan);
+    if (rc) return rc;
+    return mggx::run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, wpb, dist, o);
+}
+
+MGGX_EXPORT int mggx_sag_parts(float *d_out, const float *d_in, const int *d_row_ptr, const int *d_col,
+                               const int *d_part_ptr, const int *d_part2node, int lowbound, int num_nodes,
+                               int num_parts, int ps, int dim, int wpb, int dist)
+{
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    if (!d_row_ptr || !d_part_ptr || !d_part2node || num_nodes < 0 || num_parts < 0 || ps < 1)
+        return fail(MGGX_EINVAL, "sag_parts: bad argument");
+    mggx::Plan *plan = nullptr;
+    rc = mggx::plan_get_explicit(d_row_ptr, d_part_ptr, d_part2node, num_nodes, num_parts, ps, &plan);
+    if (rc) return rc;
+    mggx_agg_opts o{};
+    o.flags = MGGX_AGG_ACCUMULATE;
+    return mggx::run_agg(plan, d_out, d_in, nullptr, d_col, nullptr, lowbound, dim, wpb, dist, o);
+}
+
+MGGX_EXPORT int mggx_spmm(float *d_out, const float *d_in, const int *d_row_ptr, const int *d_col, int num_nodes,
+                          int dim, int ps, int wpb)
+{
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    if (!d_row_ptr || num_nodes < 0 || ps < 1) return fail(MGGX_EINVAL, "spmm: bad argument");
+    mggx::Plan *plan = nullptr;
+    rc = mggx::plan_get(d_row_ptr, nullptr, num_nodes, ps, &plan);
+    if (rc) return rc;
+    mggx_agg_opts o{};
+    o.flags = MGGX_AGG_ACCUMULATE;
+    return mggx::run_agg(plan, d_out, d_in, nullptr, d_col, nullptr, 0, dim, wpb, 1, o);
+}

@@ -1,0 +1,81 @@
+// Device-side internals of libmggx.so (HIP translation units only).
+#ifndef MGGX_DEV_H
+#define MGGX_DEV_H
+
+#include <hip/hip_runtime.h>
+
+#include <vector>
+
+#include "mggx_internal.h"
+
+#define MGGX_HIP(call)                                                                               \
+    do {                                                                                             \
+        hipError_t e_ = (call);                                                                      \
+        if (e_ != hipSuccess)                                                                        \
+            return mggx::fail(MGGX_EHIP, "%s failed: %s (%s:%d)", #call, hipGetErrorString(e_),      \
+                              __FILE__, __LINE__);                                                   \
+    } while (0)
+
+#define MGGX_LAUNCH_CHECK(name)                                                                      \
+    do {                                                                                             \
+        hipError_t e_ = hipGetLastError();                                                           \
+        if (e_ != hipSuccess)                                                                        \
+            return mggx::fail(MGGX_EHIP, "launch of %s failed: %s", name, hipGetErrorString(e_));    \
+    } while (0)
+
+namespace mggx {
+
+// Partition descriptor consumed by the aggregation kernels, one per neighbor
+// partition, in row-major order with a row's local partitions before its
+// remote ones.
+//   x: first edge index inside col_l / col_r; bit 31 set = remote side
+//   y: destination row (0-based inside the share)
+//   z: number of neighbors (1..ps) | FIRST<<30 | LAST<<31
+//   w: unused (0)
+static constexpr unsigned DESC_REMOTE = 0x80000000u;
+static constexpr unsigned DESC_FIRST = 0x40000000u;  // first partition of its row
+static constexpr unsigned DESC_LAST = 0x80000000u;   // last partition of its row
+static constexpr unsigned DESC_LEN_MASK = 0x3FFFFFFFu;
+
+struct Plan {
+    // cache key
+    const int *d_ptr_l = nullptr;
+    const int *d_ptr_r = nullptr;
+    const int *d_part_ptr = nullptr;   // explicit-partition plans only
+    const int *d_part2node = nullptr;  // explicit-partition plans only
+    int rows = 0;
+    int ps = 0;
+    // contents (device)
+    int4 *d_desc = nullptr;      // [num_parts]
+    int *d_off = nullptr;        // [rows+1] first descriptor of each row
+    int *d_empty_rows = nullptr; // rows without any partition
+    int num_parts = 0;
+    int num_empty = 0;
+    int64_t nnz_l = 0, nnz_r = 0;
+};
+
+struct State {
+    int device = -1;
+    hipStream_t stream = nullptr;
+    void *ws = nullptr;
+    size_t ws_bytes = 0;
+    std::vector<Plan *> plans;
+    char last_kernel[160] = "";
+};
+
+State &state();
+int ensure_init();
+// Grow-only scratch owned by the library; valid until the next call that grows it.
+int workspace(size_t bytes, void **p);
+
+// d_out[0..n] = exclusive prefix sum of d_in[0..n) (d_out has n+1 entries); the
+// total is also copied to *total_host when non-NULL (synchronises).
+int exclusive_scan_i32(const int *d_in, int *d_out, int n, long long *total_host);
+
+int plan_get(const int *d_ptr_l, const int *d_ptr_r, int rows, int ps, Plan **out);
+int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows,
+                      int num_parts, int ps, Plan **out);
+void plan_free(Plan *p);
+
+}  // namespace mggx
+#endif

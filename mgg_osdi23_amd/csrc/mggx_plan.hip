@@ -1,0 +1,428 @@
+// Neighbor partitioning on the GPU: prefix sums, the build_part arrays in the
+// reference's layout, and the merged partition-descriptor list the aggregation
+// kernels consume.
+#include <algorithm>
+
+#include "mggx_dev.h"
+
+namespace mggx {
+namespace {
+
+constexpr int SCAN_THREADS = 256;
+constexpr int SCAN_ITEMS = 4;
+constexpr int SCAN_TILE = SCAN_THREADS * SCAN_ITEMS;
+
+// Block-wide exclusive scan of one int per thread (256 threads); returns the
+// exclusive prefix and leaves the block total in *total.
+__device__ __forceinline__ int block_exclusive_scan(int v, int *lds /* 256 ints */, int *total)
+{
+    const int t = threadIdx.x;
+    lds[t] = v;
+    __syncthreads();
+    for (int o = 1; o < SCAN_THREADS; o <<= 1) {
+        int add = t >= o ? lds[t - o] : 0;
+        __syncthreads();
+        lds[t] += add;
+        __syncthreads();
+    }
+    const int incl = lds[t];
+    *total = lds[SCAN_THREADS - 1];
+    __syncthreads();
+    return incl - v;
+}
+
+__global__ void __launch_bounds__(SCAN_THREADS) k_scan_tile_sums(const int *__restrict__ in, int n, long long *__restrict__ tile_sum)
+{
+    __shared__ long long red[SCAN_THREADS];
+    const long long base = (long long)blockIdx.x * SCAN_TILE;
+    long long s = 0;
+    for (int i = 0; i < SCAN_ITEMS; ++i) {
+        long long idx = base + (long long)threadIdx.x * SCAN_ITEMS + i;
+        if (idx < n) s += in[idx];
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int o = SCAN_THREADS / 2; o > 0; o >>= 1) {
+        if (threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) tile_sum[blockIdx.x] = red[0];
+}
+
+// One block turns tile sums into exclusive tile offsets; tile_sum[num_tiles] receives the total.
+__global__ void __launch_bounds__(SCAN_THREADS) k_scan_tile_offsets(long long *__restrict__ tile_sum, int num_tiles)
+{
+    __shared__ long long buf[SCAN_THREADS];
+    __shared__ long long carry;
+    if (threadIdx.x == 0) carry = 0;
+    __syncthreads();
+    for (int base = 0; base < num_tiles; base += SCAN_THREADS) {
+        const int idx = base + threadIdx.x;
+        const long long v = idx < num_tiles ? tile_sum[idx] : 0;
+        buf[threadIdx.x] = v;
+        __syncthreads();
+        for (int o = 1; o < SCAN_THREADS; o <<= 1) {
+            long long add = threadIdx.x >= o ? buf[threadIdx.x - o] : 0;
+            __syncthreads();
+            buf[threadIdx.x] += add;
+            __syncthreads();
+        }
+        const long long incl = buf[threadIdx.x];
+        const long long c = carry;
+        if (idx < num_tiles) tile_sum[idx] = c + incl - v;
+        __syncthreads();
+        if (threadIdx.x == SCAN_THREADS - 1) carry = c + incl;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) tile_sum[num_tiles] = carry;
+}
+
+__global__ void __launch_bounds__(SCAN_THREADS) k_scan_apply(const int *__restrict__ in, int *__restrict__ out, int n,
+                                                             const long long *__restrict__ tile_off)
+{
+    __shared__ int lds[SCAN_THREADS];
+    const long long base = (long long)blockIdx.x * SCAN_TILE;
+    int v[SCAN_ITEMS];
+    int local = 0;
+    for (int i = 0; i < SCAN_ITEMS; ++i) {
+        long long idx = base + (long long)threadIdx.x * SCAN_ITEMS + i;
+        v[i] = idx < n ? in[idx] : 0;
+        local += v[i];
+    }
+    int total;
+    int excl = block_exclusive_scan(local, lds, &total);
+    long long run = tile_off[blockIdx.x] + excl;
+    for (int i = 0; i < SCAN_ITEMS; ++i) {
+        long long idx = base + (long long)threadIdx.x * SCAN_ITEMS + i;
+        if (idx < n) out[idx] = (int)run;
+        run += v[i];
+    }
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == SCAN_THREADS - 1) out[n] = (int)run;
+}
+
+// parts of one CSR side per row: ceil(deg/ps); both sides summed when ptr_r != NULL
+__global__ void __launch_bounds__(256) k_count_parts(const int *__restrict__ ptr_l, const int *__restrict__ ptr_r, int rows,
+                                                     int ps, int *__restrict__ cnt)
+{
+    const int r = blockIdx.x * 256 + threadIdx.x;
+    if (r >= rows) return;
+    long long c = ((long long)ptr_l[r + 1] - ptr_l[r] + ps - 1) / ps;
+    if (ptr_r) c += ((long long)ptr_r[r + 1] - ptr_r[r] + ps - 1) / ps;
+    cnt[r] = (int)c;
+}
+
+// largest r in [0, rows) with off[r] <= q (off is non-decreasing, off[rows] > q)
+__device__ __forceinline__ int row_of_part(const int *__restrict__ off, int rows, int q)
+{
+    int lo = 0, hi = rows;  // invariant: off[lo] <= q < off[hi]
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (off[mid] <= q) lo = mid;
+        else hi = mid;
+    }
+    return lo;
+}
+
+__global__ void __launch_bounds__(256) k_fill_desc(const int *__restrict__ off, const int *__restrict__ ptr_l,
+                                                   const int *__restrict__ ptr_r, int rows, int ps, int num_parts,
+                                                   int4 *__restrict__ desc)
+{
+    const int q = blockIdx.x * 256 + threadIdx.x;
+    if (q >= num_parts) return;
+    const int r = row_of_part(off, rows, q);
+    const int j = q - off[r];
+    const int total = off[r + 1] - off[r];
+    const int nl = (int)(((long long)ptr_l[r + 1] - ptr_l[r] + ps - 1) / ps);
+    unsigned start, len;
+    if (j < nl) {
+        const long long beg = (long long)ptr_l[r] + (long long)j * ps;
+        start = (unsigned)beg;
+        len = (unsigned)min((long long)ps, (long long)ptr_l[r + 1] - beg);
+    } else {
+        const long long beg = (long long)ptr_r[r] + (long long)(j - nl) * ps;
+        start = (unsigned)beg | DESC_REMOTE;
+        len = (unsigned)min((long long)ps, (long long)ptr_r[r + 1] - beg);
+    }
+    unsigned z = len;
+    if (j == 0) z |= DESC_FIRST;
+    if (j == total - 1) z |= DESC_LAST;
+    desc[q] = make_int4((int)start, r, (int)z, 0);
+}
+
+// explicit partition arrays (reference layout) -> descriptors; lengths from row_ptr
+__global__ void __launch_bounds__(256) k_desc_from_parts(const int *__restrict__ row_ptr, const int *__restrict__ part_ptr,
+                                                         const int *__restrict__ part2node, int num_parts, int ps,
+                                                         int4 *__restrict__ desc)
+{
+    const int q = blockIdx.x * 256 + threadIdx.x;
+    if (q >= num_parts) return;
+    const int r = part2node[q];
+    const int beg = part_ptr[q];
+    unsigned z = (unsigned)max(0, min(ps, row_ptr[r + 1] - beg));
+    if (q == 0 || part2node[q - 1] != r) z |= DESC_FIRST;
+    if (q == num_parts - 1 || part2node[q + 1] != r) z |= DESC_LAST;
+    desc[q] = make_int4(beg, r, (int)z, 0);
+}
+
+// off[r] for explicit plans: first descriptor of row r = lower bound of r in part2node
+__global__ void __launch_bounds__(256) k_off_from_parts(const int *__restrict__ part2node, int num_parts, int rows,
+                                                        int *__restrict__ off)
+{
+    const int r = blockIdx.x * 256 + threadIdx.x;
+    if (r > rows) return;
+    int lo = 0, hi = num_parts;  // first index with part2node[idx] >= r
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (part2node[mid] < r) lo = mid + 1;
+        else hi = mid;
+    }
+    off[r] = lo;
+}
+
+__global__ void __launch_bounds__(256) k_collect_empty(const int *__restrict__ off, int rows, int *__restrict__ list,
+                                                       int *__restrict__ counter)
+{
+    const int r = blockIdx.x * 256 + threadIdx.x;
+    if (r >= rows) return;
+    if (off[r + 1] == off[r]) list[atomicAdd(counter, 1)] = r;
+}
+
+// reference-layout arrays
+__global__ void __launch_bounds__(256) k_parts_ref_layout(const int *__restrict__ indptr, const int *__restrict__ node2part,
+                                                          int num_nodes, int ps, int num_parts, int compat,
+                                                          int *__restrict__ part_ptr, int *__restrict__ part2node)
+{
+    const int p = blockIdx.x * 256 + threadIdx.x;
+    if (p > num_parts) return;
+    if (p == num_parts) {
+        const bool last_has = num_nodes > 0 && indptr[num_nodes] > indptr[num_nodes - 1];
+        part_ptr[p] = (compat && !last_has) ? 0 : (num_nodes > 0 ? indptr[num_nodes] : 0);
+        return;
+    }
+    const int i = row_of_part(node2part, num_nodes, p);
+    part_ptr[p] = indptr[i] + (p - node2part[i]) * ps;
+    part2node[p] = i;
+}
+
+__global__ void k_set_tail(int *node2part, int num_nodes)
+{
+    node2part[num_nodes + 1] = node2part[num_nodes];
+}
+
+}  // namespace
+
+int exclusive_scan_i32(const int *d_in, int *d_out, int n, long long *total_host)
+{
+    State &s = state();
+    if (n <= 0) {
+        MGGX_HIP(hipMemsetAsync(d_out, 0, sizeof(int), s.stream));
+        if (total_host) *total_host = 0;
+        return MGGX_OK;
+    }
+    const int tiles = (n + SCAN_TILE - 1) / SCAN_TILE;
+    long long *d_tile = nullptr;
+    MGGX_HIP(hipMalloc((void **)&d_tile, sizeof(long long) * ((size_t)tiles + 1)));
+    k_scan_tile_sums<<<tiles, SCAN_THREADS, 0, s.stream>>>(d_in, n, d_tile);
+    k_scan_tile_offsets<<<1, SCAN_THREADS, 0, s.stream>>>(d_tile, tiles);
+    k_scan_apply<<<tiles, SCAN_THREADS, 0, s.stream>>>(d_in, d_out, n, d_tile);
+    hipError_t e = hipGetLastError();
+    long long total = 0;
+    if (e == hipSuccess) e = hipMemcpyAsync(&total, d_tile + tiles, sizeof(long long), hipMemcpyDeviceToHost, s.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(s.stream);
+    (void)hipFree(d_tile);
+    if (e != hipSuccess) return fail(MGGX_EHIP, "exclusive_scan: %s", hipGetErrorString(e));
+    if (total > 0x7fffffffLL) return fail(MGGX_ELIMIT, "exclusive_scan: total %lld exceeds int32", total);
+    if (total_host) *total_host = total;
+    return MGGX_OK;
+}
+
+void plan_free(Plan *p)
+{
+    if (!p) return;
+    if (p->d_desc) (void)hipFree(p->d_desc);
+    if (p->d_off) (void)hipFree(p->d_off);
+    if (p->d_empty_rows) (void)hipFree(p->d_empty_rows);
+    delete p;
+}
+
+static int plan_finish(Plan *p)
+{
+    State &s = state();
+    // rows without partitions
+    int *d_counter = nullptr;
+    MGGX_HIP(hipMalloc((void **)&d_counter, sizeof(int)));
+    MGGX_HIP(hipMemsetAsync(d_counter, 0, sizeof(int), s.stream));
+    MGGX_HIP(hipMalloc((void **)&p->d_empty_rows, sizeof(int) * (size_t)std::max(p->rows, 1)));
+    if (p->rows > 0) {
+        k_collect_empty<<<(p->rows + 255) / 256, 256, 0, s.stream>>>(p->d_off, p->rows, p->d_empty_rows, d_counter);
+        MGGX_LAUNCH_CHECK("k_collect_empty");
+    }
+    MGGX_HIP(hipMemcpyAsync(&p->num_empty, d_counter, sizeof(int), hipMemcpyDeviceToHost, s.stream));
+    MGGX_HIP(hipStreamSynchronize(s.stream));
+    MGGX_HIP(hipFree(d_counter));
+    return MGGX_OK;
+}
+
+static void cache_insert(Plan *p)
+{
+    State &s = state();
+    const size_t max_plans = 16;
+    if (s.plans.size() >= max_plans) {
+        (void)hipStreamSynchronize(s.stream);
+        plan_free(s.plans.front());
+        s.plans.erase(s.plans.begin());
+    }
+    s.plans.push_back(p);
+}
+
+int plan_get(const int *d_ptr_l, const int *d_ptr_r, int rows, int ps, Plan **out)
+{
+    State &s = state();
+    for (Plan *p : s.plans)
+        if (p->d_ptr_l == d_ptr_l && p->d_ptr_r == d_ptr_r && p->rows == rows && p->ps == ps && !p->d_part_ptr) {
+            *out = p;
+            return MGGX_OK;
+        }
+    Plan *p = new Plan;
+    p->d_ptr_l = d_ptr_l;
+    p->d_ptr_r = d_ptr_r;
+    p->rows = rows;
+    p->ps = ps;
+    int rc = MGGX_OK;
+    int *d_cnt = nullptr;
+    do {
+        if (hipMalloc((void **)&d_cnt, sizeof(int) * (size_t)std::max(rows, 1)) != hipSuccess ||
+            hipMalloc((void **)&p->d_off, sizeof(int) * ((size_t)rows + 1)) != hipSuccess) {
+            rc = fail(MGGX_ENOMEM, "plan: row arrays for %d rows", rows);
+            break;
+        }
+        if (rows > 0) k_count_parts<<<(rows + 255) / 256, 256, 0, s.stream>>>(d_ptr_l, d_ptr_r, rows, ps, d_cnt);
+        long long total = 0;
+        rc = exclusive_scan_i32(d_cnt, p->d_off, rows, &total);
+        if (rc) break;
+        p->num_parts = (int)total;
+        int ends[2] = {0, 0};
+        if (rows > 0) {
+            if (hipMemcpy(&ends[0], d_ptr_l + rows, sizeof(int), hipMemcpyDeviceToHost) != hipSuccess ||
+                (d_ptr_r && hipMemcpy(&ends[1], d_ptr_r + rows, sizeof(int), hipMemcpyDeviceToHost) != hipSuccess)) {
+                rc = fail(MGGX_EHIP, "plan: reading edge counts");
+                break;
+            }
+        }
+        p->nnz_l = ends[0];
+        p->nnz_r = ends[1];
+        if (hipMalloc((void **)&p->d_desc, sizeof(int4) * (size_t)std::max(p->num_parts, 1)) != hipSuccess) {
+            rc = fail(MGGX_ENOMEM, "plan: %d descriptors", p->num_parts);
+            break;
+        }
+        if (p->num_parts > 0) {
+            k_fill_desc<<<(p->num_parts + 255) / 256, 256, 0, s.stream>>>(p->d_off, d_ptr_l, d_ptr_r, rows, ps,
+                                                                          p->num_parts, p->d_desc);
+            if (hipGetLastError() != hipSuccess) {
+                rc = fail(MGGX_EHIP, "plan: descriptor kernel launch failed");
+                break;
+            }
+        }
+        rc = plan_finish(p);
+    } while (0);
+    if (d_cnt) (void)hipFree(d_cnt);
+    if (rc) {
+        plan_free(p);
+        return rc;
+    }
+    cache_insert(p);
+    *out = p;
+    return MGGX_OK;
+}
+
+int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows, int num_parts,
+                      int ps, Plan **out)
+{
+    State &s = state();
+    for (Plan *p : s.plans)
+        if (p->d_ptr_l == d_row_ptr && p->d_part_ptr == d_part_ptr && p->d_part2node == d_part2node && p->rows == rows &&
+            p->ps == ps && p->num_parts == num_parts) {
+            *out = p;
+            return MGGX_OK;
+        }
+    Plan *p = new Plan;
+    p->d_ptr_l = d_row_ptr;
+    p->d_part_ptr = d_part_ptr;
+    p->d_part2node = d_part2node;
+    p->rows = rows;
+    p->ps = ps;
+    p->num_parts = num_parts;
+    int rc = MGGX_OK;
+    do {
+        if (hipMalloc((void **)&p->d_off, sizeof(int) * ((size_t)rows + 1)) != hipSuccess ||
+            hipMalloc((void **)&p->d_desc, sizeof(int4) * (size_t)std::max(num_parts, 1)) != hipSuccess) {
+            rc = fail(MGGX_ENOMEM, "plan: explicit arrays");
+            break;
+        }
+        k_off_from_parts<<<(rows + 1 + 255) / 256, 256, 0, s.stream>>>(d_part2node, num_parts, rows, p->d_off);
+        if (num_parts > 0)
+            k_desc_from_parts<<<(num_parts + 255) / 256, 256, 0, s.stream>>>(d_row_ptr, d_part_ptr, d_part2node, num_parts,
+                                                                            ps, p->d_desc);
+        if (hipGetLastError() != hipSuccess) {
+            rc = fail(MGGX_EHIP, "plan: explicit descriptor kernel launch failed");
+            break;
+        }
+        int end = 0;
+        if (rows > 0 && hipMemcpy(&end, d_row_ptr + rows, sizeof(int), hipMemcpyDeviceToHost) != hipSuccess) {
+            rc = fail(MGGX_EHIP, "plan: reading edge count");
+            break;
+        }
+        p->nnz_l = end;
+        rc = plan_finish(p);
+    } while (0);
+    if (rc) {
+        plan_free(p);
+        return rc;
+    }
+    cache_insert(p);
+    *out = p;
+    return MGGX_OK;
+}
+
+}  // namespace mggx
+
+using mggx::fail;
+
+MGGX_EXPORT int mggx_build_part_device(const int *d_indptr, int num_nodes, int part_size, int compat, int *d_part_ptr,
+                                       int *d_part2node, int *d_node2part, int *num_parts)
+{
+    if (!d_indptr || num_nodes < 0 || part_size <= 0 || !num_parts)
+        return fail(MGGX_EINVAL, "build_part_device: indptr NULL, num_nodes=%d, part_size=%d", num_nodes, part_size);
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    mggx::State &s = mggx::state();
+    int *d_cnt = nullptr, *d_n2p = d_node2part;
+    bool own_n2p = false;
+    MGGX_HIP(hipMalloc((void **)&d_cnt, sizeof(int) * (size_t)std::max(num_nodes, 1)));
+    if (!d_n2p) {
+        if (hipMalloc((void **)&d_n2p, sizeof(int) * ((size_t)num_nodes + 2)) != hipSuccess) {
+            (void)hipFree(d_cnt);
+            return fail(MGGX_ENOMEM, "build_part_device: node2part");
+        }
+        own_n2p = true;
+    }
+    long long total = 0;
+    do {
+        if (num_nodes > 0)
+            mggx::k_count_parts<<<(num_nodes + 255) / 256, 256, 0, s.stream>>>(d_indptr, nullptr, num_nodes, part_size, d_cnt);
+        rc = mggx::exclusive_scan_i32(d_cnt, d_n2p, num_nodes, &total);
+        if (rc) break;
+        mggx::k_set_tail<<<1, 1, 0, s.stream>>>(d_n2p, num_nodes);
+        *num_parts = (int)total;
+        if (d_part_ptr && d_part2node) {
+            const int n = (int)total + 1;
+            mggx::k_parts_ref_layout<<<(n + 255) / 256, 256, 0, s.stream>>>(d_indptr, d_n2p, num_nodes, part_size, (int)total,
+                                                                            compat, d_part_ptr, d_part2node);
+        }
+        if (hipGetLastError() != hipSuccess || hipStreamSynchronize(s.stream) != hipSuccess)
+            rc = fail(MGGX_EHIP, "build_part_device: kernel failed");
+    } while (0);
+    (void)hipFree(d_cnt);
+    if (own_n2p) (void)hipFree(d_n2p);
+    return rc;
+}

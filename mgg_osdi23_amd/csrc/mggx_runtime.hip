@@ -1,0 +1,269 @@
+// Runtime half of libmggx.so: device selection, stream, memory, timers, the
+// library-owned workspace and small utility kernels.
+#include <cstdio>
+#include <cstring>
+
+#include "mggx_dev.h"
+
+namespace mggx {
+
+State &state()
+{
+    static State s;
+    return s;
+}
+
+int ensure_init()
+{
+    State &s = state();
+    if (s.device >= 0) return MGGX_OK;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0)
+        return fail(MGGX_EHIP, "no HIP device available (%s)", e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+    int cur = 0;
+    MGGX_HIP(hipGetDevice(&cur));
+    s.device = cur;
+    return MGGX_OK;
+}
+
+int workspace(size_t bytes, void **p)
+{
+    State &s = state();
+    if (bytes > s.ws_bytes) {
+        if (s.ws) {
+            MGGX_HIP(hipStreamSynchronize(s.stream));
+            MGGX_HIP(hipFree(s.ws));
+            s.ws = nullptr;
+            s.ws_bytes = 0;
+        }
+        size_t want = bytes + bytes / 4 + 4096;
+        hipError_t e = hipMalloc(&s.ws, want);
+        if (e != hipSuccess) {
+            s.ws = nullptr;
+            return fail(MGGX_ENOMEM, "workspace of %zu bytes: %s", want, hipGetErrorString(e));
+        }
+        s.ws_bytes = want;
+    }
+    *p = s.ws;
+    return MGGX_OK;
+}
+
+}  // namespace mggx
+
+using mggx::fail;
+using mggx::state;
+
+MGGX_EXPORT int mggx_init(int device)
+{
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0)
+        return fail(MGGX_EHIP, "no HIP device available (%s)", e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+    if (device < 0 || device >= count) return fail(MGGX_EINVAL, "init: device %d of %d", device, count);
+    MGGX_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    MGGX_HIP(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(MGGX_EHIP, "init: device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+    state().device = device;
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_device_name(char *buf, size_t len)
+{
+    if (!buf || !len) return fail(MGGX_EINVAL, "device_name: NULL buffer");
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    hipDeviceProp_t prop;
+    MGGX_HIP(hipGetDeviceProperties(&prop, state().device));
+    snprintf(buf, len, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_set_stream(void *hip_stream)
+{
+    state().stream = static_cast<hipStream_t>(hip_stream);
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_sync(void)
+{
+    MGGX_HIP(hipStreamSynchronize(state().stream));
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_malloc(void **d_ptr, size_t bytes)
+{
+    if (!d_ptr) return fail(MGGX_EINVAL, "malloc: NULL result pointer");
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    *d_ptr = nullptr;
+    hipError_t e = hipMalloc(d_ptr, bytes ? bytes : 1);
+    if (e != hipSuccess) return fail(MGGX_ENOMEM, "malloc of %zu bytes: %s", bytes, hipGetErrorString(e));
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_free(void *d_ptr)
+{
+    if (!d_ptr) return MGGX_OK;
+    MGGX_HIP(hipFree(d_ptr));
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_memset(void *d_ptr, int value, size_t bytes)
+{
+    if (!bytes) return MGGX_OK;
+    if (!d_ptr) return fail(MGGX_EINVAL, "memset: NULL pointer");
+    MGGX_HIP(hipMemsetAsync(d_ptr, value, bytes, state().stream));
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_memcpy_h2d(void *d_dst, const void *src, size_t bytes)
+{
+    if (!bytes) return MGGX_OK;
+    if (!d_dst || !src) return fail(MGGX_EINVAL, "memcpy_h2d: NULL pointer");
+    MGGX_HIP(hipMemcpyAsync(d_dst, src, bytes, hipMemcpyHostToDevice, state().stream));
+    MGGX_HIP(hipStreamSynchronize(state().stream));
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_memcpy_d2h(void *dst, const void *d_src, size_t bytes)
+{
+    if (!bytes) return MGGX_OK;
+    if (!dst || !d_src) return fail(MGGX_EINVAL, "memcpy_d2h: NULL pointer");
+    MGGX_HIP(hipMemcpyAsync(dst, d_src, bytes, hipMemcpyDeviceToHost, state().stream));
+    MGGX_HIP(hipStreamSynchronize(state().stream));
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes)
+{
+    if (!bytes) return MGGX_OK;
+    if (!d_dst || !d_src) return fail(MGGX_EINVAL, "memcpy_d2d: NULL pointer");
+    MGGX_HIP(hipMemcpyAsync(d_dst, d_src, bytes, hipMemcpyDeviceToDevice, state().stream));
+    return MGGX_OK;
+}
+
+namespace {
+struct Timer {
+    hipEvent_t start, stop;
+};
+}  // namespace
+
+MGGX_EXPORT int mggx_timer_create(void **timer)
+{
+    if (!timer) return fail(MGGX_EINVAL, "timer_create: NULL");
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    Timer *t = new Timer;
+    if (hipEventCreate(&t->start) != hipSuccess || hipEventCreate(&t->stop) != hipSuccess) {
+        delete t;
+        return fail(MGGX_EHIP, "timer_create: hipEventCreate failed");
+    }
+    *timer = t;
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_timer_start(void *timer)
+{
+    if (!timer) return fail(MGGX_EINVAL, "timer_start: NULL");
+    MGGX_HIP(hipEventRecord(static_cast<Timer *>(timer)->start, state().stream));
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_timer_stop(void *timer)
+{
+    if (!timer) return fail(MGGX_EINVAL, "timer_stop: NULL");
+    MGGX_HIP(hipEventRecord(static_cast<Timer *>(timer)->stop, state().stream));
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_timer_elapsed_ms(void *timer, float *ms)
+{
+    if (!timer || !ms) return fail(MGGX_EINVAL, "timer_elapsed_ms: NULL");
+    Timer *t = static_cast<Timer *>(timer);
+    MGGX_HIP(hipEventSynchronize(t->stop));
+    MGGX_HIP(hipEventElapsedTime(ms, t->start, t->stop));
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_timer_destroy(void *timer)
+{
+    if (!timer) return MGGX_OK;
+    Timer *t = static_cast<Timer *>(timer);
+    (void)hipEventDestroy(t->start);
+    (void)hipEventDestroy(t->stop);
+    delete t;
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_release_cached(void)
+{
+    mggx::State &s = state();
+    if (s.device >= 0) MGGX_HIP(hipStreamSynchronize(s.stream));
+    for (mggx::Plan *p : s.plans) mggx::plan_free(p);
+    s.plans.clear();
+    if (s.ws) {
+        MGGX_HIP(hipFree(s.ws));
+        s.ws = nullptr;
+        s.ws_bytes = 0;
+    }
+    return MGGX_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Utility kernels.
+namespace {
+
+__global__ void __launch_bounds__(256) k_copy16(int4 *__restrict__ dst, const int4 *__restrict__ src, size_t n16)
+{
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (; i < n16; i += stride) dst[i] = src[i];
+}
+
+__global__ void __launch_bounds__(256) k_cast_bf16(unsigned short *__restrict__ dst, const float *__restrict__ src, long long n)
+{
+    long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long stride = (long long)gridDim.x * 256;
+    for (; i < n; i += stride) {
+        unsigned u = __float_as_uint(src[i]);
+        unsigned r;
+        if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu)) r = (u >> 16) | 0x40u;  // quiet NaN
+        else r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;                                    // round to nearest even
+        dst[i] = (unsigned short)r;
+    }
+}
+
+}  // namespace
+
+MGGX_EXPORT int mggx_copy_bytes(void *d_dst, const void *d_src, size_t n)
+{
+    if (!d_dst || !d_src || (n % 16)) return fail(MGGX_EINVAL, "copy_bytes: NULL pointer or size not a multiple of 16");
+    if (!n) return MGGX_OK;
+    const size_t n16 = n / 16;
+    size_t blocks = (n16 + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    k_copy16<<<dim3((unsigned)blocks), dim3(256), 0, state().stream>>>((int4 *)d_dst, (const int4 *)d_src, n16);
+    MGGX_LAUNCH_CHECK("k_copy16");
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_cast_f32_to_bf16(void *d_dst, const float *d_src, int64_t n)
+{
+    if (n < 0 || (n && (!d_dst || !d_src))) return fail(MGGX_EINVAL, "cast_f32_to_bf16: bad argument");
+    if (!n) return MGGX_OK;
+    long long blocks = (n + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    k_cast_bf16<<<dim3((unsigned)blocks), dim3(256), 0, state().stream>>>((unsigned short *)d_dst, d_src, (long long)n);
+    MGGX_LAUNCH_CHECK("k_cast_bf16");
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_last_agg_kernel(char *buf, size_t len)
+{
+    if (!buf || !len) return fail(MGGX_EINVAL, "last_agg_kernel: NULL buffer");
+    snprintf(buf, len, "%s", state().last_kernel);
+    return MGGX_OK;
+}

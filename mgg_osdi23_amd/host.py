@@ -1,0 +1,311 @@
+"""ctypes binding of libmggx.so: the same C ABI the C++ layer in include/mgg/ uses.
+
+Function names follow the reference's host API (split_CSR, build_part,
+mgg_SAG_np_div, mgg_GIN_np_div, SAG_host, dense/softmax forward).  Device
+memory is passed as torch CUDA tensors (their data_ptr()); torch is used for
+nothing else.  There is no CPU fallback: a missing library raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional, Tuple
+
+import numpy as np
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libmggx.so")
+
+AGG_ACCUMULATE = 1
+AGG_GIN = 2
+AGG_RELU = 4
+F32 = 0
+BF16 = 1
+
+
+class MggxError(RuntimeError):
+    pass
+
+
+class _AggOpts(C.Structure):
+    _fields_ = [("flags", C.c_uint32), ("eps", C.c_float), ("ld_in", C.c_int64), ("ld_out", C.c_int64),
+                ("d_row_scale_out", C.c_void_p), ("in_dtype", C.c_int)]
+
+
+class _DenseOpts(C.Structure):
+    _fields_ = [("ld_x", C.c_int64), ("ld_out", C.c_int64), ("d_row_scale", C.c_void_p), ("relu", C.c_uint32)]
+
+
+_lib = None
+
+# every symbol include/mggx.h declares
+EXPORTS = [
+    "mggx_last_error", "mggx_version", "mggx_init", "mggx_device_name", "mggx_set_stream", "mggx_sync",
+    "mggx_malloc", "mggx_free", "mggx_memset", "mggx_memcpy_h2d", "mggx_memcpy_d2h", "mggx_memcpy_d2d",
+    "mggx_timer_create", "mggx_timer_start", "mggx_timer_stop", "mggx_timer_elapsed_ms", "mggx_timer_destroy",
+    "mggx_release_cached", "mggx_range_partition", "mggx_split_csr", "mggx_build_part", "mggx_graph_read",
+    "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
+    "mggx_fill_uniform", "mggx_build_part_device", "mggx_sag_np_div", "mggx_sag_parts", "mggx_spmm",
+    "mggx_dense_xw", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_last_agg_kernel",
+]
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise MggxError("libmggx.so is not built (run `python -m mgg_osdi23_amd.build`); there is no fallback path")
+        _lib = C.CDLL(LIB_PATH)
+        _lib.mggx_last_error.restype = C.c_char_p
+        _lib.mggx_version.restype = C.c_char_p
+    return _lib
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise MggxError("mggx error %d: %s" % (rc, lib().mggx_last_error().decode()))
+
+
+def _iptr(a: Optional[np.ndarray]):
+    if a is None:
+        return None
+    assert a.dtype == np.int32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(C.POINTER(C.c_int))
+
+
+def _dptr(t) -> C.c_void_p:
+    """Device address of a torch CUDA tensor (None -> NULL)."""
+    if t is None:
+        return C.c_void_p(0)
+    assert t.is_cuda and t.is_contiguous(), "device tensors must be contiguous CUDA tensors"
+    return C.c_void_p(t.data_ptr())
+
+
+# --------------------------------------------------------------------------- host-side graph preparation
+def range_partition(num_nodes: int, num_gpus: int, pe: int) -> Tuple[int, int, int]:
+    npp, lb, ub = C.c_int(), C.c_int(), C.c_int()
+    _check(lib().mggx_range_partition(num_nodes, num_gpus, pe, C.byref(npp), C.byref(lb), C.byref(ub)))
+    return npp.value, lb.value, ub.value
+
+
+def split_CSR(ptr: np.ndarray, col: np.ndarray, lb: int, ub: int):
+    """-> (local_ptr, remote_ptr, local_col_idx, remote_col_idx), the reference's return order."""
+    ptr = np.ascontiguousarray(ptr, dtype=np.int32)
+    col = np.ascontiguousarray(col, dtype=np.int32)
+    nl, nr = C.c_int64(), C.c_int64()
+    _check(lib().mggx_split_csr(_iptr(ptr), _iptr(col), lb, ub, None, None, None, None, C.byref(nl), C.byref(nr)))
+    rows = ub - lb
+    lp = np.zeros(rows + 1, np.int32)
+    rp = np.zeros(rows + 1, np.int32)
+    lc = np.zeros(nl.value, np.int32)
+    rc = np.zeros(nr.value, np.int32)
+    _check(lib().mggx_split_csr(_iptr(ptr), _iptr(col), lb, ub, _iptr(lp), _iptr(rp), _iptr(lc), _iptr(rc),
+                                C.byref(nl), C.byref(nr)))
+    return lp, rp, lc, rc
+
+
+def build_part(indptr: np.ndarray, num_nodes: int, part_size: int, compat: bool = True):
+    """-> (partPtr, part2Node, node2Part), the reference's return order."""
+    indptr = np.ascontiguousarray(indptr, dtype=np.int32)
+    n = C.c_int()
+    _check(lib().mggx_build_part(_iptr(indptr), num_nodes, part_size, int(compat), None, None, None, C.byref(n)))
+    pp = np.zeros(n.value + 1, np.int32)
+    p2n = np.zeros(n.value, np.int32)
+    n2p = np.zeros(num_nodes + 2, np.int32)
+    _check(lib().mggx_build_part(_iptr(indptr), num_nodes, part_size, int(compat), _iptr(pp), _iptr(p2n), _iptr(n2p),
+                                 C.byref(n)))
+    return pp, p2n, n2p
+
+
+def graph_read(beg_file: str, csr_file: str, weight_file: str):
+    v, e = C.c_int(), C.c_int()
+    _check(lib().mggx_graph_read(beg_file.encode(), csr_file.encode(), weight_file.encode(), C.byref(v), C.byref(e),
+                                 None, None, None))
+    beg = np.zeros(v.value + 1, np.int32)
+    csr = np.zeros(e.value, np.int32)
+    w = np.zeros(e.value, np.int32)
+    _check(lib().mggx_graph_read(beg_file.encode(), csr_file.encode(), weight_file.encode(), C.byref(v), C.byref(e),
+                                 _iptr(beg), _iptr(csr), _iptr(w)))
+    return beg, csr, w
+
+
+def graph_write(beg_file: str, csr_file: str, weight_file: str, beg_pos: np.ndarray, csr: np.ndarray,
+                weight: Optional[np.ndarray] = None) -> None:
+    beg_pos = np.ascontiguousarray(beg_pos, dtype=np.int32)
+    csr = np.ascontiguousarray(csr, dtype=np.int32)
+    if weight is not None:
+        weight = np.ascontiguousarray(weight, dtype=np.int32)
+    _check(lib().mggx_graph_write(beg_file.encode(), csr_file.encode(), weight_file.encode(), len(beg_pos) - 1,
+                                  _iptr(beg_pos), _iptr(csr), _iptr(weight)))
+
+
+def mtx_read(path: str):
+    m, l = C.c_int(), C.c_int()
+    _check(lib().mggx_mtx_read(path.encode(), C.byref(m), C.byref(l), None, None))
+    rp = np.zeros(m.value + 1, np.int32)
+    ci = np.zeros(l.value, np.int32)
+    _check(lib().mggx_mtx_read(path.encode(), C.byref(m), C.byref(l), _iptr(rp), _iptr(ci)))
+    return rp, ci
+
+
+def gen_rmat(scale: int, num_nodes: int, num_draws: int, a=0.57, b=0.19, c=0.19, seed=0, scramble=False,
+             row_lo=0, row_hi=None, threads=0):
+    if row_hi is None:
+        row_hi = num_nodes
+    h, nnz = C.c_void_p(), C.c_int64()
+    _check(lib().mggx_gen_rmat(scale, num_nodes, C.c_int64(num_draws), C.c_double(a), C.c_double(b), C.c_double(c),
+                               C.c_uint64(seed), int(scramble), row_lo, row_hi, threads, C.byref(h), C.byref(nnz)))
+    ptr = np.zeros(row_hi - row_lo + 1, np.int32)
+    col = np.zeros(nnz.value, np.int32)
+    _check(lib().mggx_gen_fetch(h, _iptr(ptr), _iptr(col)))
+    return ptr, col
+
+
+def gen_er(num_nodes: int, avg_degree: float, seed=0):
+    h, nnz = C.c_void_p(), C.c_int64()
+    _check(lib().mggx_gen_er(num_nodes, C.c_double(avg_degree), C.c_uint64(seed), C.byref(h), C.byref(nnz)))
+    ptr = np.zeros(num_nodes + 1, np.int32)
+    col = np.zeros(nnz.value, np.int32)
+    _check(lib().mggx_gen_fetch(h, _iptr(ptr), _iptr(col)))
+    return ptr, col
+
+
+def fill_normal(shape, seed: int) -> np.ndarray:
+    out = np.empty(shape, np.float32)
+    _check(lib().mggx_fill_normal(out.ctypes.data_as(C.POINTER(C.c_float)), C.c_int64(out.size), C.c_uint64(seed)))
+    return out
+
+
+def fill_uniform(shape, lo: float, hi: float, seed: int) -> np.ndarray:
+    out = np.empty(shape, np.float32)
+    _check(lib().mggx_fill_uniform(out.ctypes.data_as(C.POINTER(C.c_float)), C.c_int64(out.size), C.c_float(lo),
+                                   C.c_float(hi), C.c_uint64(seed)))
+    return out
+
+
+def glorot(d1: int, d2: int, seed: int) -> np.ndarray:
+    lim = float(np.sqrt(6.0 / (d1 + d2)))
+    return fill_uniform((d1, d2), -lim, lim, seed)
+
+
+# --------------------------------------------------------------------------- device side
+def init(device: int = 0) -> None:
+    _check(lib().mggx_init(device))
+
+
+def use_torch_stream() -> None:
+    """Issue the library's work on torch's current stream (so torch ops and events order with it)."""
+    import torch
+    _check(lib().mggx_set_stream(C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+
+
+def sync() -> None:
+    _check(lib().mggx_sync())
+
+
+_pinned = {}  # CSR tensors of cached plans, by address: keeps the addresses from being reused while cached
+
+
+def _pin(*tensors) -> None:
+    key = tuple(t.data_ptr() if t is not None else 0 for t in tensors)
+    if key in _pinned:
+        return
+    _pinned[key] = tensors
+    while len(_pinned) > 32:  # the library keeps at most 16 plans; anything older is already evicted there
+        _pinned.pop(next(iter(_pinned)))
+
+
+def release_cached() -> None:
+    _check(lib().mggx_release_cached())
+    _pinned.clear()
+
+
+def device_name() -> str:
+    buf = C.create_string_buffer(256)
+    _check(lib().mggx_device_name(buf, 256))
+    return buf.value.decode()
+
+
+def last_agg_kernel() -> str:
+    buf = C.create_string_buffer(256)
+    _check(lib().mggx_last_agg_kernel(buf, 256))
+    return buf.value.decode()
+
+
+def build_part_device(d_indptr, num_nodes: int, part_size: int, compat: bool = True):
+    import torch
+    n = C.c_int()
+    _check(lib().mggx_build_part_device(_dptr(d_indptr), num_nodes, part_size, int(compat), None, None, None, C.byref(n)))
+    pp = torch.zeros(n.value + 1, dtype=torch.int32, device=d_indptr.device)
+    p2n = torch.zeros(max(n.value, 1), dtype=torch.int32, device=d_indptr.device)[: n.value]
+    n2p = torch.zeros(num_nodes + 2, dtype=torch.int32, device=d_indptr.device)
+    _check(lib().mggx_build_part_device(_dptr(d_indptr), num_nodes, part_size, int(compat), _dptr(pp),
+                                        C.c_void_p(p2n.data_ptr()) if n.value else C.c_void_p(pp.data_ptr()),
+                                        _dptr(n2p), C.byref(n)))
+    return pp, p2n, n2p
+
+
+def _agg(out, in_local, in_remote, ptr_l, col_l, ptr_r, col_r, lb, ub, dim, npp, ps, wpb, dist, flags, eps,
+         ld_in, ld_out, row_scale_out):
+    import torch
+    o = _AggOpts()
+    o.flags = flags
+    o.eps = eps
+    o.ld_in = ld_in
+    o.ld_out = ld_out
+    o.d_row_scale_out = row_scale_out.data_ptr() if row_scale_out is not None else None
+    o.in_dtype = BF16 if in_local.dtype == torch.bfloat16 else F32
+    _pin(ptr_l, ptr_r)
+    _check(lib().mggx_sag_np_div(_dptr(out), _dptr(in_local), _dptr(in_remote), _dptr(ptr_l), _dptr(col_l),
+                                 _dptr(ptr_r), _dptr(col_r), lb, ub, dim, npp, ps, wpb, dist, C.byref(o)))
+
+
+def mgg_SAG_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb, ub, dim,
+                   nodePerPE, peid, np_size, warpPerBlock, interleaved_dist, *, input_remote=None, accumulate=False,
+                   ld_in=0, ld_out=0, row_scale_out=None, relu=False):
+    """Argument order of the reference's mgg_SAG_np_div.  `input` is this rank's table; `input_remote` the
+    global-id-indexed table the reference reaches with remote GETs (defaults to `input`, the single-GPU case).
+    The reference adds into `output`; pass accumulate=True for that, the default overwrites."""
+    flags = (AGG_ACCUMULATE if accumulate else 0) | (AGG_RELU if relu else 0)
+    _agg(output, input, input_remote if input_remote is not None else input, row_pointers_l, column_index_l,
+         row_pointers_r, column_index_r, lb, ub, dim, nodePerPE, np_size, warpPerBlock, interleaved_dist, flags, 0.0,
+         ld_in, ld_out, row_scale_out)
+
+
+def mgg_GIN_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb, ub, dim,
+                   nodePerPE, peid, np_size, warpPerBlock, interleaved_dist, eps, *, input_remote=None, ld_in=0,
+                   ld_out=0):
+    _agg(output, input, input_remote if input_remote is not None else input, row_pointers_l, column_index_l,
+         row_pointers_r, column_index_r, lb, ub, dim, nodePerPE, np_size, warpPerBlock, interleaved_dist, AGG_GIN,
+         float(eps), ld_in, ld_out, None)
+
+
+def SAG_host(output, input, row_pointers, column_index, part_pointers, part2Node, lowbound, num_nodes, num_parts,
+             partSize, dim, dimWorker, warpPerBlock, interleaved_dist=1):
+    _pin(row_pointers, part_pointers, part2Node)
+    _check(lib().mggx_sag_parts(_dptr(output), _dptr(input), _dptr(row_pointers), _dptr(column_index),
+                                _dptr(part_pointers), _dptr(part2Node), lowbound, num_nodes, num_parts, partSize, dim,
+                                warpPerBlock, interleaved_dist))
+
+
+def SpMM(output, input, row_pointers, column_index, num_nodes, dim, partSize, warpPerBlock):
+    _pin(row_pointers)
+    _check(lib().mggx_spmm(_dptr(output), _dptr(input), _dptr(row_pointers), _dptr(column_index), num_nodes, dim,
+                           partSize, warpPerBlock))
+
+
+def dense_forward(out, x, w, n, d1, d2, ld_x=0, ld_out=0, row_scale=None, relu=False):
+    o = _DenseOpts()
+    o.ld_x = ld_x
+    o.ld_out = ld_out
+    o.d_row_scale = row_scale.data_ptr() if row_scale is not None else None
+    o.relu = int(relu)
+    _check(lib().mggx_dense_xw(_dptr(out), _dptr(x), _dptr(w), C.c_int64(n), d1, d2, C.byref(o)))
+
+
+def softmax_forward(out, x, n, c, ld_in=0, ld_out=0):
+    _check(lib().mggx_softmax_rows(_dptr(out), _dptr(x), C.c_int64(n), c, C.c_int64(ld_in), C.c_int64(ld_out)))
+
+
+def copy_bytes(dst, src, nbytes: int) -> None:
+    _check(lib().mggx_copy_bytes(_dptr(dst), _dptr(src), C.c_size_t(nbytes)))
