@@ -592,6 +592,7 @@ MGGX_EXPORT int mggx_sag_np_div(float *d_out, const void *d_in_local, const void
     if (ub < lb || !d_ptr_l) return fail(MGGX_EINVAL, "sag_np_div: bad row range [%d,%d) or NULL row pointers", lb, ub);
     if (ps < 1) return fail(MGGX_EINVAL, "sag_np_div: ps %d must be positive", ps);
     if (nodes_per_pe < ub - lb) return fail(MGGX_EINVAL, "sag_np_div: nodes_per_pe %d smaller than the row range", nodes_per_pe);
+    if (ps > (int)mggx::DESC_LEN_MASK) ps = (int)mggx::DESC_LEN_MASK;  // longer than any row: same partitions
     mggx_agg_opts o{};
     if (opts) o = *opts;
     mggx::Plan *plan = nullptr;

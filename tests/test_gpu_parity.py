@@ -1,0 +1,347 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle.
+
+Tolerances (fp32): |gpu - oracle_f64| <= 1e-5 * sum|terms| per element; closed
+forms (all-ones inputs, one-hot inputs) must be bit-exact.
+"""
+import numpy as np
+import pytest
+
+from oracle import orc
+from tests.util import BF16_TOL, FP32_TOL, assert_close_to_oracle, share_of, sym_norm_scale, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def run_agg(host, sh, x_local, x_remote, dim, ps, wpb, dist, *, gin=False, eps=0.0, accumulate_into=None,
+            ld_in=0, ld_out=0, row_scale_out=None, relu=False):
+    import torch
+    R = sh["ub"] - sh["lb"]
+    ldo = ld_out or dim
+    if accumulate_into is not None:
+        out = to_dev(accumulate_into)
+    else:
+        out = torch.full((max(R, 1), ldo), 7.5, dtype=torch.float32, device="cuda")[:R]  # poison: must be overwritten
+    d = dict(ptr_l=to_dev(sh["ptr_l"]), col_l=to_dev(sh["col_l"]) if len(sh["col_l"]) else torch.zeros(1, dtype=torch.int32, device="cuda"),
+             ptr_r=to_dev(sh["ptr_r"]), col_r=to_dev(sh["col_r"]) if len(sh["col_r"]) else torch.zeros(1, dtype=torch.int32, device="cuda"))
+    rs = to_dev(row_scale_out) if row_scale_out is not None else None
+    if gin:
+        host.mgg_GIN_np_div(out, x_local, d["ptr_l"], d["col_l"], d["ptr_r"], d["col_r"], sh["lb"], sh["ub"], dim,
+                            sh["npp"], 0, ps, wpb, dist, eps, input_remote=x_remote, ld_in=ld_in, ld_out=ld_out)
+    else:
+        host.mgg_SAG_np_div(out, x_local, d["ptr_l"], d["col_l"], d["ptr_r"], d["col_r"], sh["lb"], sh["ub"], dim,
+                            sh["npp"], 0, ps, wpb, dist, input_remote=x_remote, accumulate=accumulate_into is not None,
+                            ld_in=ld_in, ld_out=ld_out, row_scale_out=rs, relu=relu)
+    host.sync()
+    return out.cpu().numpy()
+
+
+def oracle_agg(sh, xl, xr, dim, **kw):
+    want = orc.sag_np_div(xl, xr, sh["ptr_l"], sh["col_l"], sh["ptr_r"], sh["col_r"], sh["lb"], sh["ub"], dim, sh["npp"], **kw)
+    rows = np.arange(sh["ub"] - sh["lb"], dtype=np.int32)
+    kw2 = {k: v for k, v in kw.items() if k in ("flags", "eps", "rs_in", "rs_out")}
+    kw2["flags"] = kw2.get("flags", 0) & ~orc.ACCUMULATE
+    mag = orc.sag_np_div_rows(rows, xl, xr, sh["ptr_l"], sh["col_l"], sh["ptr_r"], sh["col_r"], sh["lb"], sh["ub"], dim,
+                              sh["npp"], abs_sum=True, **kw2)
+    return want, mag
+
+
+@pytest.fixture(scope="module")
+def er_graph():
+    from mgg_osdi23_amd import host
+    return host.gen_er(4096, 16.0, seed=0)
+
+
+@pytest.fixture(scope="module")
+def rmat_graph():
+    from mgg_osdi23_amd import host
+    V = 6000
+    ptr, col = host.gen_rmat(13, V, 220_000, seed=5)
+    return V, ptr, col
+
+
+# --------------------------------------------------------------------------- config 1
+@pytest.mark.parametrize("num_gpus,pe", [(1, 0), (8, 0), (8, 3), (8, 7)])
+def test_config1_er_sum_aggregation(gpu, er_graph, num_gpus, pe):
+    """4096-node Erdos-Renyi graph, avg degree 16, self loops, fp32 dim 16 ~U[-1,1] seed 0, ps=16:
+    plain sum and D^-1/2 A D^-1/2 weighting; whole graph and an 8-way share with local/remote tables."""
+    ptr, col = er_graph
+    V, dim = 4096, 16
+    x = gpu.fill_uniform((V, dim), -1.0, 1.0, seed=0)
+    sh = share_of(ptr, col, V, num_gpus, pe)
+    xl = x[sh["lb"]:sh["ub"]]
+    got = run_agg(gpu, sh, to_dev(xl), to_dev(x), dim, 16, 4, 1)
+    want, mag = oracle_agg(sh, xl, x, dim)
+    assert_close_to_oracle(got, want, mag, FP32_TOL, "plain sum")
+    # symmetric normalisation: pre-scaled table, post-scaled rows
+    s = sym_norm_scale(ptr)
+    xs = (x * s[:, None]).astype(np.float32)
+    got = run_agg(gpu, sh, to_dev(xs[sh["lb"]:sh["ub"]]), to_dev(xs), dim, 16, 4, 1, row_scale_out=s[sh["lb"]:sh["ub"]])
+    want, mag = oracle_agg(sh, xl, x, dim, rs_in=s, rs_out=s[sh["lb"]:sh["ub"]])
+    assert_close_to_oracle(got, want, mag, FP32_TOL, "sym-norm")
+
+
+# --------------------------------------------------------------------------- closed forms (bit-exact)
+@pytest.mark.parametrize("dim", [16, 41, 64])
+def test_all_ones_gives_degree_exactly(gpu, rmat_graph, dim):
+    V, ptr, col = rmat_graph
+    sh = share_of(ptr, col, V, 4, 1)
+    ones = np.ones((V, dim), np.float32)
+    got = run_agg(gpu, sh, to_dev(ones[sh["lb"]:sh["ub"]]), to_dev(ones), dim, 16, 8, 2)
+    deg = (np.diff(sh["ptr_l"]) + np.diff(sh["ptr_r"])).astype(np.float32)
+    assert np.array_equal(got, np.repeat(deg[:, None], dim, 1))
+    got = run_agg(gpu, sh, to_dev(ones[sh["lb"]:sh["ub"]]), to_dev(ones), dim, 16, 8, 2, gin=True, eps=0.5)
+    assert np.array_equal(got, np.repeat((deg + 1.5)[:, None], dim, 1))
+
+
+def test_one_hot_gives_adjacency_rows_exactly(gpu):
+    ptr, col = gpu.gen_rmat(7, 100, 700, seed=11)
+    V = 100
+    eye = np.zeros((V, 128), np.float32)
+    eye[np.arange(V), np.arange(V)] = 1.0
+    sh = share_of(ptr, col, V, 2, 1)
+    got = run_agg(gpu, sh, to_dev(eye[sh["lb"]:sh["ub"]]), to_dev(eye), 128, 4, 2, 1)
+    A = np.zeros((sh["ub"] - sh["lb"], 128), np.float32)
+    for r in range(sh["lb"], sh["ub"]):
+        for e in range(ptr[r], ptr[r + 1]):
+            A[r - sh["lb"], col[e]] += 1.0
+    assert np.array_equal(got, A)
+
+
+# --------------------------------------------------------------------------- knob independence
+@pytest.mark.parametrize("ps", [1, 2, 4, 8, 16, 32, 65536])
+@pytest.mark.parametrize("wpb,dist", [(1, 1), (2, 4), (4, 1), (8, 1), (8, 16), (16, 2)])
+def test_knobs_change_speed_not_result(gpu, rmat_graph, ps, wpb, dist):
+    V, ptr, col = rmat_graph
+    dim = 16
+    x = gpu.fill_normal((V, dim), seed=2)
+    sh = share_of(ptr, col, V, 4, 0)  # rank 0 owns the hubs of an unscrambled RMAT graph
+    xl = x[sh["lb"]:sh["ub"]]
+    got = run_agg(gpu, sh, to_dev(xl), to_dev(x), dim, ps, wpb, dist)
+    want, mag = oracle_agg(sh, xl, x, dim)
+    assert_close_to_oracle(got, want, mag, FP32_TOL, "ps=%d wpb=%d dist=%d" % (ps, wpb, dist))
+
+
+# --------------------------------------------------------------------------- widths, strides, options
+@pytest.mark.parametrize("dim", [1, 2, 3, 4, 5, 8, 12, 16, 17, 24, 32, 41, 47, 64, 100, 128, 200, 256])
+def test_feature_widths(gpu, rmat_graph, dim):
+    V, ptr, col = rmat_graph
+    x = gpu.fill_normal((V, dim), seed=100 + dim)
+    sh = share_of(ptr, col, V, 2, 0)
+    xl = x[sh["lb"]:sh["ub"]]
+    got = run_agg(gpu, sh, to_dev(xl), to_dev(x), dim, 16, 4, 2)
+    want, mag = oracle_agg(sh, xl, x, dim)
+    assert_close_to_oracle(got, want, mag, FP32_TOL, "dim=%d" % dim)
+
+
+@pytest.mark.parametrize("dim,ld", [(41, 44), (16, 20), (47, 48), (10, 12)])
+def test_padded_row_strides(gpu, rmat_graph, dim, ld):
+    V, ptr, col = rmat_graph
+    xp = gpu.fill_normal((V, ld), seed=9)  # padding columns hold junk on purpose
+    sh = share_of(ptr, col, V, 2, 1)
+    got = run_agg(gpu, sh, to_dev(xp[sh["lb"]:sh["ub"]]), to_dev(xp), dim, 8, 4, 1, ld_in=ld, ld_out=ld)
+    x = np.ascontiguousarray(xp[:, :dim])
+    want, mag = oracle_agg(sh, x[sh["lb"]:sh["ub"]], x, dim)
+    assert_close_to_oracle(got[:, :dim], want, mag, FP32_TOL, "dim=%d ld=%d" % (dim, ld))
+    assert np.all(got[:, dim:] == 7.5), "padding columns of the output must stay untouched"
+
+
+@pytest.mark.parametrize("dim", [16, 41, 64])
+def test_gin_accumulate_relu(gpu, rmat_graph, dim):
+    V, ptr, col = rmat_graph
+    x = gpu.fill_normal((V, dim), seed=4)
+    sh = share_of(ptr, col, V, 3, 1)
+    xl = x[sh["lb"]:sh["ub"]]
+    R = sh["ub"] - sh["lb"]
+    # GIN: (1+eps) x_v + sum
+    got = run_agg(gpu, sh, to_dev(xl), to_dev(x), dim, 16, 8, 1, gin=True, eps=0.25)
+    want, mag = oracle_agg(sh, xl, x, dim, flags=orc.GIN, eps=0.25)
+    assert_close_to_oracle(got, want, mag, FP32_TOL, "GIN")
+    # accumulate: out += sum (the reference's SAG behaviour)
+    base = gpu.fill_normal((R, dim), seed=5)
+    got = run_agg(gpu, sh, to_dev(xl), to_dev(x), dim, 16, 8, 1, accumulate_into=base)
+    want, mag = oracle_agg(sh, xl, x, dim, flags=orc.ACCUMULATE, out=base.copy())
+    assert_close_to_oracle(got, want, mag + np.abs(base), FP32_TOL, "accumulate")
+    # ReLU epilogue
+    got = run_agg(gpu, sh, to_dev(xl), to_dev(x), dim, 16, 8, 1, relu=True)
+    want, mag = oracle_agg(sh, xl, x, dim)
+    assert_close_to_oracle(got, np.maximum(want, 0), mag, FP32_TOL, "relu")
+
+
+# --------------------------------------------------------------------------- ragged / empty inputs
+def test_empty_rows_isolated_nodes_and_hub(gpu):
+    # hand-built graph: empty rows at both ends and in the middle, one hub with 5000 neighbors
+    V, dim = 300, 16
+    rows = [[] for _ in range(V)]
+    rng = np.random.default_rng(0)
+    rows[5] = list(rng.integers(0, V, 5000))
+    rows[6] = [1, 2, 3]
+    rows[150] = list(rng.integers(0, V, 33))
+    rows[298] = [0]
+    ptr = np.zeros(V + 1, np.int32)
+    ptr[1:] = np.cumsum([len(r) for r in rows])
+    col = np.array([c for r in rows for c in r], np.int32)
+    x = gpu.fill_normal((V, dim), seed=8)
+    for num_gpus, pe in [(1, 0), (2, 0), (2, 1)]:
+        sh = share_of(ptr, col, V, num_gpus, pe)
+        xl = x[sh["lb"]:sh["ub"]]
+        for ps, wpb, dist in [(16, 1, 1), (16, 4, 1), (4, 2, 3), (65536, 4, 1)]:
+            got = run_agg(gpu, sh, to_dev(xl), to_dev(x), dim, ps, wpb, dist)
+            want, mag = oracle_agg(sh, xl, x, dim)
+            assert_close_to_oracle(got, want, mag, FP32_TOL, "ragged %s" % ((num_gpus, pe, ps, wpb, dist),))
+            got = run_agg(gpu, sh, to_dev(xl), to_dev(x), dim, ps, wpb, dist, gin=True, eps=0.0)
+            want, mag = oracle_agg(sh, xl, x, dim, flags=orc.GIN)
+            assert_close_to_oracle(got, want, mag, FP32_TOL, "ragged GIN")
+
+
+def test_graph_without_edges_and_zero_rows(gpu):
+    import torch
+    V, dim = 64, 16
+    ptr = np.zeros(V + 1, np.int32)
+    col = np.zeros(0, np.int32)
+    x = gpu.fill_normal((V, dim), seed=1)
+    sh = share_of(ptr, col, V, 1, 0)
+    got = run_agg(gpu, sh, to_dev(x), to_dev(x), dim, 16, 4, 1)
+    assert np.array_equal(got, np.zeros((V, dim), np.float32))
+    # zero rows: a no-op that must not fail
+    z = torch.zeros(1, dtype=torch.int32, device="cuda")
+    gpu.mgg_SAG_np_div(torch.zeros(1, dim, device="cuda"), to_dev(x), z, z, z, z, 0, 0, dim, 16, 0, 16, 4, 1)
+    gpu.sync()
+
+
+# --------------------------------------------------------------------------- explicit partition arrays
+@pytest.mark.parametrize("ps,wpb,dist", [(16, 4, 1), (3, 2, 2), (32, 8, 1)])
+def test_explicit_partition_arrays(gpu, rmat_graph, ps, wpb, dist):
+    """SAG_host / SAG_host_fused_interleaved (local half): build_part arrays in, out += partition sums."""
+    import torch
+    V, ptr, col = rmat_graph
+    dim = 16
+    sh = share_of(ptr, col, V, 2, 1)
+    R = sh["ub"] - sh["lb"]
+    x = gpu.fill_normal((V, dim), seed=6)
+    xl = np.ascontiguousarray(x[sh["lb"]:sh["ub"]])
+    pp, p2n, _ = orc.build_part(sh["ptr_l"], R, ps)
+    base = gpu.fill_normal((R, dim), seed=7)
+    out = to_dev(base)
+    gpu.SAG_host(out, to_dev(xl), to_dev(sh["ptr_l"]), to_dev(sh["col_l"]), to_dev(pp), to_dev(p2n), sh["lb"], R, len(p2n),
+                 ps, dim, 32, wpb, dist)
+    gpu.sync()
+    want = orc.sag_parts(xl, sh["col_l"], pp, p2n, sh["lb"], dim, base.copy())
+    only_local = dict(sh, ptr_r=np.zeros(R + 1, np.int32), col_r=np.zeros(0, np.int32))
+    _, mag = oracle_agg(only_local, xl, x, dim)
+    assert_close_to_oracle(out.cpu().numpy(), want, mag + np.abs(base), FP32_TOL, "explicit parts")
+
+
+def test_explicit_parts_missing_terminal_entry(gpu):
+    """The reference leaves partPtr[numParts] at 0 when the last node has no neighbors; lengths come from the row
+    pointers here, so the last partition is still summed."""
+    ptr = np.array([0, 3, 3, 8, 8], np.int32)
+    col = np.array([0, 1, 3, 0, 1, 2, 3, 2], np.int32)
+    pp, p2n, _ = orc.build_part(ptr, 4, 2)
+    assert pp[-1] == 0
+    x = np.arange(4 * 4, dtype=np.float32).reshape(4, 4) + 1
+    import torch
+    out = torch.zeros(4, 4, device="cuda")
+    gpu.SAG_host(out, to_dev(x), to_dev(ptr), to_dev(col), to_dev(pp), to_dev(p2n), 0, 4, len(p2n), 2, 4, 32, 2, 1)
+    gpu.sync()
+    want = orc.sag_ref(x, ptr, col)
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
+def test_single_gpu_spmm(gpu, rmat_graph):
+    import torch
+    V, ptr, col = rmat_graph
+    dim = 32
+    x = gpu.fill_normal((V, dim), seed=12)
+    out = torch.zeros(V, dim, device="cuda")
+    gpu.SpMM(out, to_dev(x), to_dev(ptr), to_dev(col), V, dim, 16, 8)
+    gpu.sync()
+    want = orc.sag_np_div(x, x, ptr, col, None, None, 0, V, dim, V)
+    rows = np.arange(V, dtype=np.int32)
+    mag = orc.sag_np_div_rows(rows, x, x, ptr, col, None, None, 0, V, dim, V, abs_sum=True)
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "spmm")
+
+
+# --------------------------------------------------------------------------- GPU-side build_part (bit-exact)
+@pytest.mark.parametrize("ps", [1, 2, 16, 65536])
+def test_build_part_device_bit_exact(gpu, rmat_graph, ps):
+    V, ptr, col = rmat_graph
+    for indptr in (ptr, np.array([0, 3, 3, 8, 8], np.int32), np.array([0, 0, 0], np.int32), np.array([0, 5], np.int32)):
+        n = len(indptr) - 1
+        want = orc.build_part(indptr, n, ps)
+        got = gpu.build_part_device(to_dev(indptr), n, ps, compat=True)
+        for g, w, name in zip(got, want, ("partPtr", "part2Node", "node2Part")):
+            assert np.array_equal(g.cpu().numpy(), w), name
+
+
+# --------------------------------------------------------------------------- dense update and softmax
+@pytest.mark.parametrize("n,d1,d2", [(1000, 602, 16), (1000, 16, 41), (777, 100, 64), (512, 64, 64), (300, 64, 47),
+                                     (256, 128, 128), (65, 7, 3), (1, 1, 1), (130, 33, 130)])
+def test_dense_update(gpu, n, d1, d2):
+    import torch
+    x = gpu.fill_normal((n, d1), seed=20)
+    w = gpu.glorot(d1, d2, seed=21)
+    out = torch.full((n, d2), 3.0, device="cuda")
+    gpu.dense_forward(out, to_dev(x), to_dev(w), n, d1, d2)
+    gpu.sync()
+    want = orc.dense(x, w, f64=True)
+    mag = np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64)
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "dense %dx%dx%d" % (n, d1, d2))
+
+
+def test_dense_closed_forms_and_epilogue(gpu):
+    import torch
+    n, d1, d2 = 200, 602, 16
+    out = torch.zeros(n, d2, device="cuda")
+    gpu.dense_forward(out, torch.ones(n, d1, device="cuda"), torch.ones(d1, d2, device="cuda"), n, d1, d2)
+    gpu.sync()
+    assert np.array_equal(out.cpu().numpy(), np.full((n, d2), float(d1), np.float32))  # the reference's all-ones setup
+    x = gpu.fill_normal((n, 48), seed=3)
+    out = torch.zeros(n, 48, device="cuda")
+    gpu.dense_forward(out, to_dev(x), torch.eye(48, device="cuda"), n, 48, 48)
+    gpu.sync()
+    assert np.array_equal(out.cpu().numpy(), x)
+    # row scale + relu epilogue, padded output stride
+    s = gpu.fill_uniform((n,), 0.1, 2.0, seed=4)
+    w = gpu.glorot(48, 41, seed=5)
+    out = torch.full((n, 44), 9.0, device="cuda")
+    gpu.dense_forward(out, to_dev(x), to_dev(w), n, 48, 41, ld_out=44, row_scale=to_dev(s), relu=True)
+    gpu.sync()
+    want = np.maximum(orc.dense(x, w) * s[:, None], 0)
+    mag = (np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64)) * s[:, None]
+    got = out.cpu().numpy()
+    assert_close_to_oracle(got[:, :41], want, mag, FP32_TOL, "dense epilogue")
+    assert np.all(got[:, 41:] == 9.0)
+
+
+@pytest.mark.parametrize("n,c", [(1000, 41), (333, 47), (64, 1), (10, 200), (5, 64)])
+def test_softmax_rows(gpu, n, c):
+    import torch
+    x = gpu.fill_normal((n, c), seed=30) * 5
+    out = torch.zeros(n, c, device="cuda")
+    gpu.softmax_forward(out, to_dev(x), n, c)
+    gpu.sync()
+    want = orc.softmax_rows(x)
+    got = out.cpu().numpy()
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-7)
+    assert np.allclose(got.sum(1), 1.0, atol=1e-5)
+    # in place
+    t = to_dev(x)
+    gpu.softmax_forward(t, t, n, c)
+    gpu.sync()
+    assert np.allclose(t.cpu().numpy(), want, rtol=1e-5, atol=1e-7)
+
+
+# --------------------------------------------------------------------------- bf16 tables, fp32 accumulation
+@pytest.mark.parametrize("dim", [8, 64, 128, 256])
+def test_bf16_tables(gpu, rmat_graph, dim):
+    import torch
+    V, ptr, col = rmat_graph
+    x = gpu.fill_normal((V, dim), seed=40)
+    xb = to_dev(x).to(torch.bfloat16)
+    xf = xb.to(torch.float32).cpu().numpy()  # the exact values the kernel sees
+    sh = share_of(ptr, col, V, 2, 0)
+    got = run_agg(gpu, sh, xb[sh["lb"]:sh["ub"]].contiguous(), xb, dim, 16, 8, 1)
+    want, mag = oracle_agg(sh, xf[sh["lb"]:sh["ub"]], xf, dim)
+    assert_close_to_oracle(got, want, mag, FP32_TOL, "bf16 in, fp32 accumulate (vs the same rounded inputs)")
+    want_f, mag_f = oracle_agg(sh, x[sh["lb"]:sh["ub"]], x, dim)
+    assert_close_to_oracle(got, want_f, mag_f, BF16_TOL, "bf16 in vs unrounded inputs")
