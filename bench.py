@@ -1,0 +1,295 @@
+#!/usr/bin/env python3
+"""Benchmark of the neighbor-partitioned aggregation path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gcn2|share] [--no-cpu]
+
+Default workload (`gcn2`): 2-layer GCN forward on the whole graph -- seeded RMAT
+power-law graph (a=.57 b=.19 c=.19), 233,000 nodes, ~114 M undirected edges,
+self loops, D^-1/2 (A+I) D^-1/2 weighting; fp32 features 602 -> 16 -> 41, Glorot
+weights; ps=16, wpb=8.  One step = dense, aggregate, dense, aggregate, softmax,
+all inputs resident in HBM.  Prints ONE JSON line: forward ms per step, the
+roofline figures of the dominant (aggregation) kernel from HIP events recorded
+inside the timed region, and the CPU oracle timed on this host's cores.
+
+`share` times the aggregation alone on rank 0's 1/8 share of a 4.2 M-node RMAT
+graph with the remote rows pre-staged in a second HBM table.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def agg_bytes(nnz, rows, dim, s_in=4, ptr_arrays=1, gin=False):
+    """Algorithmic bytes of one aggregation call: per edge one index and one feature row, per row one output
+    row and the row pointers; no cache credit."""
+    b = nnz * (4 + dim * s_in) + rows * dim * 4 + (rows + 1) * 4 * ptr_arrays
+    if gin:
+        b += rows * dim * s_in
+    return b
+
+
+class StageTimer:
+    """HIP events (torch wrappers on the stream the library launches on) around each stage of every step."""
+
+    def __init__(self, torch, names):
+        self.torch = torch
+        self.names = names
+        self.events = []
+
+    def step(self, stages):
+        ev = [self.torch.cuda.Event(enable_timing=True)]
+        ev[0].record()
+        for fn in stages:
+            fn()
+            e = self.torch.cuda.Event(enable_timing=True)
+            e.record()
+            ev.append(e)
+        self.events.append(ev)
+
+    def averages(self):
+        self.torch.cuda.synchronize()
+        sums = [0.0] * len(self.names)
+        for ev in self.events:
+            for i in range(len(self.names)):
+                sums[i] += ev[i].elapsed_time(ev[i + 1])
+        n = max(1, len(self.events))
+        return {k: s / n for k, s in zip(self.names, sums)}
+
+
+def load_traffic(kernel_key):
+    """HBM bytes per launch measured offline with rocprofv3 --pmc (see profiles/); None when not recorded."""
+    p = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(p):
+        with open(p) as f:
+            return json.load(f).get(kernel_key)
+    return None
+
+
+def bench_gcn2(args, torch, host):
+    V, scale, draws = 233_000, 18, 216_000_000
+    in_dim, hidden, out_dim = 602, 16, 41
+    ps, wpb, dist = args.ps, args.wpb, args.dist
+    if args.small:
+        V, scale, draws = 20_000, 15, 2_000_000
+    t0 = time.time()
+    ptr, col = host.gen_rmat(scale, V, draws, seed=42)
+    nnz = int(len(col))
+    log("graph: V=%d nnz=%d (undirected %d) in %.1fs" % (V, nnz, (nnz - V) // 2, time.time() - t0))
+    X = host.fill_normal((V, in_dim), seed=1)
+    W1 = host.glorot(in_dim, hidden, seed=2)
+    W2 = host.glorot(hidden, out_dim, seed=3)
+    deg = np.diff(ptr).astype(np.float64)
+    s = (1.0 / np.sqrt(np.maximum(deg, 1.0))).astype(np.float32)
+
+    # Device layout: the 41-wide layer is kept with a row stride of 44 floats (zero padding columns), so its rows
+    # are 16-byte aligned and move as whole dwordx4 loads; bytes and flops are still counted at width 41.
+    ldo = (out_dim + 3) & ~3
+    W2p = np.zeros((hidden, ldo), np.float32)
+    W2p[:, :out_dim] = W2
+    dev = "cuda"
+    d_ptr = torch.from_numpy(ptr).to(dev)
+    d_col = torch.from_numpy(col).to(dev)
+    d_zero_ptr = torch.zeros(V + 1, dtype=torch.int32, device=dev)
+    d_zero_col = torch.zeros(1, dtype=torch.int32, device=dev)
+    d_X = torch.from_numpy(X).to(dev)
+    d_W1 = torch.from_numpy(W1).to(dev)
+    d_W2 = torch.from_numpy(W2p).to(dev)
+    d_s = torch.from_numpy(s).to(dev)
+    d_Y1 = torch.empty(V, hidden, device=dev)
+    d_H1 = torch.empty(V, hidden, device=dev)
+    d_Y2 = torch.empty(V, ldo, device=dev)
+    d_H2 = torch.empty(V, ldo, device=dev)
+    d_P = torch.empty(V, out_dim, device=dev)
+
+    stages = [
+        lambda: host.dense_forward(d_Y1, d_X, d_W1, V, in_dim, hidden, row_scale=d_s),
+        lambda: host.mgg_SAG_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, ps, wpb, dist,
+                                    row_scale_out=d_s),
+        lambda: host.dense_forward(d_Y2, d_H1, d_W2, V, hidden, ldo, row_scale=d_s),
+        lambda: host.mgg_SAG_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, 0, ps, wpb, dist,
+                                    row_scale_out=d_s),
+        lambda: host.softmax_forward(d_P, d_H2, V, out_dim, ld_in=ldo),
+    ]
+    names = ["dense1", "agg1", "dense2", "agg2", "softmax"]
+
+    def step():
+        for fn in stages:
+            fn()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = StageTimer(torch, names)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        timer.step(stages)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    avg = timer.averages()
+    log("stage ms:", {k: round(v, 4) for k, v in avg.items()}, "wall ms/step %.4f" % wall_ms)
+
+    b1 = agg_bytes(nnz, V, hidden)
+    b2 = agg_bytes(nnz, V, out_dim)
+    dom = "agg2" if avg["agg2"] >= avg["agg1"] else "agg1"
+    dom_bytes = b2 if dom == "agg2" else b1
+    achieved = dom_bytes / (avg[dom] * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": "k_agg (%s, dim %d)" % (dom, out_dim if dom == "agg2" else hidden),
+                "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": load_traffic("gcn2_" + dom),
+                "algorithmic_bytes": dom_bytes, "avg_launch_ms": round(avg[dom], 4)}
+    extra = {
+        "stage_ms": {k: round(v, 4) for k, v in avg.items()},
+        "agg1_gbps": round(b1 / (avg["agg1"] * 1e-3) / 1e9, 1),
+        "agg2_gbps": round(b2 / (avg["agg2"] * 1e-3) / 1e9, 1),
+        "dense1_gflops": round(2.0 * V * in_dim * hidden / (avg["dense1"] * 1e-3) / 1e9, 1),
+        "dense1_gbps": round((V * in_dim * 4 + V * hidden * 4) / (avg["dense1"] * 1e-3) / 1e9, 1),
+    }
+
+    cpu = None
+    parity = None
+    if not args.no_cpu:
+        from oracle import orc
+        th = orc.max_threads()
+        t0 = time.perf_counter()
+        P_ref, H2_ref, H1_ref = orc.gcn2_forward(X, W1, W2, ptr, col, None, None, 0, V, V, rs=s, f64=False, threads=th)
+        cpu_s = time.perf_counter() - t0
+        cpu = {"value": round(cpu_s * 1e3, 1), "unit": "ms", "cores": th, "kind": "port",
+               "sample": "1 full forward of the same workload (OpenMP over rows, fp32)"}
+        P = d_P.cpu().numpy()
+        parity = {"softmax_max_abs_err": float(np.abs(P - P_ref).max()),
+                  "h1_max_rel_err": float(np.abs(d_H1.cpu().numpy() - H1_ref).max() / np.abs(H1_ref).max())}
+        log("cpu forward %.1f ms on %d threads; parity %s" % (cpu_s * 1e3, th, parity))
+
+    return {
+        "metric": "gcn_2layer_fwd_ms", "value": round(wall_ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: 2-layer GCN forward, RMAT(a=.57,b=.19,c=.19) V=%d nnz=%d (self loops, sym-norm), "
+                               "602->16->41 fp32, ps=%d wpb=%d dist=%d" % (V, nnz, ps, wpb, dist)},
+        "roofline": roofline, "cpu_baseline": cpu, "parity": parity, "detail": extra,
+    }
+
+
+def bench_share(args, torch, host):
+    """Aggregation alone on rank 0's share of an 8-way partitioned RMAT graph, remote rows pre-staged."""
+    scale, V, draws, dim, num_gpus = 22, 4_194_304, 52_000_000 * args.share_density, 16, 8
+    ps, wpb, dist = args.ps, args.wpb, args.dist
+    npp, lb, ub = host.range_partition(V, num_gpus, 0)
+    t0 = time.time()
+    ptr, col = host.gen_rmat(scale, V, draws, seed=7, scramble=True, row_lo=lb, row_hi=ub)
+    lp, rp, lc, rc = host.split_CSR(np.concatenate([np.zeros(lb, np.int32), ptr]) if lb else ptr, col, lb, ub)
+    R = ub - lb
+    nnz = len(col)
+    log("share: rows=%d nnz=%d local=%d remote=%d in %.1fs" % (R, nnz, len(lc), len(rc), time.time() - t0))
+    dev = "cuda"
+    x_remote = host.fill_normal((num_gpus * npp, dim), seed=11)
+    d_xr = torch.from_numpy(x_remote).to(dev)
+    d_xl = torch.from_numpy(np.ascontiguousarray(x_remote[lb:ub])).to(dev)  # separate allocation
+    d = [torch.from_numpy(a).to(dev) if len(a) else torch.zeros(1, dtype=torch.int32, device=dev) for a in (lp, lc, rp, rc)]
+    d_out = torch.empty(R, dim, device=dev)
+
+    def call():
+        host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, ps, wpb, dist, input_remote=d_xr)
+
+    for _ in range(args.warmup):
+        call()
+    torch.cuda.synchronize()
+    timer = StageTimer(torch, ["agg"])
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        timer.step([call])
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms = timer.averages()["agg"]
+    nbytes = agg_bytes(nnz, R, dim, ptr_arrays=2)
+    achieved = nbytes / (ms * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu:
+        from oracle import orc
+        th = orc.max_threads()
+        t0 = time.perf_counter()
+        ref = orc.sag_np_div(x_remote[lb:ub], x_remote, lp, lc, rp, rc, lb, ub, dim, npp, f64=False, threads=th)
+        cpu_s = time.perf_counter() - t0
+        err = float(np.abs(d_out.cpu().numpy() - ref).max())
+        cpu = {"value": round(cpu_s * 1e3, 1), "unit": "ms", "cores": th, "kind": "port",
+               "sample": "the same aggregation call, whole share", "max_abs_err_vs_gpu": err}
+    return {
+        "metric": "np_aggregation_ms", "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[3]: rank-0 1/8 share of RMAT V=%d (ids scrambled), rows=%d nnz=%d (local %d, remote %d), "
+                               "fp32 dim %d, ps=%d wpb=%d dist=%d" % (V, R, nnz, len(lc), len(rc), dim, ps, wpb, dist)},
+        "roofline": {"bound": "hbm", "kernel": "k_agg (dim 16, local+remote)", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": load_traffic("share_agg"), "algorithmic_bytes": nbytes, "avg_launch_ms": round(ms, 4)},
+        "cpu_baseline": cpu,
+    }
+
+
+def bench_copy(args, torch, host):
+    """Plain device copy of a known size: the stream-copy ceiling, and the yardstick the profiler's FETCH_SIZE /
+    WRITE_SIZE counters are scaled against."""
+    nbytes = 1 << 30
+    src = torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(args.warmup):
+        host.copy_bytes(dst, src, nbytes)
+    torch.cuda.synchronize()
+    timer = StageTimer(torch, ["copy"])
+    for _ in range(args.steps):
+        timer.step([lambda: host.copy_bytes(dst, src, nbytes)])
+    ms = timer.averages()["copy"]
+    gbps = 2 * nbytes / (ms * 1e-3) / 1e9
+    return {"metric": "stream_copy_gbps", "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": "k_copy16: %d bytes read + %d bytes written per launch" % (nbytes, nbytes)}}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="gcn2", choices=["gcn2", "share", "copy"])
+    ap.add_argument("--ps", type=int, default=16)
+    ap.add_argument("--wpb", type=int, default=8)
+    ap.add_argument("--dist", type=int, default=1)
+    ap.add_argument("--share-density", type=int, default=1, help="multiplies the number of RMAT draws of --workload share")
+    ap.add_argument("--small", action="store_true", help="tiny graph, for a quick functional run")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs one GPU's share on one GPU; --gpus %d is not offered (no collectives, no "
+              "second device are used)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from mgg_osdi23_amd import host
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+    host.init(0)
+    host.use_torch_stream()
+    log("device:", host.device_name())
+    res = {"gcn2": bench_gcn2, "share": bench_share, "copy": bench_copy}[args.workload](args, torch, host)
+    print(json.dumps(res), flush=True)
+
+
+if __name__ == "__main__":
+    main()

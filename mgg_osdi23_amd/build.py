@@ -75,6 +75,26 @@ def build(force: bool = False, jobs: int = 4) -> str:
     return LIB
 
 
+def build_examples(force: bool = False) -> list[str]:
+    """Compiles the harness programs (plain C++ against include/mgg/*.h and libmggx.so) into mgg_osdi23_amd/bin/."""
+    src_dir = os.path.join(PKG_DIR, "harness")
+    out_dir = os.path.join(PKG_DIR, "bin")
+    os.makedirs(out_dir, exist_ok=True)
+    outs = []
+    hdrs = [os.path.join(src_dir, "harness_common.h")] + [
+        os.path.join(ROOT, "include", "mgg", h) for h in os.listdir(os.path.join(ROOT, "include", "mgg"))]
+    for name in sorted(os.listdir(src_dir)):
+        if not name.endswith(".cpp"):
+            continue
+        src = os.path.join(src_dir, name)
+        exe = os.path.join(out_dir, name[:-4])
+        outs.append(exe)
+        if force or not _newer(exe, [src, LIB] + hdrs):
+            _run(["g++", "-O2", "-std=c++17", "-Wall", "-I", os.path.join(ROOT, "include"), "-I", src_dir, src, "-o", exe,
+                  "-L", PKG_DIR, "-lmggx", "-Wl,-rpath,$ORIGIN/.."])
+    return outs
+
+
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--force", action="store_true")

@@ -1,0 +1,61 @@
+// Aggregation-only benchmark: the counterpart of the reference's
+// src/mgg_np_div_kernel.cu (the binary behind its NP / WL / design-space
+// studies).  Same command line, same log lines; times `iters` calls of
+// mgg_SAG_np_div at width `hidden` on one rank's share.
+#include "harness_common.h"
+
+int main(int argc, char *argv[])
+{
+    HarnessArgs a;
+    if (!parse_args(argc, argv, a)) return -1;
+    MGG_CHECK(mggx_init(0));
+    Share s;
+    load_share(a, s);
+    const nidType rows = s.ub - s.lb;
+    const int dim = a.hiddenSize;  // the reference aggregates at hiddenSize (src/mgg_np_div_kernel.cu:186-187)
+
+    // Feature tables: ones, as the reference fills its inputs (:122).  The staged table stands for the
+    // symmetric buffers of all ranks back to back; this rank's own rows sit in a separate allocation.
+    float *d_table = device_filled((size_t)a.num_GPUs * s.nodesPerPE * dim, 1.0f);
+    float *d_local = device_filled((size_t)s.nodesPerPE * dim, 1.0f);
+    float *dsp_out = device_filled((size_t)s.nodesPerPE * dim, 0.0f);
+    mgg_stage_remote(d_table);
+    mgg_options().accumulate = true;  // reference behaviour: every call adds into dsp_out
+
+    // first call builds and caches the partition plan, like the reference's untimed set-up
+    if (a.validate) {
+        mgg_SAG_np_div(dsp_out, d_local, s.d_row_ptr_l, s.d_col_ind_l, s.d_row_ptr_r, s.d_col_ind_r, s.lb, s.ub, dim,
+                       s.nodesPerPE, a.pe, a.partSize, a.warpPerBlock, a.interleaved_dist);
+        std::vector<float> h_out((size_t)rows * dim), h_ref((size_t)s.numNodes * dim, 0.0f), ones((size_t)s.numNodes * dim, 1.0f);
+        MGG_CHECK(mggx_memcpy_d2h(h_out.data(), dsp_out, h_out.size() * sizeof(float)));
+        SAG_ref(h_ref.data(), ones.data(), s.global_row_ptr.data(), s.global_col_ind.data(), s.numNodes, s.numEdges, dim);
+        bool ok = check_equal(h_ref.data(), h_out.data(), rows * dim, dim, s.lb * dim);
+        printf("Validation on PE-{%d}, status: %s\n", a.pe, ok ? "True" : "False");
+        MGG_CHECK(mggx_memset(dsp_out, 0, (size_t)s.nodesPerPE * dim * sizeof(float)));
+    } else {
+        mgg_SAG_np_div(dsp_out, d_local, s.d_row_ptr_l, s.d_col_ind_l, s.d_row_ptr_r, s.d_col_ind_r, s.lb, s.ub, dim,
+                       s.nodesPerPE, a.pe, a.partSize, a.warpPerBlock, a.interleaved_dist);
+    }
+    MGG_CHECK(mggx_sync());
+
+    std::clock_t c_start = std::clock();
+    const double t1 = now_ms();
+    for (int i = 0; i < a.iters; i++)
+        mgg_SAG_np_div(dsp_out, d_local, s.d_row_ptr_l, s.d_col_ind_l, s.d_row_ptr_r, s.d_col_ind_r, s.lb, s.ub, dim,
+                       s.nodesPerPE, a.pe, a.partSize, a.warpPerBlock, a.interleaved_dist);
+    MGG_CHECK(mggx_sync());
+    const double t2 = now_ms();
+    std::clock_t c_end = std::clock();
+    printf("PE-%d, Total (ms): %.3f\n", a.pe, 1000.0 * (c_end - c_start) / CLOCKS_PER_SEC / a.iters);
+    printf("MPI time (ms) %.3f\n", (t2 - t1) / a.iters);  // the line the reference's analysis scripts parse
+
+    mggx_free(dsp_out);
+    mggx_free(d_local);
+    mggx_free(d_table);
+    mggx_free(s.d_row_ptr_l);
+    mggx_free(s.d_col_ind_l);
+    mggx_free(s.d_row_ptr_r);
+    mggx_free(s.d_col_ind_r);
+    printf("===================================\n");
+    return 0;
+}
