@@ -212,6 +212,11 @@ int mggx_cast_f32_to_bf16(void *d_dst, const float *d_src, int64_t n);
  * profiler's HBM byte counters are scaled against. */
 int mggx_copy_bytes(void *d_dst, const void *d_src, size_t n);
 
+/* How the aggregation kernels address feature rows: 0 (default) picks per call -- 32-bit buffer offsets when both
+ * tables lie inside one window of < 2 GiB and < 2^24 rows, 64-bit addresses otherwise; 1 always uses 64-bit
+ * addresses.  Results are identical; the switch exists for tests and measurements. */
+int mggx_set_gather_addressing(int mode);
+
 /* Name and launch count of the aggregation kernel the last mggx_sag_np_div /
  * mggx_sag_parts / mggx_spmm call dispatched (for matching profiler rows). */
 int mggx_last_agg_kernel(char *buf, size_t len);

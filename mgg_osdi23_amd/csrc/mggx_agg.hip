@@ -52,7 +52,16 @@ struct AggArgs {
     unsigned flags;
     float eps;
     int in_is_bf16;
+    // gather addressing
+    unsigned ld_bytes;        // row stride of the feature tables in bytes
+    const void *win_base;     // buffer-load path: one window over both tables ...
+    unsigned win_bytes;       // ... of this many bytes,
+    unsigned delta_l, delta_r;// ... the tables starting at these byte offsets;
+    int sentinel;             // ... and a row index whose offset falls outside the window (reads as zero)
 };
+
+// What padding neighbors read on the 64-bit address path: 4 KiB of zeros.
+static __device__ __align__(256) float g_zero_row[1024];
 
 template <int I, int N, typename F>
 __device__ __forceinline__ void static_for(F &&f)
@@ -79,9 +88,9 @@ __device__ __forceinline__ int slot_bcast(int v, int slot_base)
     if constexpr (LPR == 1) {
         return v;
     } else if constexpr (LPR == 2) {
-        return __builtin_amdgcn_update_dpp(0, v, SRC | (SRC << 2) | ((2 + SRC) << 4) | ((2 + SRC) << 6), 0xf, 0xf, false);
+        return __builtin_amdgcn_update_dpp(v, v, SRC | (SRC << 2) | ((2 + SRC) << 4) | ((2 + SRC) << 6), 0xf, 0xf, true);
     } else if constexpr (LPR == 4) {
-        return __builtin_amdgcn_update_dpp(0, v, SRC | (SRC << 2) | (SRC << 4) | (SRC << 6), 0xf, 0xf, false);
+        return __builtin_amdgcn_update_dpp(v, v, SRC | (SRC << 2) | (SRC << 4) | (SRC << 6), 0xf, 0xf, true);
     } else if constexpr (LPR == 64) {
         return __builtin_amdgcn_readlane(v, SRC);
     } else {
@@ -102,33 +111,59 @@ __device__ __forceinline__ int elem_of(int l, int i)
     else return ModeTraits<MODE>::NV * l + i;
 }
 
-// Unconditional load of this lane's share of table row `r`; lanes past the row
-// width read lane 0's share instead (their values are never used).
-template <int LPR, int MODE>
-__device__ __forceinline__ void gather_row(float (&v)[ModeTraits<MODE>::NV], const void *tbl, long long r, long long ld,
-                                           int l, int dim)
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+template <int MODE>
+__device__ __forceinline__ void unpack16(float (&v)[ModeTraits<MODE>::NV], const v4u t)
 {
-    constexpr int NV = ModeTraits<MODE>::NV;
-    if constexpr (MODE == MODE_F32_VEC4) {
-        const int le = (NV * l < dim) ? l : 0;
-        const float4 t = *reinterpret_cast<const float4 *>(static_cast<const float *>(tbl) + r * ld + 4 * le);
-        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-    } else if constexpr (MODE == MODE_F32_STRIDED) {
-        const float *p = static_cast<const float *>(tbl) + r * ld;
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int d = l + i * LPR;
-            v[i] = p[d < dim ? d : 0];
-        }
-    } else {
-        const int le = (NV * l < dim) ? l : 0;
-        const uint4 t = *reinterpret_cast<const uint4 *>(static_cast<const unsigned short *>(tbl) + r * ld + 8 * le);
+    if constexpr (MODE == MODE_BF16_VEC8) {
         v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xFFFF0000u);
         v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xFFFF0000u);
         v[4] = __uint_as_float(t.z << 16); v[5] = __uint_as_float(t.z & 0xFFFF0000u);
         v[6] = __uint_as_float(t.w << 16); v[7] = __uint_as_float(t.w & 0xFFFF0000u);
+    } else {
+        v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y); v[2] = __uint_as_float(t.z); v[3] = __uint_as_float(t.w);
     }
 }
+
+// Per-slot addressing state of one round.  `cofs` is this lane's byte offset inside a row (lanes past the row width
+// use lane 0's offset: they load valid memory and their values are dropped).
+//   buffer path: offset = (row & 0xFFFFFF) * ld_bytes + cbase inside one window holding both tables; a padding
+//                neighbor carries the sentinel row, whose offset lies past the window, and reads as zero
+//   64-bit path: address = base + row * ld_bytes; a padding neighbor (row < 0) reads the zero row
+template <int LPR, int MODE, bool BUF>
+struct Gather {
+    static constexpr int NV = ModeTraits<MODE>::NV;
+    __amdgpu_buffer_rsrc_t rsrc;
+    unsigned ld24;
+    unsigned cbase;        // buffer path: table offset in the window + cofs
+    const char *base;      // 64-bit path: table + cofs
+    const char *zero;      // 64-bit path: zero row + cofs
+    unsigned ld_bytes;
+    unsigned sofs[4];      // strided mode: byte offsets of this lane's 4 elements inside a row
+
+    __device__ __forceinline__ void load(float (&v)[NV], int row) const
+    {
+        if constexpr (BUF) {
+            const unsigned off = ((unsigned)row & 0xFFFFFFu) * ld24 + cbase;
+            if constexpr (MODE == MODE_F32_STRIDED) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    v[i] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, off + sofs[i], 0, 0));
+            } else {
+                unpack16<MODE>(v, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0));
+            }
+        } else {
+            const char *p = row >= 0 ? base + (unsigned long long)(unsigned)row * ld_bytes : zero;
+            if constexpr (MODE == MODE_F32_STRIDED) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[i] = *reinterpret_cast<const float *>(p + sofs[i]);
+            } else {
+                unpack16<MODE>(v, *reinterpret_cast<const v4u *>(p));
+            }
+        }
+    }
+};
 
 __device__ __forceinline__ float load_self(const AggArgs &a, int row, int d)
 {
@@ -181,7 +216,7 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int row, int l, con
 
 // One wavefront-wide aggregation kernel; see the file header for the scheme.
 // Dynamic LDS: int2 hdr[2*wpb] (head, tail per wavefront), then float vals[2*wpb][cpad].
-template <int LPR, int MODE>
+template <int LPR, int MODE, bool BUF>
 __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
 {
     constexpr int NV = ModeTraits<MODE>::NV;
@@ -206,6 +241,25 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     }
 
     const long long q_wave = ((long long)blockIdx.x * wpb + wave) * ((long long)S * a.dist);
+
+    // this lane's place inside a feature row
+    Gather<LPR, MODE, BUF> g;
+    g.ld_bytes = a.ld_bytes;
+    g.ld24 = a.ld_bytes & 0xFFFFFFu;
+    unsigned cofs;
+    if constexpr (MODE == MODE_F32_STRIDED) {
+        cofs = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int dd = l + i * LPR;
+            g.sofs[i] = 4u * (unsigned)(dd < a.dim ? dd : 0);
+        }
+    } else {
+        cofs = 16u * (unsigned)(NV * l < a.dim ? l : 0);
+    }
+    if constexpr (BUF) g.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(a.win_base), 0, a.win_bytes, 0x00020000);
+    g.zero = reinterpret_cast<const char *>(g_zero_row) + cofs;
+    const int pad_id = BUF ? a.sentinel : -1;  // what a slot holds past the end of its partition
 
     float acc[NV];
 #pragma unroll
@@ -237,20 +291,21 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
         const int len = (int)((unsigned)d.z & DESC_LEN_MASK);
         const bool remote = d.x < 0;
         const long long start = (long long)((unsigned)d.x & 0x7FFFFFFFu);
-        const void *tbl = remote ? a.in_r : a.in_l;
         const int *col = remote ? a.col_r : a.col_l;
         const int idbase = remote ? 0 : a.lb;
         const int nnz_side = remote ? a.nnz_r : a.nnz_l;
+        if constexpr (BUF) g.cbase = (remote ? a.delta_r : a.delta_l) + cofs;
+        else g.base = static_cast<const char *>(remote ? a.in_r : a.in_l) + cofs;
 
         for (int k0 = 0; k0 < a.ps; k0 += CH) {
             if (!__any(len > k0)) break;
-            // this lane's IPL neighbor ids of the chunk (-1 past the partition's end)
+            // this lane's IPL neighbor rows of the chunk, as row indices of the slot's table (pad_id past the end)
             int ids[IPL];
             {
                 const int kk = k0 + l * IPL;
                 const long long e0 = start + kk;
 #pragma unroll
-                for (int t = 0; t < IPL; ++t) ids[t] = -1;
+                for (int t = 0; t < IPL; ++t) ids[t] = pad_id;
                 if (kk < len) {
                     if constexpr (IPL == 4) {
                         if (e0 + 4 <= nnz_side) {
@@ -268,27 +323,24 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
                             if (kk + t < len) ids[t] = col[e0 + t];
                     }
 #pragma unroll
-                    for (int t = 0; t < IPL; ++t)
-                        if (kk + t >= len) ids[t] = -1;
+                    for (int t = 0; t < IPL; ++t) ids[t] = (kk + t < len) ? ids[t] - idbase : pad_id;
                 }
             }
             static_for<0, CH / BATCH>([&](auto bb) {
                 constexpr int b = decltype(bb)::value;
                 if (__any(len > k0 + b * BATCH)) {
                     float v[BATCH][NV];
-                    bool ok[BATCH];
                     static_for<0, BATCH>([&](auto tt) {
                         constexpr int t = decltype(tt)::value;
                         constexpr int k = b * BATCH + t;
-                        const int id = slot_bcast<LPR, k / IPL>(ids[k % IPL], slot_base);
-                        ok[t] = id >= 0;
-                        const long long r = ok[t] ? (long long)(id - idbase) : 0;
-                        gather_row<LPR, MODE>(v[t], tbl, r, a.ld_in, l, a.dim);
+                        g.load(v[t], slot_bcast<LPR, k / IPL>(ids[k % IPL], slot_base));
                     });
+                    // keep every load of the batch in flight before the first sum waits on one
+                    __builtin_amdgcn_sched_barrier(0);
                     static_for<0, BATCH>([&](auto tt) {
                         constexpr int t = decltype(tt)::value;
 #pragma unroll
-                        for (int i = 0; i < NV; ++i) acc[i] += ok[t] ? v[t][i] : 0.0f;
+                        for (int i = 0; i < NV; ++i) acc[i] += v[t][i];
                     });
                 }
             });
@@ -464,13 +516,13 @@ int pow2_ceil(int x)
     return p;
 }
 
-template <int MODE>
+template <int MODE, bool BUF>
 int launch_agg(int lpr, dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream, const AggArgs &a)
 {
     switch (lpr) {
 #define MGGX_CASE(L)                                                      \
     case L:                                                               \
-        k_agg<L, MODE><<<grid, block, lds_bytes, stream>>>(a);            \
+        k_agg<L, MODE, BUF><<<grid, block, lds_bytes, stream>>>(a);       \
         break;
         MGGX_CASE(1)
         MGGX_CASE(2)
@@ -546,6 +598,33 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     a.eps = o.eps;
     a.in_is_bf16 = o.in_dtype == MGGX_BF16;
 
+    // Gather addressing.  Extent of each table: the local one holds the share's rows, the remote one at least the
+    // largest remote id.  When both fit one window of < 2 GiB and < 2^24 rows, offsets are 32-bit buffer offsets.
+    const unsigned long long esize = a.in_is_bf16 ? 2 : 4;
+    const unsigned long long ld_bytes = (unsigned long long)ld_in * esize;
+    if (ld_bytes > 0xFFFFFFFFull) return fail(MGGX_ELIMIT, "aggregation: row stride of %llu bytes", ld_bytes);
+    a.ld_bytes = (unsigned)ld_bytes;
+    bool buf = false;
+    {
+        const unsigned long long pl = reinterpret_cast<uintptr_t>(a.in_l), pr = reinterpret_cast<uintptr_t>(a.in_r);
+        const unsigned long long el = pl + (unsigned long long)plan->rows * ld_bytes;
+        const bool has_r = plan->nnz_r > 0;
+        const unsigned long long er = has_r ? pr + ((unsigned long long)plan->max_col_r + 1) * ld_bytes : el;
+        const unsigned long long lo = has_r ? (pl < pr ? pl : pr) : pl;
+        const unsigned long long hi = el > er ? el : er;
+        const unsigned long long win = hi - lo;
+        const unsigned long long sentinel = (win + ld_bytes - 1) / ld_bytes;
+        if (win < 0x7FF00000ull && ld_bytes < (1ull << 24) && sentinel < (1ull << 24) - 1 && plan->rows < (1 << 24) &&
+            (!has_r || plan->max_col_r < (1 << 24) - 1) && st.gather_addressing == 0) {
+            buf = true;
+            a.win_base = reinterpret_cast<const void *>(static_cast<uintptr_t>(lo));
+            a.win_bytes = (unsigned)win;
+            a.delta_l = (unsigned)(pl - lo);
+            a.delta_r = has_r ? (unsigned)(pr - lo) : 0;
+            a.sentinel = (int)sentinel;
+        }
+    }
+
     if (num_wg > 0) {
         const size_t hdr_bytes = (size_t)num_wg * 2 * sizeof(int2);
         const size_t hdr_pad = (hdr_bytes + 255) & ~(size_t)255;
@@ -556,9 +635,15 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         a.c_val = reinterpret_cast<float *>(static_cast<char *>(ws) + hdr_pad);
         const size_t lds_bytes = (size_t)wpb * 2 * sizeof(int2) + (size_t)wpb * 2 * cpad * sizeof(float);
         const dim3 grid((unsigned)num_wg), block((unsigned)(64 * wpb));
-        if (mode == MODE_F32_VEC4) rc = launch_agg<MODE_F32_VEC4>(lpr, grid, block, lds_bytes, st.stream, a);
-        else if (mode == MODE_F32_STRIDED) rc = launch_agg<MODE_F32_STRIDED>(lpr, grid, block, lds_bytes, st.stream, a);
-        else rc = launch_agg<MODE_BF16_VEC8>(lpr, grid, block, lds_bytes, st.stream, a);
+        if (buf) {
+            if (mode == MODE_F32_VEC4) rc = launch_agg<MODE_F32_VEC4, true>(lpr, grid, block, lds_bytes, st.stream, a);
+            else if (mode == MODE_F32_STRIDED) rc = launch_agg<MODE_F32_STRIDED, true>(lpr, grid, block, lds_bytes, st.stream, a);
+            else rc = launch_agg<MODE_BF16_VEC8, true>(lpr, grid, block, lds_bytes, st.stream, a);
+        } else {
+            if (mode == MODE_F32_VEC4) rc = launch_agg<MODE_F32_VEC4, false>(lpr, grid, block, lds_bytes, st.stream, a);
+            else if (mode == MODE_F32_STRIDED) rc = launch_agg<MODE_F32_STRIDED, false>(lpr, grid, block, lds_bytes, st.stream, a);
+            else rc = launch_agg<MODE_BF16_VEC8, false>(lpr, grid, block, lds_bytes, st.stream, a);
+        }
         if (rc) return rc;
         MGGX_LAUNCH_CHECK("k_agg");
         if (num_wg > 1) {
@@ -573,7 +658,7 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         k_agg_empty_rows<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(a, plan->d_empty_rows, plan->num_empty);
         MGGX_LAUNCH_CHECK("k_agg_empty_rows");
     }
-    snprintf(st.last_kernel, sizeof(st.last_kernel), "k_agg<%d,%d> grid=%lld block=%d parts=%d", lpr, mode, num_wg, 64 * wpb,
+    snprintf(st.last_kernel, sizeof(st.last_kernel), "k_agg<%d,%d,%d> grid=%lld block=%d parts=%d", lpr, mode, (int)buf, num_wg, 64 * wpb,
              plan->num_parts);
     return MGGX_OK;
 }
@@ -596,7 +681,7 @@ MGGX_EXPORT int mggx_sag_np_div(float *d_out, const void *d_in_local, const void
     mggx_agg_opts o{};
     if (opts) o = *opts;
     mggx::Plan *plan = nullptr;
-    rc = mggx::plan_get(d_ptr_l, d_ptr_r, ub - lb, ps, &plan);
+    rc = mggx::plan_get(d_ptr_l, d_ptr_r, d_col_r, ub - lb, ps, &plan);
     if (rc) return rc;
     return mggx::run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, wpb, dist, o);
 }
@@ -624,7 +709,7 @@ MGGX_EXPORT int mggx_spmm(float *d_out, const float *d_in, const int *d_row_ptr,
     if (rc) return rc;
     if (!d_row_ptr || num_nodes < 0 || ps < 1) return fail(MGGX_EINVAL, "spmm: bad argument");
     mggx::Plan *plan = nullptr;
-    rc = mggx::plan_get(d_row_ptr, nullptr, num_nodes, ps, &plan);
+    rc = mggx::plan_get(d_row_ptr, nullptr, nullptr, num_nodes, ps, &plan);
     if (rc) return rc;
     mggx_agg_opts o{};
     o.flags = MGGX_AGG_ACCUMULATE;

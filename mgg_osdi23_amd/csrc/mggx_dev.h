@@ -52,6 +52,7 @@ struct Plan {
     int num_parts = 0;
     int num_empty = 0;
     int64_t nnz_l = 0, nnz_r = 0;
+    int max_col_r = -1;        // largest remote neighbor id (bounds the remote table)
 };
 
 struct State {
@@ -61,6 +62,7 @@ struct State {
     size_t ws_bytes = 0;
     std::vector<Plan *> plans;
     char last_kernel[160] = "";
+    int gather_addressing = 0;  // 0 = choose per call, 1 = always 64-bit addresses
 };
 
 State &state();
@@ -72,7 +74,7 @@ int workspace(size_t bytes, void **p);
 // total is also copied to *total_host when non-NULL (synchronises).
 int exclusive_scan_i32(const int *d_in, int *d_out, int n, long long *total_host);
 
-int plan_get(const int *d_ptr_l, const int *d_ptr_r, int rows, int ps, Plan **out);
+int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int rows, int ps, Plan **out);
 int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows,
                       int num_parts, int ps, Plan **out);
 void plan_free(Plan *p);

@@ -204,6 +204,21 @@ __global__ void __launch_bounds__(256) k_parts_ref_layout(const int *__restrict_
     part2node[p] = i;
 }
 
+// max over non-negative ints (atomicMax once per block; set-up time only)
+__global__ void __launch_bounds__(256) k_max_i32(const int *__restrict__ v, long long n, int *__restrict__ out)
+{
+    __shared__ int red[256];
+    int m = 0;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) m = max(m, v[i]);
+    red[threadIdx.x] = m;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if (threadIdx.x < o) red[threadIdx.x] = max(red[threadIdx.x], red[threadIdx.x + o]);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) atomicMax(out, red[0]);
+}
+
 __global__ void k_set_tail(int *node2part, int num_nodes)
 {
     node2part[num_nodes + 1] = node2part[num_nodes];
@@ -275,7 +290,7 @@ static void cache_insert(Plan *p)
     s.plans.push_back(p);
 }
 
-int plan_get(const int *d_ptr_l, const int *d_ptr_r, int rows, int ps, Plan **out)
+int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int rows, int ps, Plan **out)
 {
     State &s = state();
     for (Plan *p : s.plans)
@@ -311,6 +326,26 @@ int plan_get(const int *d_ptr_l, const int *d_ptr_r, int rows, int ps, Plan **ou
         }
         p->nnz_l = ends[0];
         p->nnz_r = ends[1];
+        if (p->nnz_r > 0) {
+            if (!d_col_r) {
+                rc = fail(MGGX_EINVAL, "plan: remote edges but no remote column array");
+                break;
+            }
+            int *d_max = nullptr;
+            if (hipMalloc((void **)&d_max, sizeof(int)) != hipSuccess) {
+                rc = fail(MGGX_ENOMEM, "plan: scratch");
+                break;
+            }
+            (void)hipMemsetAsync(d_max, 0, sizeof(int), s.stream);
+            k_max_i32<<<256, 256, 0, s.stream>>>(d_col_r, p->nnz_r, d_max);
+            hipError_t e = hipMemcpyAsync(&p->max_col_r, d_max, sizeof(int), hipMemcpyDeviceToHost, s.stream);
+            if (e == hipSuccess) e = hipStreamSynchronize(s.stream);
+            (void)hipFree(d_max);
+            if (e != hipSuccess) {
+                rc = fail(MGGX_EHIP, "plan: remote id scan: %s", hipGetErrorString(e));
+                break;
+            }
+        }
         if (hipMalloc((void **)&p->d_desc, sizeof(int4) * (size_t)std::max(p->num_parts, 1)) != hipSuccess) {
             rc = fail(MGGX_ENOMEM, "plan: %d descriptors", p->num_parts);
             break;

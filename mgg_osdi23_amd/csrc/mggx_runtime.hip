@@ -261,6 +261,13 @@ MGGX_EXPORT int mggx_cast_f32_to_bf16(void *d_dst, const float *d_src, int64_t n
     return MGGX_OK;
 }
 
+MGGX_EXPORT int mggx_set_gather_addressing(int mode)
+{
+    if (mode != 0 && mode != 1) return fail(MGGX_EINVAL, "set_gather_addressing: mode %d", mode);
+    state().gather_addressing = mode;
+    return MGGX_OK;
+}
+
 MGGX_EXPORT int mggx_last_agg_kernel(char *buf, size_t len)
 {
     if (!buf || !len) return fail(MGGX_EINVAL, "last_agg_kernel: NULL buffer");

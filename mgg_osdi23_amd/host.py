@@ -46,7 +46,7 @@ EXPORTS = [
     "mggx_release_cached", "mggx_range_partition", "mggx_split_csr", "mggx_build_part", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
     "mggx_fill_uniform", "mggx_build_part_device", "mggx_sag_np_div", "mggx_sag_parts", "mggx_spmm",
-    "mggx_dense_xw", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_last_agg_kernel",
+    "mggx_dense_xw", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
 ]
 
 
@@ -224,6 +224,10 @@ def device_name() -> str:
     buf = C.create_string_buffer(256)
     _check(lib().mggx_device_name(buf, 256))
     return buf.value.decode()
+
+
+def set_gather_addressing(mode: int) -> None:
+    _check(lib().mggx_set_gather_addressing(mode))
 
 
 def last_agg_kernel() -> str:

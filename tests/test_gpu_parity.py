@@ -12,6 +12,14 @@ from tests.util import BF16_TOL, FP32_TOL, assert_close_to_oracle, share_of, sym
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, params=["auto", "wide"])
+def addressing(request, gpu):
+    """Every case runs with both gather addressing schemes (32-bit buffer offsets where they apply, and 64-bit)."""
+    gpu.set_gather_addressing(1 if request.param == "wide" else 0)
+    yield request.param
+    gpu.set_gather_addressing(0)
+
+
 def run_agg(host, sh, x_local, x_remote, dim, ps, wpb, dist, *, gin=False, eps=0.0, accumulate_into=None,
             ld_in=0, ld_out=0, row_scale_out=None, relu=False):
     import torch
