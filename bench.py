@@ -269,7 +269,7 @@ def main():
     ap.add_argument("--workload", default="gcn2", choices=["gcn2", "share", "copy"])
     ap.add_argument("--ps", type=int, default=16)
     ap.add_argument("--wpb", type=int, default=8)
-    ap.add_argument("--dist", type=int, default=1)
+    ap.add_argument("--dist", type=int, default=0, help="0 = the workload's default (16 for gcn2, as the reference's bench_MGG.py; 1 for share)")
     ap.add_argument("--share-density", type=int, default=1, help="multiplies the number of RMAT draws of --workload share")
     ap.add_argument("--small", action="store_true", help="tiny graph, for a quick functional run")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -287,6 +287,8 @@ def main():
     host.init(0)
     host.use_torch_stream()
     log("device:", host.device_name())
+    if args.dist <= 0:
+        args.dist = 16 if args.workload == "gcn2" else 1
     res = {"gcn2": bench_gcn2, "share": bench_share, "copy": bench_copy}[args.workload](args, torch, host)
     print(json.dumps(res), flush=True)
 

@@ -31,7 +31,7 @@ HIP_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
     "-I", os.path.join(ROOT, "include"), "-I", CSRC,
-]
+] + os.environ.get("MGGX_HIPCC_EXTRA", "").split()
 HOST_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-fopenmp", "-Wall",
               "-I", os.path.join(ROOT, "include"), "-I", CSRC]
 

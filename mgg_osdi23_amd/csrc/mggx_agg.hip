@@ -25,6 +25,10 @@
 namespace mggx {
 namespace {
 
+#ifndef MGGX_BATCH
+#define MGGX_BATCH 8
+#endif
+
 constexpr int HDR_VALID = 1;   // entry holds a partial row
 constexpr int HDR_ENDS = 2;    // head entry: the row ends inside this unit
 constexpr int HDR_STARTS = 4;  // tail entry: the row started inside this unit
@@ -223,7 +227,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     constexpr int S = 64 / LPR;
     constexpr int CH = LPR > 16 ? LPR : 16;  // neighbor ids fetched per slot per chunk
     constexpr int IPL = CH / LPR;            // ids fetched per lane
-    constexpr int BATCH = 8;                 // gathers issued back to back
+    constexpr int BATCH = MGGX_BATCH;        // gathers issued back to back
     extern __shared__ float lds[];
 
     const int lane = lane_id();
