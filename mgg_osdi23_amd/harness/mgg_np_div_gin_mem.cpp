@@ -1,0 +1,102 @@
+// 5-layer GIN forward: the counterpart of the reference's src/mgg_np_div_gin_mem.cu
+// (the binary its bench_MGG_GIN.py runs).  Same command line and log lines.
+// Per iteration, in the reference's order (:195-222):
+//   dense(in->hidden); 5 x [ GIN aggregate (eps = 0.5) ; dense(hidden->hidden, last: hidden->out) ]; softmax
+// Differences, on purpose: every aggregation writes to its own buffer (layers 2-5 of the reference aggregate
+// from and into the same symmetric buffer, :203-218); with nGPU > 1 the other ranks' rows of every layer are
+// produced once, before the timed loop, by a whole-graph pass on this GPU and staged as the remote tables.
+#include "harness_common.h"
+
+int main(int argc, char *argv[])
+{
+    HarnessArgs a;
+    if (!parse_args(argc, argv, a)) return -1;
+    MGG_CHECK(mggx_init(0));
+    Share s;
+    load_share(a, s);
+    const nidType rows = s.ub - s.lb, npp = s.nodesPerPE;
+    const int dim = a.dim, hidden = a.hiddenSize, outdim = a.outdim;
+    const int layers = 5;
+    const float eps = 0.5f;  // src/mgg_np_div_gin.cu:58
+    const size_t padded = (size_t)a.num_GPUs * npp;
+    mgg_options().synchronize = true;
+
+    float *d_input = device_filled((size_t)npp * std::max(dim, outdim), 1.0f);
+    float *dsp_out = device_filled((size_t)npp * hidden, 0.0f);
+    float *den_out = device_filled((size_t)npp * std::max(hidden, outdim), 0.0f);
+    float *d_prob = device_filled((size_t)npp * outdim, 0.0f);
+
+    dense_param_new_beg *dp1 = new dense_param_new_beg("d-1", d_input, den_out, rows, dim, hidden);
+    dense_param_new_hidden *dpl[layers];
+    for (int l = 0; l < layers; ++l)
+        dpl[l] = new dense_param_new_hidden("d-n", dsp_out, den_out, rows, hidden, l == layers - 1 ? outdim : hidden);
+    softmax_new_param *smx = new softmax_new_param("smx-2", den_out, d_prob, rows, outdim);
+
+    // ---- staging pass (untimed): the dense outputs of all ranks for every layer ----
+    float *d_stage[layers] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+    if (a.num_GPUs > 1) {
+        nidType *d_gptr = to_device(s.global_row_ptr), *d_gcol = to_device(s.global_col_ind);
+        float *d_Xg = device_filled(padded * dim, 1.0f);
+        float *d_Hg = device_filled(padded * hidden, 0.0f);
+        mggx_agg_opts o{};
+        o.flags = MGGX_AGG_GIN;
+        o.eps = eps;
+        d_stage[0] = device_filled(padded * hidden, 0.0f);
+        MGG_CHECK(mggx_dense_xw(d_stage[0], d_Xg, dp1->d_W, s.numNodes, dim, hidden, nullptr));
+        for (int l = 0; l + 1 < layers; ++l) {
+            MGG_CHECK(mggx_sag_np_div(d_Hg, d_stage[l], d_stage[l], d_gptr, d_gcol, nullptr, nullptr, 0, s.numNodes, hidden,
+                                      (int)padded, a.partSize, a.warpPerBlock, a.interleaved_dist, &o));
+            d_stage[l + 1] = device_filled(padded * hidden, 0.0f);
+            MGG_CHECK(mggx_dense_xw(d_stage[l + 1], d_Hg, dpl[l]->d_W, s.numNodes, hidden, hidden, nullptr));
+        }
+        MGG_CHECK(mggx_sync());
+        MGG_CHECK(mggx_release_cached());
+        mggx_free(d_gptr); mggx_free(d_gcol); mggx_free(d_Xg); mggx_free(d_Hg);
+    }
+
+    auto forward = [&](bool with_softmax) {
+        dense_beg_new_forward(dp1);
+        for (int l = 0; l < layers; ++l) {
+            mgg_stage_remote(d_stage[l]);
+            mgg_GIN_np_div(dsp_out, den_out, s.d_row_ptr_l, s.d_col_ind_l, s.d_row_ptr_r, s.d_col_ind_r, s.lb, s.ub, hidden, npp,
+                           a.pe, a.partSize, a.warpPerBlock, a.interleaved_dist, eps);
+            dense_hidden_new_forward(dpl[l]);
+        }
+        if (with_softmax) softmax_new_forward(smx);
+    };
+
+    forward(!a.validate);
+    MGG_CHECK(mggx_sync());
+    if (a.validate) {
+        // all-ones closed form: y0 = dim; y_{l+1}[v] = hidden * ((1+eps) y_l[v] + sum_{u in N(v)} y_l[u]); logits = y_5
+        std::vector<double> y((size_t)s.numNodes, (double)dim), z((size_t)s.numNodes);
+        for (int l = 0; l < layers; ++l) {
+            for (nidType v = 0; v < s.numNodes; ++v) {
+                double acc = (1.0 + eps) * y[(size_t)v];
+                for (nidType e = s.global_row_ptr[v]; e < s.global_row_ptr[v + 1]; ++e) acc += y[(size_t)s.global_col_ind[e]];
+                z[(size_t)v] = acc * hidden;
+            }
+            y.swap(z);
+        }
+        std::vector<float> h((size_t)rows * outdim);
+        MGG_CHECK(mggx_memcpy_d2h(h.data(), den_out, h.size() * sizeof(float)));
+        double worst = 0.0;
+        for (nidType v = 0; v < rows; ++v)
+            for (int d = 0; d < outdim; ++d) {
+                const double ref = y[(size_t)s.lb + v];
+                worst = std::max(worst, std::abs((double)h[(size_t)v * outdim + d] - ref) / ref);
+            }
+        printf("Validation on PE-{%d}, status: %s (max relative error %.3g)\n", a.pe, worst < 1e-5 ? "True" : "False", worst);
+    }
+
+    std::clock_t c_start = std::clock();
+    const double t1 = now_ms();
+    for (int i = 0; i < a.iters; i++) forward(true);
+    MGG_CHECK(mggx_sync());
+    const double t2 = now_ms();
+    std::clock_t c_end = std::clock();
+    printf("PE-%d, Total (ms): %.3f\n", a.pe, 1000.0 * (c_end - c_start) / CLOCKS_PER_SEC / a.iters);
+    printf("MPI time (ms) %.3f\n", (t2 - t1) / a.iters);
+    printf("===================================\n");
+    return 0;
+}
