@@ -200,6 +200,12 @@ typedef struct mggx_dense_opts {
 int mggx_dense_xw(float *d_out, const float *d_x, const float *d_w, int64_t n, int d1, int d2,
                   const mggx_dense_opts *opts);
 
+/* The same update on the bf16 matrix cores (no counterpart in the reference, which is fp32 only): W is bf16
+ * [d1 x d2]; X is fp32 (rounded to bf16, nearest even, inside the kernel) or bf16 (x_dtype); products are
+ * accumulated in fp32; Out is fp32 or bf16 (out_dtype).  Strides are in elements of the respective type. */
+int mggx_dense_xw_bf16(void *d_out, const void *d_x, const void *d_w_bf16, int64_t n, int d1, int d2,
+                       int x_dtype, int out_dtype, const mggx_dense_opts *opts);
+
 /* softmax_forward / softmax_new_forward (include/gnn_layer.cuh:15-20,36-40):
  * cudnnSoftmaxForward(ACCURATE, MODE_CHANNEL) on (n, c, 1, 1) == stable row
  * softmax.  In place (d_out == d_in) is allowed. */

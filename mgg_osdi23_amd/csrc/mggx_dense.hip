@@ -1,18 +1,22 @@
-// Dense node update Out = X . W on the fp32 matrix cores, and the row softmax.
+// Dense node update Out = X . W on the matrix cores (fp32 and bf16 MFMA), and the row softmax.
 #include "mggx_dev.h"
 
 namespace mggx {
 namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 
-constexpr int GEMM_KC = 64;       // K extent of the W tile staged in LDS
+constexpr int GEMM_KC = 64;       // K extent of the W tile staged in LDS by the chunked kernel
 constexpr int GEMM_ROWS_WG = 64;  // 4 wavefronts x 16 rows
+constexpr size_t LDS_RESIDENT_LIMIT = 72 * 1024;  // keep W resident in LDS up to this size (two workgroups per CU)
 
 struct DenseArgs {
-    float *out;
-    const float *x;
-    const float *w;
+    void *out;
+    const void *x;
+    const void *w;
     const float *rs;
     long long n;
     long long ld_x, ld_out;
@@ -24,61 +28,27 @@ struct DenseArgs {
 //   A (16 x 4): lane L holds A[L % 16][L / 16]
 //   B (4 x 16): lane L holds B[L / 16][L % 16]
 //   D (16 x 16): lane L holds D[4 * (L / 16) + r][L % 16], r = 0..3
-// Each lane loads 4 consecutive K values of one X row; MFMA step t then
-// multiplies the K indices {4*(L/16) + t}, and B is read from LDS with the same
-// index, so the sum over K is complete after 4 steps per 16 K values.
-template <int NB>
-__global__ void __launch_bounds__(256) k_dense_xw(const DenseArgs a)
+// Each lane loads 4 consecutive K values of one X row; MFMA step t then multiplies the K indices {4*(L/16) + t},
+// and B is read from LDS with the same index, so the sum over K is complete after 4 steps per 16 K values.
+__device__ __forceinline__ void load_x4(float (&xv)[4], const float *xrow, int kb, int d1, bool row_ok)
 {
-    constexpr int RS = NB * 16 + 4;  // LDS row stride in floats; the +4 keeps the four K groups on distinct banks
-    __shared__ float wt[GEMM_KC * RS];
-    const int lane = (int)(threadIdx.x & 63u);
-    const int wave = (int)(threadIdx.x >> 6);
-    const int i = lane & 15, kq = lane >> 4;
-    const long long row = (long long)blockIdx.x * GEMM_ROWS_WG + wave * 16 + i;
-    const int c0 = (int)blockIdx.y * (NB * 16);
-    const bool row_ok = row < a.n;
-    const float *xrow = a.x + (row_ok ? row : 0) * a.ld_x;
-
-    v4f acc[NB];
+    xv[0] = xv[1] = xv[2] = xv[3] = 0.f;
+    if (!row_ok) return;
+    if (kb + 3 < d1) {
+        float4 t4;
+        __builtin_memcpy(&t4, xrow + kb, 16);
+        xv[0] = t4.x; xv[1] = t4.y; xv[2] = t4.z; xv[3] = t4.w;
+    } else {
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) acc[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
-
-    for (int k0 = 0; k0 < a.d1; k0 += GEMM_KC) {
-        __syncthreads();
-        for (int idx = (int)threadIdx.x; idx < GEMM_KC * NB * 16; idx += 256) {
-            const int k = idx / (NB * 16), j = idx % (NB * 16);
-            float v = 0.f;
-            if (k0 + k < a.d1 && c0 + j < a.d2) v = a.w[(long long)(k0 + k) * a.d2 + c0 + j];
-            wt[k * RS + j] = v;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int ks = 0; ks < GEMM_KC / 16; ++ks) {
-            const int kb = k0 + ks * 16 + 4 * kq;
-            float xv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (row_ok) {
-                if (kb + 3 < a.d1) {
-                    float4 t4;
-                    __builtin_memcpy(&t4, xrow + kb, 16);
-                    xv[0] = t4.x; xv[1] = t4.y; xv[2] = t4.z; xv[3] = t4.w;
-                } else {
-#pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        if (kb + t < a.d1) xv[t] = xrow[kb + t];
-                }
-            }
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const float *wrow = wt + (ks * 16 + 4 * kq + t) * RS + i;
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
-                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[t], wrow[nb * 16], acc[nb], 0, 0, 0);
-            }
-        }
+        for (int t = 0; t < 4; ++t)
+            if (kb + t < d1) xv[t] = xrow[kb + t];
     }
+}
 
-    const long long row_base = (long long)blockIdx.x * GEMM_ROWS_WG + wave * 16 + 4 * kq;
+template <int NB>
+__device__ __forceinline__ void store_tile_f32(const DenseArgs &a, const v4f (&acc)[NB], long long row_base, int c0, int i)
+{
+    float *out = static_cast<float *>(a.out);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const long long orow = row_base + r;
@@ -90,7 +60,214 @@ __global__ void __launch_bounds__(256) k_dense_xw(const DenseArgs a)
             if (c < a.d2) {
                 float v = acc[nb][r] * scale;
                 if (a.relu) v = fmaxf(v, 0.f);
-                a.out[orow * a.ld_out + c] = v;
+                out[orow * a.ld_out + c] = v;
+            }
+        }
+    }
+}
+
+// W kept whole in LDS (zero padded to a multiple of 64 rows); the 8 wavefronts of a workgroup walk over 16-row
+// tiles of X.  X is read four 16-wide K steps at a time, one group ahead of the matrix cores.
+constexpr int RES_THREADS = 512;
+template <int NB>
+__global__ void __launch_bounds__(RES_THREADS) k_dense_xw_resident(const DenseArgs a)
+{
+    constexpr int RS = NB * 16 + 4;  // LDS row stride in floats; the +4 keeps the four K groups on distinct banks
+    constexpr int WAVES = RES_THREADS / 64;
+    extern __shared__ float wt[];
+    const int lane = (int)(threadIdx.x & 63u);
+    const int wave = (int)(threadIdx.x >> 6);
+    const int i = lane & 15, kq = lane >> 4;
+    const int c0 = (int)blockIdx.y * (NB * 16);
+    const int d1p = (a.d1 + 63) & ~63;
+    const float *w = static_cast<const float *>(a.w);
+    for (int idx = (int)threadIdx.x; idx < d1p * NB * 16; idx += RES_THREADS) {
+        const int k = idx / (NB * 16), j = idx % (NB * 16);
+        wt[k * RS + j] = (k < a.d1 && c0 + j < a.d2) ? w[(long long)k * a.d2 + c0 + j] : 0.f;
+    }
+    __syncthreads();
+
+    const long long tiles = (a.n + 15) / 16;
+    for (long long tile = (long long)blockIdx.x * WAVES + wave; tile < tiles; tile += (long long)gridDim.x * WAVES) {
+        const long long row = tile * 16 + i;
+        const bool row_ok = row < a.n;
+        const float *xrow = static_cast<const float *>(a.x) + (row_ok ? row : 0) * a.ld_x;
+        v4f acc[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
+        float xv[4][4], xn[4][4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) load_x4(xv[g], xrow, 16 * g + 4 * kq, a.d1, row_ok);
+        for (int k0 = 0; k0 < d1p; k0 += 64) {
+            if (k0 + 64 < d1p) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) load_x4(xn[g], xrow, k0 + 64 + 16 * g + 4 * kq, a.d1, row_ok);
+            }
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const float *wrow = wt + (k0 + 16 * g + 4 * kq + t) * RS + i;
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb)
+                        acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[g][t], wrow[nb * 16], acc[nb], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) xv[g][t] = xn[g][t];
+        }
+        store_tile_f32<NB>(a, acc, tile * 16 + 4 * kq, c0, i);
+    }
+}
+
+// W staged in K chunks (any d1): fallback when W does not fit in LDS.
+template <int NB>
+__global__ void __launch_bounds__(256) k_dense_xw(const DenseArgs a)
+{
+    constexpr int RS = NB * 16 + 4;
+    __shared__ float wt[GEMM_KC * RS];
+    const int lane = (int)(threadIdx.x & 63u);
+    const int wave = (int)(threadIdx.x >> 6);
+    const int i = lane & 15, kq = lane >> 4;
+    const long long row = (long long)blockIdx.x * GEMM_ROWS_WG + wave * 16 + i;
+    const int c0 = (int)blockIdx.y * (NB * 16);
+    const bool row_ok = row < a.n;
+    const float *xrow = static_cast<const float *>(a.x) + (row_ok ? row : 0) * a.ld_x;
+    const float *w = static_cast<const float *>(a.w);
+
+    v4f acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    for (int k0 = 0; k0 < a.d1; k0 += GEMM_KC) {
+        __syncthreads();
+        for (int idx = (int)threadIdx.x; idx < GEMM_KC * NB * 16; idx += 256) {
+            const int k = idx / (NB * 16), j = idx % (NB * 16);
+            float v = 0.f;
+            if (k0 + k < a.d1 && c0 + j < a.d2) v = w[(long long)(k0 + k) * a.d2 + c0 + j];
+            wt[k * RS + j] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < GEMM_KC / 16; ++ks) {
+            float xv[4];
+            load_x4(xv, xrow, k0 + ks * 16 + 4 * kq, a.d1, row_ok);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const float *wrow = wt + (ks * 16 + 4 * kq + t) * RS + i;
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[t], wrow[nb * 16], acc[nb], 0, 0, 0);
+            }
+        }
+    }
+    store_tile_f32<NB>(a, acc, (long long)blockIdx.x * GEMM_ROWS_WG + wave * 16 + 4 * kq, c0, i);
+}
+
+// bf16 matrix cores: v_mfma_f32_16x16x32_bf16 (wave64)
+//   A (16 x 32): lane L holds A[L % 16][8 * (L / 16) .. + 8)
+//   B (32 x 16): lane L holds B[8 * (L / 16) .. + 8)[L % 16]
+//   D (16 x 16): lane L holds D[4 * (L / 16) + r][L % 16], r = 0..3
+// W (bf16, [d1][d2]) is kept transposed in LDS, Wt[column][k], so a lane's 8 K values are one 16-byte read.
+// X is fp32 (rounded to bf16, nearest even, on the fly) or bf16; the accumulator and the epilogue are fp32; the
+// output is fp32 or bf16.
+template <int NB, bool X_F32, bool OUT_BF16>
+__global__ void __launch_bounds__(256) k_dense_xw_bf16(const DenseArgs a)
+{
+    extern __shared__ float lds_raw[];
+    __bf16 *wt = reinterpret_cast<__bf16 *>(lds_raw);
+    const int lane = (int)(threadIdx.x & 63u);
+    const int wave = (int)(threadIdx.x >> 6);
+    const int i = lane & 15, kb = lane >> 4;
+    const int c0 = (int)blockIdx.y * (NB * 16);
+    const int d1p = (a.d1 + 31) & ~31;
+    const int KP = d1p + 8;  // row stride of Wt in bf16: the +8 (16 bytes) staggers rows over the banks
+    const unsigned short *w = static_cast<const unsigned short *>(a.w);
+    unsigned short *wts = reinterpret_cast<unsigned short *>(wt);
+    for (int idx = (int)threadIdx.x; idx < d1p * NB * 16; idx += 256) {
+        const int k = idx / (NB * 16), j = idx % (NB * 16);
+        wts[j * KP + k] = (k < a.d1 && c0 + j < a.d2) ? w[(long long)k * a.d2 + c0 + j] : (unsigned short)0;
+    }
+    __syncthreads();
+
+    const long long tiles = (a.n + 15) / 16;
+    for (long long tile = (long long)blockIdx.x * 4 + wave; tile < tiles; tile += (long long)gridDim.x * 4) {
+        const long long row = tile * 16 + i;
+        const bool row_ok = row < a.n;
+        v4f acc[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
+        for (int k0 = 0; k0 < d1p; k0 += 32) {
+            const int k = k0 + 8 * kb;
+            v8bf av;
+            if constexpr (X_F32) {
+                const float *xrow = static_cast<const float *>(a.x) + (row_ok ? row : 0) * a.ld_x;
+                float f[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) f[t] = 0.f;
+                if (row_ok) {
+                    if (k + 7 < a.d1) {
+                        float4 t0, t1;
+                        __builtin_memcpy(&t0, xrow + k, 16);
+                        __builtin_memcpy(&t1, xrow + k + 4, 16);
+                        f[0] = t0.x; f[1] = t0.y; f[2] = t0.z; f[3] = t0.w;
+                        f[4] = t1.x; f[5] = t1.y; f[6] = t1.z; f[7] = t1.w;
+                    } else {
+#pragma unroll
+                        for (int t = 0; t < 8; ++t)
+                            if (k + t < a.d1) f[t] = xrow[k + t];
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const v2bf p = __builtin_convertvector((v2f){f[2 * t], f[2 * t + 1]}, v2bf);
+                    av[2 * t] = p[0];
+                    av[2 * t + 1] = p[1];
+                }
+            } else {
+                const unsigned short *xrow = static_cast<const unsigned short *>(a.x) + (row_ok ? row : 0) * a.ld_x;
+                unsigned short h[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) h[t] = 0;
+                if (row_ok) {
+                    if (k + 7 < a.d1) {
+                        __builtin_memcpy(h, xrow + k, 16);
+                    } else {
+#pragma unroll
+                        for (int t = 0; t < 8; ++t)
+                            if (k + t < a.d1) h[t] = xrow[k + t];
+                    }
+                }
+                __builtin_memcpy(&av, h, 16);
+            }
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                v8bf bv;
+                __builtin_memcpy(&bv, wt + (size_t)(nb * 16 + i) * KP + k, 16);
+                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, acc[nb], 0, 0, 0);
+            }
+        }
+        const long long row_base = tile * 16 + 4 * kb;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const long long orow = row_base + r;
+            if (orow >= a.n) continue;
+            const float scale = a.rs ? a.rs[orow] : 1.0f;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const int c = c0 + nb * 16 + i;
+                if (c < a.d2) {
+                    float v = acc[nb][r] * scale;
+                    if (a.relu) v = fmaxf(v, 0.f);
+                    if constexpr (OUT_BF16) {
+                        const v2bf p = __builtin_convertvector((v2f){v, 0.f}, v2bf);
+                        static_cast<__bf16 *>(a.out)[orow * a.ld_out + c] = p[0];
+                    } else {
+                        static_cast<float *>(a.out)[orow * a.ld_out + c] = v;
+                    }
+                }
             }
         }
     }
@@ -118,6 +295,68 @@ __global__ void __launch_bounds__(256) k_softmax_rows(float *__restrict__ out, c
         float *o_ = out + row * ld_out;
         for (int j = l; j < c; j += G) o_[j] = __expf(x[j] - m) * inv;
     }
+}
+
+// columns are covered in chunks of NB*16; pick the widest chunk that wastes no block
+int pick_nb(int d2)
+{
+    const int blocks16 = (d2 + 15) / 16;
+    int nb = blocks16 >= 8 ? 8 : blocks16;
+    if (nb == 5) nb = 6;
+    if (nb == 7) nb = 8;
+    return nb;
+}
+
+template <template <int> class Launcher>
+int dispatch_nb(int nb, dim3 grid, size_t lds, hipStream_t stream, const DenseArgs &a)
+{
+    switch (nb) {
+        case 1: Launcher<1>::run(grid, lds, stream, a); break;
+        case 2: Launcher<2>::run(grid, lds, stream, a); break;
+        case 3: Launcher<3>::run(grid, lds, stream, a); break;
+        case 4: Launcher<4>::run(grid, lds, stream, a); break;
+        case 6: Launcher<6>::run(grid, lds, stream, a); break;
+        default: Launcher<8>::run(grid, lds, stream, a); break;
+    }
+    return MGGX_OK;
+}
+
+template <typename K>
+void allow_lds(K kernel, size_t lds)
+{
+    if (lds > 48 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+}
+
+template <int NB>
+struct LaunchResident {
+    static void run(dim3 grid, size_t lds, hipStream_t s, const DenseArgs &a)
+    {
+        allow_lds(k_dense_xw_resident<NB>, lds);
+        k_dense_xw_resident<NB><<<grid, dim3(RES_THREADS), lds, s>>>(a);
+    }
+};
+template <int NB>
+struct LaunchChunked {
+    static void run(dim3 grid, size_t, hipStream_t s, const DenseArgs &a) { k_dense_xw<NB><<<grid, dim3(256), 0, s>>>(a); }
+};
+template <bool X_F32, bool OUT_BF16>
+struct LaunchBf16 {
+    template <int NB>
+    struct L {
+        static void run(dim3 grid, size_t lds, hipStream_t s, const DenseArgs &a)
+        {
+            allow_lds(k_dense_xw_bf16<NB, X_F32, OUT_BF16>, lds);
+            k_dense_xw_bf16<NB, X_F32, OUT_BF16><<<grid, dim3(256), lds, s>>>(a);
+        }
+    };
+};
+
+// persistent grid: enough workgroups to fill the device a few times over, never more than there are 64-row groups
+unsigned persistent_blocks(long long n)
+{
+    const long long groups = (n + 127) / 128;
+    const long long want = 256 * 4;
+    return (unsigned)(groups < want ? (groups > 0 ? groups : 1) : want);
 }
 
 }  // namespace
@@ -148,25 +387,59 @@ MGGX_EXPORT int mggx_dense_xw(float *d_out, const float *d_x, const float *d_w, 
     a.d2 = d2;
     a.relu = o.relu != 0;
     if (a.ld_x < d1 || a.ld_out < d2) return fail(MGGX_EINVAL, "dense_xw: row stride smaller than width");
-    const long long gx = (n + mggx::GEMM_ROWS_WG - 1) / mggx::GEMM_ROWS_WG;
-    if (gx > 0x7fffffffLL) return fail(MGGX_ELIMIT, "dense_xw: too many rows");
     hipStream_t stream = mggx::state().stream;
-    const int blocks16 = (d2 + 15) / 16;
-    // columns are covered in chunks of NB*16; pick the widest chunk that wastes no block
-    int nb = blocks16 >= 8 ? 8 : blocks16;
-    if (nb == 5) nb = 6;
-    if (nb == 7) nb = 8;
-    const int gy = (blocks16 + nb - 1) / nb;
-    const dim3 grid((unsigned)gx, (unsigned)gy), block(256);
-    switch (nb) {
-        case 1: mggx::k_dense_xw<1><<<grid, block, 0, stream>>>(a); break;
-        case 2: mggx::k_dense_xw<2><<<grid, block, 0, stream>>>(a); break;
-        case 3: mggx::k_dense_xw<3><<<grid, block, 0, stream>>>(a); break;
-        case 4: mggx::k_dense_xw<4><<<grid, block, 0, stream>>>(a); break;
-        case 6: mggx::k_dense_xw<6><<<grid, block, 0, stream>>>(a); break;
-        default: mggx::k_dense_xw<8><<<grid, block, 0, stream>>>(a); break;
+    const int nb = mggx::pick_nb(d2);
+    const int gy = ((d2 + 15) / 16 + nb - 1) / nb;
+    const size_t lds = (size_t)((d1 + 63) & ~63) * (nb * 16 + 4) * sizeof(float);
+    if (lds <= mggx::LDS_RESIDENT_LIMIT) {
+        const dim3 grid(mggx::persistent_blocks(n), (unsigned)gy);
+        mggx::dispatch_nb<mggx::LaunchResident>(nb, grid, lds, stream, a);
+        MGGX_LAUNCH_CHECK("k_dense_xw_resident");
+    } else {
+        const long long gx = (n + mggx::GEMM_ROWS_WG - 1) / mggx::GEMM_ROWS_WG;
+        if (gx > 0x7fffffffLL) return fail(MGGX_ELIMIT, "dense_xw: too many rows");
+        mggx::dispatch_nb<mggx::LaunchChunked>(nb, dim3((unsigned)gx, (unsigned)gy), 0, stream, a);
+        MGGX_LAUNCH_CHECK("k_dense_xw");
     }
-    MGGX_LAUNCH_CHECK("k_dense_xw");
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_dense_xw_bf16(void *d_out, const void *d_x, const void *d_w_bf16, int64_t n, int d1, int d2,
+                                   int x_dtype, int out_dtype, const mggx_dense_opts *opts)
+{
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    if (n < 0 || d1 < 1 || d2 < 1) return fail(MGGX_EINVAL, "dense_xw_bf16: n=%lld d1=%d d2=%d", (long long)n, d1, d2);
+    if ((x_dtype != MGGX_F32 && x_dtype != MGGX_BF16) || (out_dtype != MGGX_F32 && out_dtype != MGGX_BF16))
+        return fail(MGGX_EINVAL, "dense_xw_bf16: unknown dtype");
+    if (n == 0) return MGGX_OK;
+    if (!d_out || !d_x || !d_w_bf16) return fail(MGGX_EINVAL, "dense_xw_bf16: NULL pointer");
+    if (d_out == d_x) return fail(MGGX_EINVAL, "dense_xw_bf16: in-place update is not supported");
+    mggx_dense_opts o{};
+    if (opts) o = *opts;
+    mggx::DenseArgs a{};
+    a.out = d_out;
+    a.x = d_x;
+    a.w = d_w_bf16;
+    a.rs = o.d_row_scale;
+    a.n = n;
+    a.ld_x = o.ld_x ? o.ld_x : d1;
+    a.ld_out = o.ld_out ? o.ld_out : d2;
+    a.d1 = d1;
+    a.d2 = d2;
+    a.relu = o.relu != 0;
+    if (a.ld_x < d1 || a.ld_out < d2) return fail(MGGX_EINVAL, "dense_xw_bf16: row stride smaller than width");
+    const int nb = mggx::pick_nb(d2);
+    const int gy = ((d2 + 15) / 16 + nb - 1) / nb;
+    const size_t lds = (size_t)(nb * 16) * (((d1 + 31) & ~31) + 8) * 2;
+    if (lds > 150 * 1024) return fail(MGGX_ELIMIT, "dense_xw_bf16: W tile of %zu bytes does not fit in LDS (d1 <= ~580 at 128 columns)", lds);
+    hipStream_t stream = mggx::state().stream;
+    const dim3 grid(mggx::persistent_blocks(n), (unsigned)gy);
+    if (x_dtype == MGGX_F32 && out_dtype == MGGX_F32) mggx::dispatch_nb<mggx::LaunchBf16<true, false>::L>(nb, grid, lds, stream, a);
+    else if (x_dtype == MGGX_F32) mggx::dispatch_nb<mggx::LaunchBf16<true, true>::L>(nb, grid, lds, stream, a);
+    else if (out_dtype == MGGX_F32) mggx::dispatch_nb<mggx::LaunchBf16<false, false>::L>(nb, grid, lds, stream, a);
+    else mggx::dispatch_nb<mggx::LaunchBf16<false, true>::L>(nb, grid, lds, stream, a);
+    MGGX_LAUNCH_CHECK("k_dense_xw_bf16");
     return MGGX_OK;
 }
 

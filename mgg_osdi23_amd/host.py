@@ -46,7 +46,7 @@ EXPORTS = [
     "mggx_release_cached", "mggx_range_partition", "mggx_split_csr", "mggx_build_part", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
     "mggx_fill_uniform", "mggx_build_part_device", "mggx_sag_np_div", "mggx_sag_parts", "mggx_spmm",
-    "mggx_dense_xw", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
+    "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
 ]
 
 
@@ -305,6 +305,24 @@ def dense_forward(out, x, w, n, d1, d2, ld_x=0, ld_out=0, row_scale=None, relu=F
     o.d_row_scale = row_scale.data_ptr() if row_scale is not None else None
     o.relu = int(relu)
     _check(lib().mggx_dense_xw(_dptr(out), _dptr(x), _dptr(w), C.c_int64(n), d1, d2, C.byref(o)))
+
+
+def dense_forward_bf16(out, x, w_bf16, n, d1, d2, ld_x=0, ld_out=0, row_scale=None, relu=False):
+    """Out = X . W on the bf16 matrix cores; X fp32 or bf16, W bf16, Out fp32 or bf16 (taken from the tensors)."""
+    import torch
+    o = _DenseOpts()
+    o.ld_x = ld_x
+    o.ld_out = ld_out
+    o.d_row_scale = row_scale.data_ptr() if row_scale is not None else None
+    o.relu = int(relu)
+    assert w_bf16.dtype == torch.bfloat16
+    xd = BF16 if x.dtype == torch.bfloat16 else F32
+    od = BF16 if out.dtype == torch.bfloat16 else F32
+    _check(lib().mggx_dense_xw_bf16(_dptr(out), _dptr(x), _dptr(w_bf16), C.c_int64(n), d1, d2, xd, od, C.byref(o)))
+
+
+def cast_f32_to_bf16(dst, src, n) -> None:
+    _check(lib().mggx_cast_f32_to_bf16(_dptr(dst), _dptr(src), C.c_int64(n)))
 
 
 def softmax_forward(out, x, n, c, ld_in=0, ld_out=0):

@@ -353,3 +353,34 @@ def test_bf16_tables(gpu, rmat_graph, dim):
     assert_close_to_oracle(got, want, mag, FP32_TOL, "bf16 in, fp32 accumulate (vs the same rounded inputs)")
     want_f, mag_f = oracle_agg(sh, x[sh["lb"]:sh["ub"]], x, dim)
     assert_close_to_oracle(got, want_f, mag_f, BF16_TOL, "bf16 in vs unrounded inputs")
+
+
+# --------------------------------------------------------------------------- dense update on the bf16 matrix cores
+@pytest.mark.parametrize("n,d1,d2", [(1000, 128, 128), (333, 64, 47), (257, 100, 64), (64, 602, 16), (17, 7, 3), (500, 256, 200)])
+@pytest.mark.parametrize("x_bf16,out_bf16", [(False, False), (True, False), (False, True), (True, True)])
+def test_dense_update_bf16(gpu, n, d1, d2, x_bf16, out_bf16, addressing):
+    import torch
+    if addressing == "wide":
+        pytest.skip("addressing switch does not concern the dense kernels")
+    x = gpu.fill_normal((n, d1), seed=50)
+    w = gpu.glorot(d1, d2, seed=51)
+    wb = to_dev(w).to(torch.bfloat16)
+    xd = to_dev(x)
+    xr = xd.to(torch.bfloat16)          # what the kernel's own round-to-nearest-even must reproduce
+    x_in = xr if x_bf16 else xd
+    out = torch.full((n, d2), 3.0, device="cuda", dtype=torch.bfloat16 if out_bf16 else torch.float32)
+    gpu.dense_forward_bf16(out, x_in, wb, n, d1, d2)
+    gpu.sync()
+    xf = xr.to(torch.float32).cpu().numpy()
+    wf = wb.to(torch.float32).cpu().numpy()
+    want = orc.dense(xf, wf, f64=True)
+    mag = np.abs(xf).astype(np.float64) @ np.abs(wf).astype(np.float64)
+    got = out.to(torch.float32).cpu().numpy()
+    if out_bf16:
+        assert_close_to_oracle(got, want, mag + np.abs(want) * 400, FP32_TOL, "bf16 out: fp32 result rounded to bf16")
+    else:
+        assert_close_to_oracle(got, want, mag, FP32_TOL, "bf16 MFMA vs the same rounded inputs")
+    # against the unrounded inputs: the bf16 tolerance
+    want_f = orc.dense(x, w, f64=True)
+    mag_f = np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64)
+    assert_close_to_oracle(got, want_f, mag_f, BF16_TOL, "bf16 MFMA vs unrounded inputs")
