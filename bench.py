@@ -279,6 +279,189 @@ def bench_share(args, torch, host):
     }
 
 
+def bench_gin(args, torch, host):
+    """configs[2]: 5-layer GIN forward on the whole graph: dense(100->64); 5 x [GIN aggregate (1+eps) x_v + sum, eps = 0,
+    then a 2-layer MLP 64->64->64 with ReLU between, the last MLP ending at 47 classes]; softmax.  (The reference's main
+    has one dense per GIN layer and eps = 0.5; the benchmark configuration asks for the 2-layer MLP and eps = 0.)"""
+    V, scale, draws = 2_450_000, 22, 64_000_000
+    in_dim, hidden, out_dim, L, eps = 100, 64, 47, 5, 0.0
+    ps, wpb, dist = args.ps, args.wpb, args.dist
+    if args.small:
+        V, scale, draws = 50_000, 16, 1_300_000
+    t0 = time.time()
+    ptr, col = host.gen_rmat(scale, V, draws, seed=3)
+    nnz = int(len(col))
+    log("graph: V=%d nnz=%d in %.1fs" % (V, nnz, time.time() - t0))
+    X = host.fill_normal((V, in_dim), seed=1)
+    W0 = host.glorot(in_dim, hidden, seed=2)
+    Wa = [host.glorot(hidden, hidden, seed=10 + l) * 0.2 for l in range(L)]
+    Wb = [host.glorot(hidden, out_dim if l == L - 1 else hidden, seed=30 + l) * 0.2 for l in range(L)]
+    dev = "cuda"
+    d_ptr, d_col = torch.from_numpy(ptr).to(dev), torch.from_numpy(col).to(dev)
+    zp, zc = torch.zeros(V + 1, dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int32, device=dev)
+    d_X, d_W0 = torch.from_numpy(X).to(dev), torch.from_numpy(W0).to(dev)
+    d_Wa = [torch.from_numpy(w).to(dev) for w in Wa]
+    ldo = (out_dim + 3) & ~3
+    d_Wb = [torch.from_numpy(w).to(dev) for w in Wb]
+    d_Y = torch.empty(V, hidden, device=dev)
+    d_H = torch.empty(V, hidden, device=dev)
+    d_T = torch.empty(V, hidden, device=dev)
+    d_logits = torch.empty(V, out_dim, device=dev)
+    d_P = torch.empty(V, out_dim, device=dev)
+
+    stages, names = [lambda: host.dense_forward(d_Y, d_X, d_W0, V, in_dim, hidden)], ["dense0"]
+    for l in range(L):
+        last = l == L - 1
+        stages.append(lambda: host.mgg_GIN_np_div(d_H, d_Y, d_ptr, d_col, zp, zc, 0, V, hidden, V, 0, ps, wpb, dist, eps))
+        stages.append(lambda l=l: host.dense_forward(d_T, d_H, d_Wa[l], V, hidden, hidden, relu=True))
+        if last:
+            stages.append(lambda l=l: host.dense_forward(d_logits, d_T, d_Wb[l], V, hidden, out_dim))
+        else:
+            stages.append(lambda l=l: host.dense_forward(d_Y, d_T, d_Wb[l], V, hidden, hidden))
+        names += ["agg%d" % l, "mlp%da" % l, "mlp%db" % l]
+    stages.append(lambda: host.softmax_forward(d_P, d_logits, V, out_dim))
+    names.append("softmax")
+
+    for _ in range(args.warmup):
+        for fn in stages:
+            fn()
+    torch.cuda.synchronize()
+    timer = StageTimer(torch, names)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        timer.step(stages)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    avg = timer.averages()
+    agg_ms = sum(avg["agg%d" % l] for l in range(L)) / L
+    mlp_ms = sum(avg["mlp%da" % l] + avg["mlp%db" % l] for l in range(L))
+    log("ms: agg avg %.4f, all MLPs %.4f, dense0 %.4f, softmax %.4f, wall %.4f" % (agg_ms, mlp_ms, avg["dense0"], avg["softmax"], wall_ms))
+    nbytes = agg_bytes(nnz, V, hidden, gin=True)
+    achieved = nbytes / (agg_ms * 1e-3) / 1e9
+
+    cpu = None
+    parity = None
+    if not args.no_cpu:
+        from oracle import orc
+        th = orc.max_threads()
+        t0 = time.perf_counter()
+        Y = orc.dense(X, W0, f64=False, threads=th)
+        for l in range(L):
+            H = orc.sag_np_div(Y, Y, ptr, col, None, None, 0, V, hidden, V, flags=orc.GIN, eps=eps, f64=False, threads=th)
+            T = np.maximum(orc.dense(H, Wa[l], f64=False, threads=th), 0)
+            Y = orc.dense(T, Wb[l], f64=False, threads=th)
+        P_ref = orc.softmax_rows(Y, threads=th)
+        cpu_s = time.perf_counter() - t0
+        cpu = {"value": round(cpu_s * 1e3, 1), "unit": "ms", "cores": th, "kind": "port",
+               "sample": "1 full forward of the same workload (OpenMP over rows, fp32)"}
+        lg = d_logits.cpu().numpy()
+        parity = {"logits_max_rel_err": float(np.abs(lg - Y).max() / np.abs(Y).max()),
+                  "softmax_max_abs_err": float(np.abs(d_P.cpu().numpy() - P_ref).max())}
+        log("cpu forward %.1f ms on %d threads; parity %s" % (cpu_s * 1e3, th, parity))
+    return {
+        "metric": "gin_5layer_fwd_ms", "value": round(wall_ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[2]: 5-layer GIN forward, RMAT V=%d nnz=%d, 100->64->47, 2-layer MLP per layer, eps=0, "
+                               "ps=%d wpb=%d dist=%d" % (V, nnz, ps, wpb, dist)},
+        "roofline": {"bound": "hbm", "kernel": "k_agg (GIN, dim 64)", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "algorithmic_bytes": nbytes, "avg_launch_ms": round(agg_ms, 4)},
+        "cpu_baseline": cpu, "parity": parity,
+        "detail": {"stage_ms": {k: round(v, 4) for k, v in avg.items()}, "mlp_total_ms": round(mlp_ms, 4)},
+    }
+
+
+def bench_big(args, torch, host):
+    """configs[4]: large-share stress.  One rank's 1/8 share of a 111 M-node RMAT graph (ids scrambled): ~13.9 M rows,
+    ~200 M neighbors, bf16 width-128 tables (local + a separate remote table indexed by global id), fp32 accumulation,
+    then the 128x128 update on the bf16 matrix cores.  --big-scale shrinks every size by 2^k for a quicker run."""
+    k = args.big_scale
+    scale, V, draws, dim, num_gpus = 27 - k, 111_000_000 >> k, 790_000_000 >> k, 128, 8
+    ps, wpb, dist = args.ps, args.wpb, args.dist
+    npp, lb, ub = host.range_partition(V, num_gpus, 0)
+    t0 = time.time()
+    ptr, col = host.gen_rmat(scale, V, draws, seed=5, scramble=True, row_lo=lb, row_hi=ub)
+    lp, rp, lc, rc = host.split_CSR(ptr, col, lb, ub)
+    R, nnz = ub - lb, len(col)
+    log("share: rows=%d nnz=%d local=%d remote=%d in %.1fs" % (R, nnz, len(lc), len(rc), time.time() - t0))
+    dev = "cuda"
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(5)
+    d_xr = torch.randn(num_gpus * npp, dim, device=dev, dtype=torch.bfloat16, generator=gen)
+    d_xl = d_xr[lb:ub].clone()
+    d = [torch.from_numpy(a).to(dev) if len(a) else torch.zeros(1, dtype=torch.int32, device=dev) for a in (lp, lc, rp, rc)]
+    d_out = torch.empty(R, dim, device=dev)
+    W = host.glorot(dim, dim, seed=6)
+    d_W = torch.from_numpy(W).to(dev).to(torch.bfloat16)
+    d_next = torch.empty(R, dim, device=dev, dtype=torch.bfloat16)
+    stages = [
+        lambda: host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, ps, wpb, dist, input_remote=d_xr),
+        lambda: host.dense_forward_bf16(d_next, d_out, d_W, R, dim, dim),
+    ]
+    for _ in range(args.warmup):
+        for fn in stages:
+            fn()
+    torch.cuda.synchronize()
+    timer = StageTimer(torch, ["agg", "update"])
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        timer.step(stages)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    avg = timer.averages()
+    nbytes = agg_bytes(nnz, R, dim, s_in=2, ptr_arrays=2)
+    achieved = nbytes / (avg["agg"] * 1e-3) / 1e9
+    gflop = 2.0 * R * dim * dim / 1e9
+    gemm_bytes = R * dim * 4 + R * dim * 2 + dim * dim * 2
+    parity = None
+    cpu = None
+    if not args.no_cpu:
+        from oracle import orc
+        th = orc.max_threads()
+        deg = np.diff(lp) + np.diff(rp)
+        rng = np.random.default_rng(0)
+        rows = np.unique(np.concatenate([np.argsort(deg)[-20:], rng.integers(0, R, 2000)])).astype(np.int32)
+        # The sampled rows as a small problem of their own: a compact table with just the feature rows they touch
+        # (the local table holds the same values as rows lb..ub of the global one), ids renumbered into it.
+        nbrs = [np.concatenate([lc[lp[r]:lp[r + 1]], rc[rp[r]:rp[r + 1]]]) for r in rows]
+        need = np.unique(np.concatenate(nbrs))
+        x_small = d_xr[torch.from_numpy(need.astype(np.int64)).to(dev)].float().cpu().numpy()
+        sp = np.zeros(len(rows) + 1, np.int32)
+        sp[1:] = np.cumsum([len(x) for x in nbrs])
+        cc = np.searchsorted(need, np.concatenate(nbrs)).astype(np.int32)
+        zp_ = np.zeros(len(rows) + 1, np.int32)
+        n_small = len(rows)
+        dummy_local = np.zeros((n_small, dim), np.float32)
+        t0 = time.perf_counter()
+        want = orc.sag_np_div(dummy_local, x_small, zp_, np.zeros(0, np.int32), sp, cc, 0, n_small, dim, n_small, f64=True, threads=th)
+        cpu_s = time.perf_counter() - t0
+        mag = orc.sag_np_div_rows(np.arange(n_small, dtype=np.int32), dummy_local, x_small, zp_, np.zeros(0, np.int32), sp, cc, 0,
+                                  n_small, dim, n_small, abs_sum=True, threads=th)
+        got = d_out[torch.from_numpy(rows.astype(np.int64)).to(dev)].cpu().numpy()
+        err = float(np.max(np.abs(got - want) / (mag + 1e-30)))
+        parity = {"rows_checked": int(len(rows)), "agg_max_err_over_abs_sum": err}
+        edges = int(sp[-1])
+        cpu = {"value": round(edges / cpu_s / 1e6, 2), "unit": "M edges/s", "cores": th, "kind": "port",
+               "sample": "%d sampled rows (%d neighbors) of the same share, double accumulation" % (len(rows), edges),
+               "gpu_same_unit": round(nnz / (avg["agg"] * 1e-3) / 1e6, 1)}
+        log("parity %s; cpu %s" % (parity, cpu))
+    return {
+        "metric": "np_aggregation_plus_update_ms", "value": round(wall_ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[4] / 2^%d: rank-0 1/8 share of RMAT V=%d (scrambled), rows=%d nnz=%d (local %d, remote %d), "
+                               "bf16 dim %d, fp32 accumulate, then %dx%d bf16 MFMA update; ps=%d wpb=%d dist=%d"
+                               % (k, V, R, nnz, len(lc), len(rc), dim, dim, dim, ps, wpb, dist)},
+        "roofline": {"bound": "hbm", "kernel": "k_agg (bf16 dim 128, local+remote)", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "algorithmic_bytes": nbytes, "avg_launch_ms": round(avg["agg"], 4)},
+        "cpu_baseline": cpu, "parity": parity,
+        "detail": {"stage_ms": {k2: round(v, 4) for k2, v in avg.items()},
+                   "update_tflops": round(gflop / avg["update"], 2), "update_gbps": round(gemm_bytes / (avg["update"] * 1e-3) / 1e9, 1)},
+    }
+
+
 def bench_copy(args, torch, host):
     """Plain device copy of a known size: the stream-copy ceiling, and the yardstick the profiler's FETCH_SIZE /
     WRITE_SIZE counters are scaled against."""
@@ -304,12 +487,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gcn2", choices=["gcn2", "share", "copy"])
+    ap.add_argument("--workload", default="gcn2", choices=["gcn2", "share", "gin", "big", "copy"])
     ap.add_argument("--ps", type=int, default=16)
     ap.add_argument("--wpb", type=int, default=8)
     ap.add_argument("--dist", type=int, default=0, help="0 = the workload's default (16 for gcn2, as the reference's bench_MGG.py; 1 for share)")
     ap.add_argument("--share-density", type=int, default=1, help="multiplies the number of RMAT draws of --workload share")
     ap.add_argument("--small", action="store_true", help="tiny graph, for a quick functional run")
+    ap.add_argument("--big-scale", type=int, default=0, help="--workload big: divide every size by 2^k")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -326,8 +510,8 @@ def main():
     host.use_torch_stream()
     log("device:", host.device_name())
     if args.dist <= 0:
-        args.dist = 16 if args.workload == "gcn2" else 1
-    res = {"gcn2": bench_gcn2, "share": bench_share, "copy": bench_copy}[args.workload](args, torch, host)
+        args.dist = 1 if args.workload == "share" else 16
+    res = {"gcn2": bench_gcn2, "share": bench_share, "gin": bench_gin, "big": bench_big, "copy": bench_copy}[args.workload](args, torch, host)
     print(json.dumps(res), flush=True)
 
 
