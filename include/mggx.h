@@ -109,6 +109,12 @@ int mggx_graph_write(const char *beg_file, const char *csr_file, const char *wei
  * First call with NULL arrays returns M (rows) and L (entries). */
 int mggx_mtx_read(const char *path, int *num_rows, int *num_entries, int *row_ptr, int *col_ind);
 
+/* Text edge list -> the binary CSR triple (<prefix>_beg_pos.bin, _csr.bin, _weight.bin).  Stands in for the
+ * reference's dataset/0_to_base_zero.py + dataset/1_txt2bin.py, whose text_to_bin tool is not part of the reference
+ * tree.  is_mtx != 0: MatrixMarket-style input (1-based, size line); else a 0-based "src dst" list.  Edges are grouped
+ * by source, file order kept inside a row; weights are 1. */
+int mggx_edgelist_to_bin(const char *path, int is_mtx, const char *out_prefix, int *num_nodes, int64_t *num_edges);
+
 /* Deterministic synthetic graphs (no counterpart in the reference, which only
  * loads files).  Both produce a sorted, duplicate-free CSR of the symmetrised
  * graph with one self loop per node.  Two-call protocol: gen -> sizes, then
@@ -137,6 +143,12 @@ int mggx_fill_uniform(float *dst, int64_t n, float lo, float hi, uint64_t seed);
  * arrays to get *num_parts (synchronises), then with arrays of the right size. */
 int mggx_build_part_device(const int *d_indptr, int num_nodes, int part_size, int compat,
                            int *d_part_ptr, int *d_part2node, int *d_node2part, int *num_parts);
+
+/* split_CSR on the GPU (include/neighbor_utils.cuh:381-405), bit-identical to mggx_split_csr: d_ptr/d_col are the
+ * whole graph's CSR on the device.  Call once with the two column arrays NULL: fills d_local_ptr/d_remote_ptr
+ * ((ub-lb)+1 entries each) and returns the totals (synchronises); then again with column arrays of those sizes. */
+int mggx_split_csr_device(const int *d_ptr, const int *d_col, int lb, int ub, int *d_local_ptr, int *d_remote_ptr,
+                          int *d_local_col, int *d_remote_col, int64_t *n_local, int64_t *n_remote);
 
 /* ---- aggregation ---- */
 

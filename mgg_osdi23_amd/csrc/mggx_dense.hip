@@ -284,6 +284,35 @@ __global__ void __launch_bounds__(256) k_softmax_rows(float *__restrict__ out, c
     const long long row = wave_id * rows_per_wave + g;
     const bool ok = row < n;
     const float *x = in + (ok ? row : 0) * ld_in;
+    if (c <= 4 * G) {
+        // the whole row lives in registers: one read, one write
+        float v[4];
+        float m = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int j = l + t * G;
+            v[t] = j < c ? x[j] : -INFINITY;
+            m = fmaxf(m, v[t]);
+        }
+        for (int o = G >> 1; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        float s = 0.f;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            v[t] = __expf(v[t] - m);  // exp(-inf) = 0 for the padding
+            s += v[t];
+        }
+        for (int o = G >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+        const float inv = 1.0f / s;
+        if (ok) {
+            float *o_ = out + row * ld_out;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int j = l + t * G;
+                if (j < c) o_[j] = v[t] * inv;
+            }
+        }
+        return;
+    }
     float m = -INFINITY;
     for (int j = l; j < c; j += G) m = fmaxf(m, x[j]);
     for (int o = G >> 1; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
@@ -453,8 +482,8 @@ MGGX_EXPORT int mggx_softmax_rows(float *d_out, const float *d_in, int64_t n, in
     if (!ld_in) ld_in = c;
     if (!ld_out) ld_out = c;
     if (ld_in < c || ld_out < c) return fail(MGGX_EINVAL, "softmax_rows: row stride smaller than width");
-    int G = 1;
-    while (G < c && G < 64) G <<= 1;
+    int G = 1;  // lanes per row: up to four values per lane stay in registers
+    while (G * 4 < c && G < 64) G <<= 1;
     const long long rows_per_block = 4 * (64 / G);
     const long long blocks = (n + rows_per_block - 1) / rows_per_block;
     if (blocks > 0x7fffffffLL) return fail(MGGX_ELIMIT, "softmax_rows: too many rows");

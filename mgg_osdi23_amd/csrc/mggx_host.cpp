@@ -288,6 +288,66 @@ MGGX_EXPORT int mggx_mtx_read(const char *path, int *num_rows, int *num_entries,
 }
 
 // ---------------------------------------------------------------------------
+// Text edge list -> binary CSR triple.  Stands in for the reference's dataset pipeline (dataset/0_to_base_zero.py
+// rewrites a .mtx to a 0-based "src dst" list, dataset/1_txt2bin.py hands it to an external text_to_bin tool that is
+// not part of the reference tree).  Input: a MatrixMarket-style file (is_mtx != 0: '%' comments, a size line, then
+// 1-based "row col [value]" lines) or a 0-based "src dst" list.  Output: <prefix>_beg_pos.bin / _csr.bin /
+// _weight.bin in the layout mggx_graph_read expects; edges are grouped by source with a stable counting sort (file
+// order is kept inside a row), weights are 1.
+MGGX_EXPORT int mggx_edgelist_to_bin(const char *path, int is_mtx, const char *out_prefix, int *num_nodes, int64_t *num_edges)
+{
+    if (!path || !out_prefix) return fail(MGGX_EINVAL, "edgelist_to_bin: NULL argument");
+    FILE *f = fopen(path, "r");
+    if (!f) return fail(MGGX_EIO, "edgelist_to_bin: cannot open %s", path);
+    std::vector<int> src, dst;
+    long long declared_rows = 0;
+    char line[512];
+    bool size_line_pending = is_mtx != 0;
+    while (fgets(line, sizeof(line), f)) {
+        if (line[0] == '%' || line[0] == '#' || line[0] == '\n') continue;
+        if (size_line_pending) {
+            long long m = 0, n = 0, l = 0;
+            if (sscanf(line, "%lld %lld %lld", &m, &n, &l) < 2) {
+                fclose(f);
+                return fail(MGGX_EFORMAT, "edgelist_to_bin: bad size line in %s", path);
+            }
+            declared_rows = std::max(m, n);
+            size_line_pending = false;
+            continue;
+        }
+        long long a = 0, b = 0;
+        if (sscanf(line, "%lld %lld", &a, &b) != 2) {
+            fclose(f);
+            return fail(MGGX_EFORMAT, "edgelist_to_bin: malformed line in %s: %.40s", path, line);
+        }
+        if (is_mtx) { --a; --b; }
+        if (a < 0 || b < 0 || a > std::numeric_limits<int>::max() - 1 || b > std::numeric_limits<int>::max() - 1) {
+            fclose(f);
+            return fail(MGGX_EFORMAT, "edgelist_to_bin: node id out of range in %s", path);
+        }
+        src.push_back((int)a);
+        dst.push_back((int)b);
+    }
+    fclose(f);
+    if (src.empty()) return fail(MGGX_EFORMAT, "edgelist_to_bin: no edges in %s", path);
+    if (src.size() > (size_t)std::numeric_limits<int>::max()) return fail(MGGX_ELIMIT, "edgelist_to_bin: too many edges");
+    long long V = declared_rows;
+    for (size_t i = 0; i < src.size(); ++i) V = std::max<long long>(V, std::max(src[i], dst[i]) + 1LL);
+    std::vector<int> beg((size_t)V + 1, 0), csr(src.size());
+    for (int s : src) beg[(size_t)s + 1]++;
+    for (long long v = 0; v < V; ++v) beg[(size_t)v + 1] += beg[(size_t)v];
+    std::vector<int> cursor(beg.begin(), beg.end() - 1);
+    for (size_t i = 0; i < src.size(); ++i) csr[(size_t)cursor[(size_t)src[i]]++] = dst[i];
+    const std::string p(out_prefix);
+    int rc = mggx_graph_write((p + "_beg_pos.bin").c_str(), (p + "_csr.bin").c_str(), (p + "_weight.bin").c_str(), (int)V,
+                              beg.data(), csr.data(), nullptr);
+    if (rc) return rc;
+    if (num_nodes) *num_nodes = (int)V;
+    if (num_edges) *num_edges = (int64_t)src.size();
+    return MGGX_OK;
+}
+
+// ---------------------------------------------------------------------------
 // Synthetic graphs.
 namespace {
 

@@ -219,6 +219,53 @@ __global__ void __launch_bounds__(256) k_max_i32(const int *__restrict__ v, long
     if (threadIdx.x == 0) atomicMax(out, red[0]);
 }
 
+// split_CSR on the GPU, one wavefront per row.  Pass 1 counts the neighbors inside [lb,ub); pass 2 is a stable
+// partition of the row (ballot + prefix popcount keeps the order inside each side).
+__global__ void __launch_bounds__(256) k_split_count(const int *__restrict__ ptr, const int *__restrict__ col, int lb, int ub,
+                                                     int *__restrict__ cnt_l, int *__restrict__ cnt_r)
+{
+    const int lane = (int)(threadIdx.x & 63u);
+    const int rows = ub - lb;
+    for (long long r = (long long)blockIdx.x * 4 + (threadIdx.x >> 6); r < rows; r += (long long)gridDim.x * 4) {
+        const int beg = ptr[lb + r], end = ptr[lb + r + 1];
+        int local = 0;
+        for (int e = beg + lane; e < end; e += 64) {
+            const int u = col[e];
+            local += (u >= lb && u < ub) ? 1 : 0;
+        }
+        for (int o = 32; o > 0; o >>= 1) local += __shfl_xor(local, o, 64);
+        if (lane == 0) {
+            cnt_l[r] = local;
+            cnt_r[r] = (end - beg) - local;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) k_split_fill(const int *__restrict__ ptr, const int *__restrict__ col, int lb, int ub,
+                                                    const int *__restrict__ lptr, const int *__restrict__ rptr,
+                                                    int *__restrict__ lcol, int *__restrict__ rcol)
+{
+    const int lane = (int)(threadIdx.x & 63u);
+    const int rows = ub - lb;
+    const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    for (long long r = (long long)blockIdx.x * 4 + (threadIdx.x >> 6); r < rows; r += (long long)gridDim.x * 4) {
+        const int beg = ptr[lb + r], end = ptr[lb + r + 1];
+        int lo = lptr[r], ro = rptr[r];
+        for (int e0 = beg; e0 < end; e0 += 64) {
+            const int e = e0 + lane;
+            const bool valid = e < end;
+            const int u = valid ? col[e] : 0;
+            const bool is_local = valid && u >= lb && u < ub;
+            const unsigned long long ml = __ballot(is_local), mv = __ballot(valid);
+            const unsigned long long mr = mv & ~ml;
+            if (is_local) lcol[lo + __popcll(ml & below)] = u;
+            else if (valid) rcol[ro + __popcll(mr & below)] = u;
+            lo += __popcll(ml);
+            ro += __popcll(mr);
+        }
+    }
+}
+
 __global__ void k_set_tail(int *node2part, int num_nodes)
 {
     node2part[num_nodes + 1] = node2part[num_nodes];
@@ -460,4 +507,43 @@ MGGX_EXPORT int mggx_build_part_device(const int *d_indptr, int num_nodes, int p
     (void)hipFree(d_cnt);
     if (own_n2p) (void)hipFree(d_n2p);
     return rc;
+}
+
+MGGX_EXPORT int mggx_split_csr_device(const int *d_ptr, const int *d_col, int lb, int ub, int *d_local_ptr,
+                                      int *d_remote_ptr, int *d_local_col, int *d_remote_col, int64_t *n_local,
+                                      int64_t *n_remote)
+{
+    if (!d_ptr || lb < 0 || ub < lb || !d_local_ptr || !d_remote_ptr)
+        return fail(MGGX_EINVAL, "split_csr_device: NULL pointer or bad range [%d,%d)", lb, ub);
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    mggx::State &s = mggx::state();
+    const int rows = ub - lb;
+    const unsigned blocks = (unsigned)std::min<long long>(((long long)rows + 3) / 4 + 1, 256 * 64);
+    if (!d_local_col || !d_remote_col) {
+        // pass 1: per-row counts -> the two pointer arrays and the totals
+        int *d_cnt = nullptr;
+        MGGX_HIP(hipMalloc((void **)&d_cnt, sizeof(int) * 2 * (size_t)std::max(rows, 1)));
+        long long tl = 0, tr = 0;
+        do {
+            if (rows > 0) {
+                if (!d_col) { rc = fail(MGGX_EINVAL, "split_csr_device: NULL column array"); break; }
+                mggx::k_split_count<<<blocks, 256, 0, s.stream>>>(d_ptr, d_col, lb, ub, d_cnt, d_cnt + rows);
+            }
+            rc = mggx::exclusive_scan_i32(d_cnt, d_local_ptr, rows, &tl);
+            if (rc) break;
+            rc = mggx::exclusive_scan_i32(d_cnt + rows, d_remote_ptr, rows, &tr);
+        } while (0);
+        (void)hipFree(d_cnt);
+        if (rc) return rc;
+        if (n_local) *n_local = tl;
+        if (n_remote) *n_remote = tr;
+        return MGGX_OK;
+    }
+    // pass 2: fill, using the pointer arrays of pass 1
+    if (rows > 0) {
+        mggx::k_split_fill<<<blocks, 256, 0, s.stream>>>(d_ptr, d_col, lb, ub, d_local_ptr, d_remote_ptr, d_local_col, d_remote_col);
+        MGGX_LAUNCH_CHECK("k_split_fill");
+    }
+    return MGGX_OK;
 }

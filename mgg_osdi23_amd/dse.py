@@ -29,8 +29,11 @@ def build_workload(name: str, dim: int, small: bool):
         lp, rp, lc, rc = host.split_CSR(ptr, col, lb, ub)
         rows_tbl = num_gpus * npp
     else:
-        scale, V, draws = (18, 233_000, 216_000_000) if not small else (14, 16_000, 1_500_000)
-        ptr, col = host.gen_rmat(scale, V, draws, seed=42)
+        if name == "sparse":  # 2.45 M nodes, ~123 M nnz (avg degree ~50): the GIN benchmark's graph
+            scale, V, draws, seed = (22, 2_450_000, 64_000_000, 3) if not small else (16, 50_000, 1_300_000, 3)
+        else:                 # 233 K nodes, ~228 M nnz (avg degree ~980): the GCN benchmark's graph
+            scale, V, draws, seed = (18, 233_000, 216_000_000, 42) if not small else (14, 16_000, 1_500_000, 42)
+        ptr, col = host.gen_rmat(scale, V, draws, seed=seed)
         npp, lb, ub = V, 0, V
         lp, lc = ptr, col
         rp, rc = np.zeros(V + 1, np.int32), np.zeros(0, np.int32)
@@ -67,7 +70,7 @@ def time_setting(w, ps, wpb, dist, iters):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="share", choices=["share", "whole"])
+    ap.add_argument("--workload", default="share", choices=["share", "whole", "sparse"])
     ap.add_argument("--dim", type=int, default=16)
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--small", action="store_true")

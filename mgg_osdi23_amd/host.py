@@ -45,7 +45,7 @@ EXPORTS = [
     "mggx_timer_create", "mggx_timer_start", "mggx_timer_stop", "mggx_timer_elapsed_ms", "mggx_timer_destroy",
     "mggx_release_cached", "mggx_range_partition", "mggx_split_csr", "mggx_build_part", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
-    "mggx_fill_uniform", "mggx_build_part_device", "mggx_sag_np_div", "mggx_sag_parts", "mggx_spmm",
+    "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_parts", "mggx_spmm",
     "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
 ]
 
@@ -146,6 +146,30 @@ def mtx_read(path: str):
     ci = np.zeros(l.value, np.int32)
     _check(lib().mggx_mtx_read(path.encode(), C.byref(m), C.byref(l), _iptr(rp), _iptr(ci)))
     return rp, ci
+
+
+def edgelist_to_bin(path: str, out_prefix: str, is_mtx: bool = False):
+    """Text edge list (.mtx or 0-based 'src dst') -> <prefix>_beg_pos.bin/_csr.bin/_weight.bin; returns (V, E)."""
+    v, e = C.c_int(), C.c_int64()
+    _check(lib().mggx_edgelist_to_bin(path.encode(), int(is_mtx), out_prefix.encode(), C.byref(v), C.byref(e)))
+    return v.value, e.value
+
+
+def split_CSR_device(d_ptr, d_col, lb: int, ub: int):
+    """split_CSR on the GPU -> (local_ptr, remote_ptr, local_col_idx, remote_col_idx) as device tensors."""
+    import torch
+    rows = ub - lb
+    lp = torch.zeros(rows + 1, dtype=torch.int32, device=d_ptr.device)
+    rp = torch.zeros(rows + 1, dtype=torch.int32, device=d_ptr.device)
+    nl, nr = C.c_int64(), C.c_int64()
+    _check(lib().mggx_split_csr_device(_dptr(d_ptr), _dptr(d_col), lb, ub, _dptr(lp), _dptr(rp), None, None,
+                                       C.byref(nl), C.byref(nr)))
+    lc = torch.zeros(max(nl.value, 1), dtype=torch.int32, device=d_ptr.device)
+    rc = torch.zeros(max(nr.value, 1), dtype=torch.int32, device=d_ptr.device)
+    _check(lib().mggx_split_csr_device(_dptr(d_ptr), _dptr(d_col), lb, ub, _dptr(lp), _dptr(rp), _dptr(lc), _dptr(rc),
+                                       C.byref(nl), C.byref(nr)))
+    sync()
+    return lp, rp, lc[: nl.value], rc[: nr.value]
 
 
 def gen_rmat(scale: int, num_nodes: int, num_draws: int, a=0.57, b=0.19, c=0.19, seed=0, scramble=False,

@@ -210,6 +210,26 @@ def test_mtx_loader(tmp_path):
         host.mtx_read(str(tmp_path / "none.mtx"))
 
 
+def test_edgelist_to_bin_converter(tmp_path):
+    """.mtx / 0-based edge list -> binary triple, read back by all loaders; file order is kept inside a row."""
+    mtx = tmp_path / "g.mtx"
+    mtx.write_text("%%MatrixMarket matrix coordinate pattern general\n6 6 7\n3 1\n1 4 1.0\n3 6\n1 2\n6 6\n3 2\n5 1\n")
+    V, E = host.edgelist_to_bin(str(mtx), str(tmp_path / "g"), is_mtx=True)
+    assert (V, E) == (6, 7)
+    want_ptr, want_col = [0, 2, 2, 5, 5, 6, 7], [3, 1, 0, 5, 1, 0, 5]
+    files = [str(tmp_path / ("g" + s)) for s in ("_beg_pos.bin", "_csr.bin", "_weight.bin")]
+    for loader in (host.graph_read, orc.graph_load) + ((orc.ref_graph_load,) if orc.have_ref() else ()):
+        b, c, w = loader(*files)
+        assert b.tolist() == want_ptr and c.tolist() == want_col and w.tolist() == [1] * 7
+    el = tmp_path / "g0.txt"
+    el.write_text("2 0\n0 3\n2 5\n0 1\n5 5\n2 1\n4 0\n")  # the same graph, already 0-based (dataset/0_to_base_zero.py output)
+    assert host.edgelist_to_bin(str(el), str(tmp_path / "h")) == (6, 7)
+    b, c, _ = host.graph_read(*[str(tmp_path / ("h" + s)) for s in ("_beg_pos.bin", "_csr.bin", "_weight.bin")])
+    assert b.tolist() == want_ptr and c.tolist() == want_col
+    with pytest.raises(host.MggxError):
+        host.edgelist_to_bin(str(tmp_path / "missing.txt"), str(tmp_path / "x"))
+
+
 # --------------------------------------------------------------------------- generators
 def test_generators_are_deterministic_and_well_formed():
     for gen in (lambda: host.gen_er(2000, 10.0, seed=4), lambda: host.gen_rmat(11, 1800, 30000, seed=4, threads=3),

@@ -281,6 +281,26 @@ def test_build_part_device_bit_exact(gpu, rmat_graph, ps):
             assert np.array_equal(g.cpu().numpy(), w), name
 
 
+@pytest.mark.parametrize("num_gpus,pe", [(1, 0), (3, 0), (3, 1), (3, 2), (8, 5)])
+def test_split_csr_device_bit_exact(gpu, rmat_graph, num_gpus, pe):
+    V, ptr, col = rmat_graph
+    npp, lb, ub = orc.range_partition(V, num_gpus, pe)
+    want = orc.split_csr(ptr, col, lb, ub)
+    got = gpu.split_CSR_device(to_dev(ptr), to_dev(col), lb, ub)
+    for g, w, name in zip(got, want, ("local_ptr", "remote_ptr", "local_col_idx", "remote_col_idx")):
+        assert np.array_equal(g.cpu().numpy(), w), name
+    # ragged: empty rows, an unsorted row, a 5000-neighbor row
+    rng = np.random.default_rng(1)
+    deg = np.array([0, 5000, 3, 0, 0, 130, 64, 1, 0], np.int64)
+    p = np.zeros(len(deg) + 1, np.int32)
+    p[1:] = np.cumsum(deg)
+    c = rng.integers(0, len(deg), int(p[-1])).astype(np.int32)
+    want = orc.split_csr(p, c, 2, 7)
+    got = gpu.split_CSR_device(to_dev(p), to_dev(c), 2, 7)
+    for g, w in zip(got, want):
+        assert np.array_equal(g.cpu().numpy(), w)
+
+
 # --------------------------------------------------------------------------- dense update and softmax
 @pytest.mark.parametrize("n,d1,d2", [(1000, 602, 16), (1000, 16, 41), (777, 100, 64), (512, 64, 64), (300, 64, 47),
                                      (256, 128, 128), (65, 7, 3), (1, 1, 1), (130, 33, 130)])
@@ -358,10 +378,8 @@ def test_bf16_tables(gpu, rmat_graph, dim):
 # --------------------------------------------------------------------------- dense update on the bf16 matrix cores
 @pytest.mark.parametrize("n,d1,d2", [(1000, 128, 128), (333, 64, 47), (257, 100, 64), (64, 602, 16), (17, 7, 3), (500, 256, 200)])
 @pytest.mark.parametrize("x_bf16,out_bf16", [(False, False), (True, False), (False, True), (True, True)])
-def test_dense_update_bf16(gpu, n, d1, d2, x_bf16, out_bf16, addressing):
+def test_dense_update_bf16(gpu, n, d1, d2, x_bf16, out_bf16):
     import torch
-    if addressing == "wide":
-        pytest.skip("addressing switch does not concern the dense kernels")
     x = gpu.fill_normal((n, d1), seed=50)
     w = gpu.glorot(d1, d2, seed=51)
     wb = to_dev(w).to(torch.bfloat16)
