@@ -171,7 +171,8 @@ typedef struct mggx_agg_opts {
  * ps/wpb/dist are MGG's partSize / warpPerBlock / interleaved_dist: partitions
  * of <= ps neighbors of one row, wpb 64-lane wavefronts per workgroup, dist
  * consecutive partition rounds per wavefront.  They change speed, never the
- * mathematical result.  opts may be NULL (fp32, overwrite, ld == dim).
+ * mathematical result.  wpb = 0 and/or dist = 0 let the library choose them from the
+ * partition count per row.  opts may be NULL (fp32, overwrite, ld == dim).
  * The partition plan of (d_ptr_l, d_ptr_r, rows, ps) is built on first use and
  * cached by pointer identity: the CSR arrays must not be rewritten in place
  * while cached (mggx_release_cached() drops the cache). */

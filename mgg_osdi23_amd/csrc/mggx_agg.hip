@@ -211,6 +211,28 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int row, int l, con
             return;
         }
     }
+    if constexpr (MODE == MODE_F32_VEC4) {
+        // the same epilogue as finish_elem on this lane's four contiguous elements, with vector loads and one store
+        if (NV * l < a.dim) {
+            const float sc = a.rs_out ? a.rs_out[row] : 1.0f;
+            float4 v = make_float4(acc[0] * sc, acc[1] * sc, acc[2] * sc, acc[3] * sc);
+            if (a.flags & MGGX_AGG_GIN) {
+                const float4 s = *reinterpret_cast<const float4 *>(static_cast<const float *>(a.in_l) + (long long)row * a.ld_in + 4 * l);
+                const float k = 1.0f + a.eps;
+                v.x += k * s.x; v.y += k * s.y; v.z += k * s.z; v.w += k * s.w;
+            }
+            float4 *o = reinterpret_cast<float4 *>(a.out + (long long)row * a.ld_out + 4 * l);
+            if (a.flags & MGGX_AGG_ACCUMULATE) {
+                const float4 p = *o;
+                v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
+            }
+            if (a.flags & MGGX_AGG_RELU) {
+                v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f);
+            }
+            *o = v;
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int d = elem_of<LPR, MODE>(l, i);
@@ -475,32 +497,55 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     if (open) emit(false);
 }
 
-// Rows that cross workgroups: the workgroup where the row starts left a tail
-// entry; every later workgroup up to the one where it ends left a head entry.
-// One block per workgroup slot; it acts only when that slot's tail is valid.
+// Rows that cross workgroups: the workgroup where the row starts left a tail entry; every later workgroup up to
+// the one where it ends left a head entry.  Each wavefront scans 64 consecutive workgroup slots (one coalesced
+// header load), then finishes the rows whose tail sits there, `group` of them at a time: lane = (walker, component)
+// with `comp_lanes` = power of two >= dim (<= 64); a walker sums its row's chain of head entries in order, four loads
+// in flight.  Wider rows (dim > 64) use one walker and several components per lane.
 __global__ void __launch_bounds__(256) k_agg_fixup(const AggArgs a, int num_wg, int comp_lanes)
 {
-    __shared__ float red[256];
-    const int b = (int)blockIdx.x;
-    const int2 t = a.c_hdr[2 * b + 1];
-    if (!(t.y & HDR_VALID)) return;
-    const int row = t.x;
-    const int last_wg = (a.off[row + 1] - 1) / a.parts_per_wg;
-    const int n = last_wg - b;  // head entries of workgroups b+1 .. last_wg
-    const int c = (int)threadIdx.x % comp_lanes;
-    const int walker = (int)threadIdx.x / comp_lanes;
-    const int walkers = 256 / comp_lanes;
-    float s = 0.f;
-    if (c < a.dim)
-        for (int k = walker; k < n; k += walkers) s += a.c_val[(size_t)(2 * (b + 1 + k)) * a.cpad + c];
-    red[threadIdx.x] = s;
-    __syncthreads();
-    if (walker == 0 && c < a.dim) {
-        float total = a.c_val[(size_t)(2 * b + 1) * a.cpad + c];
-        for (int w = 0; w < walkers; ++w) total += red[w * comp_lanes + c];
-        finish_elem(a, row, c, total);
+    const int lane = lane_id();
+    const long long base = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 64;
+    if (base >= num_wg - 1) return;
+    const long long slot = base + lane;
+    int2 t = make_int2(-1, 0);
+    if (slot < num_wg - 1) t = a.c_hdr[2 * slot + 1];
+    unsigned long long todo = __ballot((t.y & HDR_VALID) != 0);
+    const int group = 64 / comp_lanes;  // rows finished at once
+    const int walker = lane / comp_lanes, c0 = lane % comp_lanes;
+    while (todo) {
+        // the walker-th set bit of `todo` is this walker's slot
+        unsigned long long m = todo;
+        int mine = -1;
+        for (int w = 0; w < group && m; ++w) {
+            const int bit = __ffsll((long long)m) - 1;
+            if (w == walker) mine = bit;
+            m &= m - 1;
+        }
+        todo = m;
+        const int src = mine >= 0 ? mine : lane;
+        const int row = lane_read(t.x, src);
+        if (mine >= 0) {
+            const long long b = base + mine;
+            const int n = (a.off[row + 1] - 1) / a.parts_per_wg - (int)b;  // head entries of workgroups b+1 .. b+n
+            for (int c = c0; c < a.dim; c += comp_lanes) {
+                float total = a.c_val[(size_t)(2 * b + 1) * a.cpad + c];
+                int k = 0;
+                for (; k + 4 <= n; k += 4) {
+                    const float v0 = a.c_val[(size_t)(2 * (b + 1 + k)) * a.cpad + c];
+                    const float v1 = a.c_val[(size_t)(2 * (b + 2 + k)) * a.cpad + c];
+                    const float v2 = a.c_val[(size_t)(2 * (b + 3 + k)) * a.cpad + c];
+                    const float v3 = a.c_val[(size_t)(2 * (b + 4 + k)) * a.cpad + c];
+                    total += v0;
+                    total += v1;
+                    total += v2;
+                    total += v3;
+                }
+                for (; k < n; ++k) total += a.c_val[(size_t)(2 * (b + 1 + k)) * a.cpad + c];
+                finish_elem(a, row, c, total);
+            }
+        }
     }
-    (void)num_wg;
 }
 
 // Rows with no neighbor at all: the sum is zero.
@@ -547,8 +592,8 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
 {
     State &st = state();
     if (dim < 1 || dim > 256) return fail(MGGX_ELIMIT, "aggregation: dim %d outside 1..256", dim);
-    if (wpb < 1 || wpb > 16) return fail(MGGX_EINVAL, "aggregation: wpb %d outside 1..16", wpb);
-    if (dist < 1) return fail(MGGX_EINVAL, "aggregation: dist %d must be positive", dist);
+    if (wpb < 0 || wpb > 16) return fail(MGGX_EINVAL, "aggregation: wpb %d outside 0..16 (0 = choose)", wpb);
+    if (dist < 0) return fail(MGGX_EINVAL, "aggregation: dist %d must not be negative (0 = choose)", dist);
     const long long ld_in = o.ld_in ? o.ld_in : dim, ld_out = o.ld_out ? o.ld_out : dim;
     if (ld_in < dim || ld_out < dim) return fail(MGGX_EINVAL, "aggregation: row stride smaller than dim");
     if (plan->rows == 0) return MGGX_OK;
@@ -572,6 +617,19 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         return fail(MGGX_EINVAL, "aggregation: unknown input dtype %d", o.in_dtype);
     }
     const int slots = 64 / lpr;
+    // 0 = let the library choose (from sweeps on the benchmark graphs): 8 wavefronts; with few slots per wavefront
+    // (wide rows) 16 rounds, so a workgroup still covers a few thousand neighbors; otherwise a workgroup tile of
+    // about 8 rows' worth of partitions (most rows then finish inside one workgroup), between 1 and 16 rounds.
+    if (wpb == 0) wpb = 8;
+    if (dist == 0) {
+        if (slots <= 4) {
+            dist = 16;
+        } else {
+            const double per_row = (double)plan->num_parts / (double)plan->rows;
+            const long long want = (long long)(8.0 * per_row / (double)(wpb * slots) + 0.999);
+            dist = (int)(want < 1 ? 1 : (want > 16 ? 16 : want));
+        }
+    }
     const long long parts_per_wg = (long long)wpb * slots * dist;
     if (parts_per_wg > 0x3fffffffLL) return fail(MGGX_ELIMIT, "aggregation: wpb*dist too large");
     const long long num_wg = (plan->num_parts + parts_per_wg - 1) / parts_per_wg;
@@ -651,8 +709,9 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         if (rc) return rc;
         MGGX_LAUNCH_CHECK("k_agg");
         if (num_wg > 1) {
-            const int comp_lanes = pow2_ceil(dim);
-            k_agg_fixup<<<dim3((unsigned)(num_wg - 1)), dim3(256), 0, st.stream>>>(a, (int)num_wg, comp_lanes);
+            const int comp_lanes = dim >= 64 ? 64 : pow2_ceil(dim);
+            const long long fix_blocks = (num_wg - 1 + 255) / 256;
+            k_agg_fixup<<<dim3((unsigned)fix_blocks), dim3(256), 0, st.stream>>>(a, (int)num_wg, comp_lanes);
             MGGX_LAUNCH_CHECK("k_agg_fixup");
         }
     }

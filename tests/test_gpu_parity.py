@@ -129,6 +129,62 @@ def test_knobs_change_speed_not_result(gpu, rmat_graph, ps, wpb, dist):
     assert_close_to_oracle(got, want, mag, FP32_TOL, "ps=%d wpb=%d dist=%d" % (ps, wpb, dist))
 
 
+@pytest.mark.parametrize("dim", [16, 64])
+def test_library_chosen_knobs(gpu, rmat_graph, dim):
+    """wpb = 0 / dist = 0 let the library pick the launch geometry; the result obeys the same tolerance."""
+    V, ptr, col = rmat_graph
+    x = gpu.fill_normal((V, dim), seed=77)
+    sh = share_of(ptr, col, V, 2, 0)
+    xl = x[sh["lb"]:sh["ub"]]
+    got = run_agg(gpu, sh, to_dev(xl), to_dev(x), dim, 16, 0, 0)
+    want, mag = oracle_agg(sh, xl, x, dim)
+    assert_close_to_oracle(got, want, mag, FP32_TOL, "auto knobs")
+
+
+def test_bad_arguments_return_errors_not_faults(gpu, rmat_graph):
+    """Shapes the kernels are not built for are refused on the host, with a message, before any launch."""
+    import torch
+    V, ptr, col = rmat_graph
+    d_ptr, d_col = to_dev(ptr), to_dev(col)
+    z = torch.zeros(V + 1, dtype=torch.int32, device="cuda")
+    x = torch.zeros(V, 16, device="cuda")
+    out = torch.zeros(V, 16, device="cuda")
+    call = lambda **kw: gpu.mgg_SAG_np_div(out, x, d_ptr, d_col, z, z, 0, V, kw.get("dim", 16), kw.get("npp", V), 0,
+                                           kw.get("ps", 16), kw.get("wpb", 4), kw.get("dist", 1), ld_in=kw.get("ld_in", 0))
+    for bad in (dict(dim=0), dict(dim=300), dict(wpb=17), dict(wpb=-1), dict(dist=-2), dict(ps=0), dict(npp=V - 1), dict(ld_in=8)):
+        with pytest.raises(gpu.MggxError):
+            call(**bad)
+    with pytest.raises(gpu.MggxError):
+        gpu.dense_forward(out, x, x, V, 16, 16, ld_x=8)
+    with pytest.raises(gpu.MggxError):
+        gpu.dense_forward(x, x, out, V, 16, 16)  # in place
+    with pytest.raises(gpu.MggxError):
+        gpu.softmax_forward(out, x, V, 0)
+    call()  # the library is still usable afterwards
+    gpu.sync()
+
+
+def test_plan_cache_eviction_and_release(gpu):
+    """More distinct graphs than the plan cache holds, then an explicit release: results stay right."""
+    import torch
+    dim = 8
+    graphs = []
+    for i in range(20):
+        V = 200 + 10 * i
+        ptr, col = gpu.gen_rmat(9, V, 1500, seed=100 + i)
+        x = gpu.fill_normal((V, dim), seed=i)
+        graphs.append((V, ptr, col, x, to_dev(ptr), to_dev(col), to_dev(x)))
+    z = torch.zeros(600, dtype=torch.int32, device="cuda")
+    for rnd in range(2):
+        for V, ptr, col, x, d_ptr, d_col, d_x in graphs:
+            out = torch.empty(V, dim, device="cuda")
+            gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, z, z, 0, V, dim, V, 0, 4, 2, 1)
+            gpu.sync()
+            want = orc.sag_np_div(x, x, ptr, col, None, None, 0, V, dim, V)
+            assert np.allclose(out.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
+        gpu.release_cached()
+
+
 # --------------------------------------------------------------------------- widths, strides, options
 @pytest.mark.parametrize("dim", [1, 2, 3, 4, 5, 8, 12, 16, 17, 24, 32, 41, 47, 64, 100, 128, 200, 256])
 def test_feature_widths(gpu, rmat_graph, dim):
