@@ -72,27 +72,41 @@ class StageTimer:
 
 
 # HBM-side bytes per aggregation call (kernel + fix-up), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by
-# what the same counters read for a 1 GiB copy (x2.000 / x1.000).  Valid for the default graphs and these knobs only.
+# what the same counters read for a 1 GiB copy (x2.000 / x1.000), and the (wpb, dist) of those runs.  The figure moves
+# by well under 1 % with (wpb, dist): the gathers are the same, only the carries differ.  Default graphs only.
 MEASURED_TRAFFIC = {
-    ("gcn2_agg2", 16, 8, 16): 28_206_272_461,
-    ("gcn2_agg1", 16, 8, 16): 6_467_971_107,
-    ("share_agg", 16, 8, 1): 1_222_766_686,
+    "gcn2_agg2": (28_216_496_128, (4, 16)),
+    "gcn2_agg1": (6_481_731_891, (4, 16)),
+    "share_agg": (1_220_807_373, (8, 1)),
+    "gin_agg": (25_550_440_960, (16, 1)),
+    "big_agg": (60_708_485_837, (4, 16)),
 }
 
 
 def load_traffic(kernel_key, args):
-    if args.small or (kernel_key == "share_agg" and args.share_density != 1):
-        return None
-    dist = args.dist
-    if dist == 0:  # what the library's own choice comes to on these graphs
-        dist = {"gcn2_agg2": 16, "gcn2_agg1": 16, "share_agg": 1}.get(kernel_key, 0)
-    return MEASURED_TRAFFIC.get((kernel_key, args.ps, args.wpb, dist))
+    """{"traffic": bytes or None, "traffic_measured_at": knobs} for the roofline object."""
+    if args.small or args.ps != 16 or (kernel_key == "share_agg" and args.share_density != 1) or \
+            (kernel_key == "big_agg" and args.big_scale != 0) or kernel_key not in MEASURED_TRAFFIC:
+        return {"traffic": None}
+    nbytes, (w, d) = MEASURED_TRAFFIC[kernel_key]
+    return {"traffic": nbytes, "traffic_measured_at": "ps=16 wpb=%d dist=%d" % (w, d)}
+
+
+def pick_knobs(args, tune):
+    """(wpb, dist) for one aggregation shape: the command line's, or, when both are 0 and tuning is on, the pair the
+    library's search measures fastest on this input (once, before the timed region; the reference fixes its pair per
+    dataset from the same kind of sweep, bench_MGG_DSE_*.py)."""
+    if args.wpb == 0 and args.dist == 0 and not args.no_tune:
+        w, d, ms = tune()
+        log("tuned: wpb=%d dist=%d (%.4f ms)" % (w, d, ms))
+        return w, d
+    return args.wpb, args.dist
 
 
 def bench_gcn2(args, torch, host):
     V, scale, draws = 233_000, 18, 216_000_000
     in_dim, hidden, out_dim = 602, 16, 41
-    ps, wpb, dist = args.ps, args.wpb, args.dist
+    ps = args.ps
     if args.small:
         V, scale, draws = 20_000, 15, 2_000_000
     t0 = time.time()
@@ -125,12 +139,18 @@ def bench_gcn2(args, torch, host):
     d_H2 = torch.empty(V, ldo, device=dev)
     d_P = torch.empty(V, out_dim, device=dev)
 
+    d_Y1.zero_()
+    d_Y2.zero_()
+    wpb1, dist1 = pick_knobs(args, lambda: host.tune_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, ps,
+                                                           row_scale_out=d_s))
+    wpb2, dist2 = pick_knobs(args, lambda: host.tune_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, ps,
+                                                           row_scale_out=d_s))
     stages = [
         lambda: host.dense_forward(d_Y1, d_X, d_W1, V, in_dim, hidden, row_scale=d_s),
-        lambda: host.mgg_SAG_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, ps, wpb, dist,
+        lambda: host.mgg_SAG_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, ps, wpb1, dist1,
                                     row_scale_out=d_s),
         lambda: host.dense_forward(d_Y2, d_H1, d_W2, V, hidden, ldo, row_scale=d_s),
-        lambda: host.mgg_SAG_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, 0, ps, wpb, dist,
+        lambda: host.mgg_SAG_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, 0, ps, wpb2, dist2,
                                     row_scale_out=d_s),
         lambda: host.softmax_forward(d_P, d_H2, V, out_dim, ld_in=ldo),
     ]
@@ -159,7 +179,7 @@ def bench_gcn2(args, torch, host):
     achieved = dom_bytes / (avg[dom] * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "k_agg (%s, dim %d)" % (dom, out_dim if dom == "agg2" else hidden),
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": load_traffic("gcn2_" + dom, args),
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("gcn2_" + dom, args),
                 "algorithmic_bytes": dom_bytes, "avg_launch_ms": round(avg[dom], 4)}
     extra = {
         "stage_ms": {k: round(v, 4) for k, v in avg.items()},
@@ -178,9 +198,9 @@ def bench_gcn2(args, torch, host):
     d_W2u = torch.from_numpy(W2).to(dev)
     alt = [
         lambda: host.dense_forward(d_Y1, d_X, d_W1, V, in_dim, hidden, row_scale=d_s),
-        lambda: host.mgg_SAG_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, ps, wpb, dist,
+        lambda: host.mgg_SAG_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, ps, wpb1, dist1,
                                     row_scale_out=d_s2),
-        lambda: host.mgg_SAG_np_div(d_G, d_H1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, ps, wpb, dist,
+        lambda: host.mgg_SAG_np_div(d_G, d_H1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, ps, wpb1, dist1,
                                     row_scale_out=d_s),
         lambda: host.dense_forward(d_Y2b, d_G, d_W2u, V, hidden, out_dim),
         lambda: host.softmax_forward(d_P2, d_Y2b, V, out_dim),
@@ -221,7 +241,8 @@ def bench_gcn2(args, torch, host):
         "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: 2-layer GCN forward, RMAT(a=.57,b=.19,c=.19) V=%d nnz=%d (self loops, sym-norm), "
-                               "602->16->41 fp32, ps=%d wpb=%d dist=%d" % (V, nnz, ps, wpb, dist)},
+                               "602->16->41 fp32, ps=%d, (wpb, dist) = (%d, %d) at width 16 and (%d, %d) at width 41"
+                               % (V, nnz, ps, wpb1, dist1, wpb2, dist2)},
         "roofline": roofline, "cpu_baseline": cpu, "parity": parity, "detail": extra,
     }
 
@@ -229,7 +250,7 @@ def bench_gcn2(args, torch, host):
 def bench_share(args, torch, host):
     """Aggregation alone on rank 0's share of an 8-way partitioned RMAT graph, remote rows pre-staged."""
     scale, V, draws, dim, num_gpus = 22, 4_194_304, 52_000_000 * args.share_density, 16, 8
-    ps, wpb, dist = args.ps, args.wpb, args.dist
+    ps = args.ps
     npp, lb, ub = host.range_partition(V, num_gpus, 0)
     t0 = time.time()
     ptr, col = host.gen_rmat(scale, V, draws, seed=7, scramble=True, row_lo=lb, row_hi=ub)
@@ -243,6 +264,7 @@ def bench_share(args, torch, host):
     d_xl = torch.from_numpy(np.ascontiguousarray(x_remote[lb:ub])).to(dev)  # separate allocation
     d = [torch.from_numpy(a).to(dev) if len(a) else torch.zeros(1, dtype=torch.int32, device=dev) for a in (lp, lc, rp, rc)]
     d_out = torch.empty(R, dim, device=dev)
+    wpb, dist = pick_knobs(args, lambda: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, ps, input_remote=d_xr))
 
     def call():
         host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, ps, wpb, dist, input_remote=d_xr)
@@ -277,7 +299,7 @@ def bench_share(args, torch, host):
                                "fp32 dim %d, ps=%d wpb=%d dist=%d" % (V, R, nnz, len(lc), len(rc), dim, ps, wpb, dist)},
         "roofline": {"bound": "hbm", "kernel": "k_agg (dim 16, local+remote)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": load_traffic("share_agg", args), "algorithmic_bytes": nbytes, "avg_launch_ms": round(ms, 4)},
+                     **load_traffic("share_agg", args), "algorithmic_bytes": nbytes, "avg_launch_ms": round(ms, 4)},
         "cpu_baseline": cpu,
     }
 
@@ -288,7 +310,7 @@ def bench_gin(args, torch, host):
     has one dense per GIN layer and eps = 0.5; the benchmark configuration asks for the 2-layer MLP and eps = 0.)"""
     V, scale, draws = 2_450_000, 22, 64_000_000
     in_dim, hidden, out_dim, L, eps = 100, 64, 47, 5, 0.0
-    ps, wpb, dist = args.ps, args.wpb, args.dist
+    ps = args.ps
     if args.small:
         V, scale, draws = 50_000, 16, 1_300_000
     t0 = time.time()
@@ -312,6 +334,8 @@ def bench_gin(args, torch, host):
     d_logits = torch.empty(V, out_dim, device=dev)
     d_P = torch.empty(V, out_dim, device=dev)
 
+    d_Y.zero_()
+    wpb, dist = pick_knobs(args, lambda: host.tune_np_div(d_H, d_Y, d_ptr, d_col, zp, zc, 0, V, hidden, V, ps, gin_eps=eps))
     stages, names = [lambda: host.dense_forward(d_Y, d_X, d_W0, V, in_dim, hidden)], ["dense0"]
     for l in range(L):
         last = l == L - 1
@@ -368,7 +392,7 @@ def bench_gin(args, torch, host):
         "config": {"workload": "configs[2]: 5-layer GIN forward, RMAT V=%d nnz=%d, 100->64->47, 2-layer MLP per layer, eps=0, "
                                "ps=%d wpb=%d dist=%d" % (V, nnz, ps, wpb, dist)},
         "roofline": {"bound": "hbm", "kernel": "k_agg (GIN, dim 64)", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("gin_agg", args),
                      "algorithmic_bytes": nbytes, "avg_launch_ms": round(agg_ms, 4)},
         "cpu_baseline": cpu, "parity": parity,
         "detail": {"stage_ms": {k: round(v, 4) for k, v in avg.items()}, "mlp_total_ms": round(mlp_ms, 4)},
@@ -381,7 +405,7 @@ def bench_big(args, torch, host):
     then the 128x128 update on the bf16 matrix cores.  --big-scale shrinks every size by 2^k for a quicker run."""
     k = args.big_scale
     scale, V, draws, dim, num_gpus = 27 - k, 111_000_000 >> k, 790_000_000 >> k, 128, 8
-    ps, wpb, dist = args.ps, args.wpb, args.dist
+    ps = args.ps
     npp, lb, ub = host.range_partition(V, num_gpus, 0)
     t0 = time.time()
     ptr, col = host.gen_rmat(scale, V, draws, seed=5, scramble=True, row_lo=lb, row_hi=ub)
@@ -398,6 +422,7 @@ def bench_big(args, torch, host):
     W = host.glorot(dim, dim, seed=6)
     d_W = torch.from_numpy(W).to(dev).to(torch.bfloat16)
     d_next = torch.empty(R, dim, device=dev, dtype=torch.bfloat16)
+    wpb, dist = pick_knobs(args, lambda: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, ps, input_remote=d_xr))
     stages = [
         lambda: host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, ps, wpb, dist, input_remote=d_xr),
         lambda: host.dense_forward_bf16(d_next, d_out, d_W, R, dim, dim),
@@ -457,7 +482,7 @@ def bench_big(args, torch, host):
                                "bf16 dim %d, fp32 accumulate, then %dx%d bf16 MFMA update; ps=%d wpb=%d dist=%d"
                                % (k, V, R, nnz, len(lc), len(rc), dim, dim, dim, ps, wpb, dist)},
         "roofline": {"bound": "hbm", "kernel": "k_agg (bf16 dim 128, local+remote)", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("big_agg", args),
                      "algorithmic_bytes": nbytes, "avg_launch_ms": round(avg["agg"], 4)},
         "cpu_baseline": cpu, "parity": parity,
         "detail": {"stage_ms": {k2: round(v, 4) for k2, v in avg.items()},
@@ -492,9 +517,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="gcn2", choices=["gcn2", "share", "gin", "big", "copy"])
     ap.add_argument("--ps", type=int, default=16)
-    ap.add_argument("--wpb", type=int, default=8)
-    ap.add_argument("--dist", type=int, default=0, help="interleaved_dist; 0 = let the library choose it per call from the partitions per row (comes to 16 and 4 "
-                         "for the two GCN aggregations, 1 for the share and the sparse graphs)")
+    ap.add_argument("--wpb", type=int, default=0, help="wavefronts per workgroup; 0 = let the library choose")
+    ap.add_argument("--dist", type=int, default=0, help="interleaved_dist; 0 = let the library choose.  With --wpb 0 --dist 0 (the default) the "
+                         "library's search picks the pair once per aggregation shape before the timed region")
+    ap.add_argument("--no-tune", action="store_true", help="with --wpb 0 --dist 0: use the library's rule of thumb instead of its search")
     ap.add_argument("--share-density", type=int, default=1, help="multiplies the number of RMAT draws of --workload share")
     ap.add_argument("--small", action="store_true", help="tiny graph, for a quick functional run")
     ap.add_argument("--big-scale", type=int, default=0, help="--workload big: divide every size by 2^k")

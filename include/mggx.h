@@ -181,6 +181,17 @@ int mggx_sag_np_div(float *d_out, const void *d_in_local, const void *d_in_remot
                     int lb, int ub, int dim, int nodes_per_pe,
                     int ps, int wpb, int dist, const mggx_agg_opts *opts);
 
+/* The design-space search of bench_MGG_DSE_dist_ps.py:12-42 / bench_MGG_DSE_dist_wpb.py (one process launch per
+ * setting there) as one call: runs the aggregation of mggx_sag_np_div with wpb in {4, 8, 16} x dist in {1, 2, 4, 8, 16}
+ * (three runs each, the faster of the last two counts), returns the fastest pair and its time, and remembers it in
+ * the cached plan, so later mggx_sag_np_div calls on the same CSR arrays with the same dim and in_dtype and
+ * wpb = dist = 0 use it.  d_out holds a valid result afterwards.  Synchronises; not for stream capture.
+ * MGGX_AGG_ACCUMULATE is rejected (the repeated runs would add up).  Any out-pointer may be NULL. */
+int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const void *d_in_remote,
+                         const int *d_ptr_l, const int *d_col_l, const int *d_ptr_r, const int *d_col_r,
+                         int lb, int ub, int dim, int nodes_per_pe, int ps, const mggx_agg_opts *opts,
+                         int *wpb_best, int *dist_best, float *ms_best);
+
 /* SAG_host / SAG_cuda_kernel (include/neighbor_utils.cuh:463-506, 2373-2447) and
  * the local half of SAG_host_fused_interleaved (:593-676, 2598-2688): explicit
  * partition arrays from build_part; out[part2node[p],:] += sum over the

@@ -498,53 +498,35 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
 }
 
 // Rows that cross workgroups: the workgroup where the row starts left a tail entry; every later workgroup up to
-// the one where it ends left a head entry.  Each wavefront scans 64 consecutive workgroup slots (one coalesced
-// header load), then finishes the rows whose tail sits there, `group` of them at a time: lane = (walker, component)
-// with `comp_lanes` = power of two >= dim (<= 64); a walker sums its row's chain of head entries in order, four loads
-// in flight.  Wider rows (dim > 64) use one walker and several components per lane.
+// the one where it ends left a head entry.  A wavefront finishes 64/comp_lanes consecutive workgroup slots at once:
+// lane = (walker, component) with `comp_lanes` = power of two >= dim (<= 64); a walker whose slot holds a tail sums
+// that row's chain of head entries in order, four loads in flight.  Wider rows (dim > 64) use one walker per
+// wavefront and several components per lane.
 __global__ void __launch_bounds__(256) k_agg_fixup(const AggArgs a, int num_wg, int comp_lanes)
 {
     const int lane = lane_id();
-    const long long base = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 64;
-    if (base >= num_wg - 1) return;
-    const long long slot = base + lane;
-    int2 t = make_int2(-1, 0);
-    if (slot < num_wg - 1) t = a.c_hdr[2 * slot + 1];
-    unsigned long long todo = __ballot((t.y & HDR_VALID) != 0);
-    const int group = 64 / comp_lanes;  // rows finished at once
-    const int walker = lane / comp_lanes, c0 = lane % comp_lanes;
-    while (todo) {
-        // the walker-th set bit of `todo` is this walker's slot
-        unsigned long long m = todo;
-        int mine = -1;
-        for (int w = 0; w < group && m; ++w) {
-            const int bit = __ffsll((long long)m) - 1;
-            if (w == walker) mine = bit;
-            m &= m - 1;
+    const int group = 64 / comp_lanes;
+    const long long b = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * group + lane / comp_lanes;
+    if (b >= num_wg - 1) return;
+    const int2 t = a.c_hdr[2 * b + 1];
+    if (!(t.y & HDR_VALID)) return;
+    const int row = t.x;
+    const int n = (a.off[row + 1] - 1) / a.parts_per_wg - (int)b;  // head entries of workgroups b+1 .. b+n
+    for (int c = lane % comp_lanes; c < a.dim; c += comp_lanes) {
+        float total = a.c_val[(size_t)(2 * b + 1) * a.cpad + c];
+        int k = 0;
+        for (; k + 4 <= n; k += 4) {
+            const float v0 = a.c_val[(size_t)(2 * (b + 1 + k)) * a.cpad + c];
+            const float v1 = a.c_val[(size_t)(2 * (b + 2 + k)) * a.cpad + c];
+            const float v2 = a.c_val[(size_t)(2 * (b + 3 + k)) * a.cpad + c];
+            const float v3 = a.c_val[(size_t)(2 * (b + 4 + k)) * a.cpad + c];
+            total += v0;
+            total += v1;
+            total += v2;
+            total += v3;
         }
-        todo = m;
-        const int src = mine >= 0 ? mine : lane;
-        const int row = lane_read(t.x, src);
-        if (mine >= 0) {
-            const long long b = base + mine;
-            const int n = (a.off[row + 1] - 1) / a.parts_per_wg - (int)b;  // head entries of workgroups b+1 .. b+n
-            for (int c = c0; c < a.dim; c += comp_lanes) {
-                float total = a.c_val[(size_t)(2 * b + 1) * a.cpad + c];
-                int k = 0;
-                for (; k + 4 <= n; k += 4) {
-                    const float v0 = a.c_val[(size_t)(2 * (b + 1 + k)) * a.cpad + c];
-                    const float v1 = a.c_val[(size_t)(2 * (b + 2 + k)) * a.cpad + c];
-                    const float v2 = a.c_val[(size_t)(2 * (b + 3 + k)) * a.cpad + c];
-                    const float v3 = a.c_val[(size_t)(2 * (b + 4 + k)) * a.cpad + c];
-                    total += v0;
-                    total += v1;
-                    total += v2;
-                    total += v3;
-                }
-                for (; k < n; ++k) total += a.c_val[(size_t)(2 * (b + 1 + k)) * a.cpad + c];
-                finish_elem(a, row, c, total);
-            }
-        }
+        for (; k < n; ++k) total += a.c_val[(size_t)(2 * (b + 1 + k)) * a.cpad + c];
+        finish_elem(a, row, c, total);
     }
 }
 
@@ -620,6 +602,9 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     // 0 = let the library choose (from sweeps on the benchmark graphs): 8 wavefronts; with few slots per wavefront
     // (wide rows) 16 rounds, so a workgroup still covers a few thousand neighbors; otherwise a workgroup tile of
     // about 8 rows' worth of partitions (most rows then finish inside one workgroup), between 1 and 16 rounds.
+    if (wpb == 0 && dist == 0)
+        for (const Plan::Tuned &t : plan->tuned)
+            if (t.dim == dim && t.dtype == o.in_dtype) { wpb = t.wpb; dist = t.dist; }
     if (wpb == 0) wpb = 8;
     if (dist == 0) {
         if (slots <= 4) {
@@ -710,7 +695,8 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         MGGX_LAUNCH_CHECK("k_agg");
         if (num_wg > 1) {
             const int comp_lanes = dim >= 64 ? 64 : pow2_ceil(dim);
-            const long long fix_blocks = (num_wg - 1 + 255) / 256;
+            const long long fix_slots_per_block = 4 * (64 / comp_lanes);
+            const long long fix_blocks = (num_wg - 1 + fix_slots_per_block - 1) / fix_slots_per_block;
             k_agg_fixup<<<dim3((unsigned)fix_blocks), dim3(256), 0, st.stream>>>(a, (int)num_wg, comp_lanes);
             MGGX_LAUNCH_CHECK("k_agg_fixup");
         }
@@ -747,6 +733,59 @@ MGGX_EXPORT int mggx_sag_np_div(float *d_out, const void *d_in_local, const void
     rc = mggx::plan_get(d_ptr_l, d_ptr_r, d_col_r, ub - lb, ps, &plan);
     if (rc) return rc;
     return mggx::run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, wpb, dist, o);
+}
+
+MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const void *d_in_remote, const int *d_ptr_l,
+                                     const int *d_col_l, const int *d_ptr_r, const int *d_col_r, int lb, int ub, int dim,
+                                     int nodes_per_pe, int ps, const mggx_agg_opts *opts, int *wpb_best, int *dist_best,
+                                     float *ms_best)
+{
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    if (ub < lb || !d_ptr_l) return fail(MGGX_EINVAL, "sag_np_div_tune: bad row range [%d,%d) or NULL row pointers", lb, ub);
+    if (ps < 1) return fail(MGGX_EINVAL, "sag_np_div_tune: ps %d must be positive", ps);
+    if (nodes_per_pe < ub - lb) return fail(MGGX_EINVAL, "sag_np_div_tune: nodes_per_pe %d smaller than the row range", nodes_per_pe);
+    if (ps > (int)mggx::DESC_LEN_MASK) ps = (int)mggx::DESC_LEN_MASK;
+    mggx_agg_opts o{};
+    if (opts) o = *opts;
+    if (o.flags & MGGX_AGG_ACCUMULATE) return fail(MGGX_EINVAL, "sag_np_div_tune: repeated runs would accumulate; clear MGGX_AGG_ACCUMULATE");
+    mggx::Plan *plan = nullptr;
+    rc = mggx::plan_get(d_ptr_l, d_ptr_r, d_col_r, ub - lb, ps, &plan);
+    if (rc) return rc;
+    mggx::State &st = mggx::state();
+    hipEvent_t e0, e1;
+    MGGX_HIP(hipEventCreate(&e0));
+    MGGX_HIP(hipEventCreate(&e1));
+    static const int wpbs[] = {8, 4, 16}, dists[] = {1, 2, 4, 8, 16};
+    float best = -1.f;
+    int bw = 8, bd = 1;
+    rc = mggx::run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, 8, 1, o);  // warm caches and workspace
+    for (int wi = 0; wi < 3 && !rc; ++wi)
+        for (int di = 0; di < 5 && !rc; ++di) {
+            float ms_min = -1.f;
+            for (int rep = 0; rep < 3 && !rc; ++rep) {
+                hipError_t e = hipEventRecord(e0, st.stream);
+                rc = mggx::run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, wpbs[wi], dists[di], o);
+                if (e == hipSuccess) e = hipEventRecord(e1, st.stream);
+                if (e == hipSuccess) e = hipEventSynchronize(e1);
+                float ms = 0.f;
+                if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+                if (e != hipSuccess && !rc) rc = fail(MGGX_EHIP, "sag_np_div_tune: timing failed: %s", hipGetErrorString(e));
+                if (!rc && rep > 0 && (ms_min < 0.f || ms < ms_min)) ms_min = ms;  // the first run of a setting is untimed
+            }
+            if (!rc && (best < 0.f || ms_min < best)) { best = ms_min; bw = wpbs[wi]; bd = dists[di]; }
+        }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc) return rc;
+    bool found = false;
+    for (mggx::Plan::Tuned &t : plan->tuned)
+        if (t.dim == dim && t.dtype == o.in_dtype) { t.wpb = bw; t.dist = bd; found = true; }
+    if (!found) plan->tuned.push_back({dim, o.in_dtype, bw, bd});
+    if (wpb_best) *wpb_best = bw;
+    if (dist_best) *dist_best = bd;
+    if (ms_best) *ms_best = best;
+    return MGGX_OK;
 }
 
 MGGX_EXPORT int mggx_sag_parts(float *d_out, const float *d_in, const int *d_row_ptr, const int *d_col,

@@ -53,6 +53,9 @@ struct Plan {
     int num_empty = 0;
     int64_t nnz_l = 0, nnz_r = 0;
     int max_col_r = -1;        // largest remote neighbor id (bounds the remote table)
+    // (wpb, dist) measured best by mggx_sag_np_div_tune for a row width and element type; used when a call passes 0/0
+    struct Tuned { int dim, dtype, wpb, dist; };
+    std::vector<Tuned> tuned;
 };
 
 struct State {

@@ -45,7 +45,7 @@ EXPORTS = [
     "mggx_timer_create", "mggx_timer_start", "mggx_timer_stop", "mggx_timer_elapsed_ms", "mggx_timer_destroy",
     "mggx_release_cached", "mggx_range_partition", "mggx_split_csr", "mggx_build_part", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
-    "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_parts", "mggx_spmm",
+    "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_spmm",
     "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
 ]
 
@@ -286,6 +286,28 @@ def _agg(out, in_local, in_remote, ptr_l, col_l, ptr_r, col_r, lb, ub, dim, npp,
     _pin(ptr_l, ptr_r)
     _check(lib().mggx_sag_np_div(_dptr(out), _dptr(in_local), _dptr(in_remote), _dptr(ptr_l), _dptr(col_l),
                                  _dptr(ptr_r), _dptr(col_r), lb, ub, dim, npp, ps, wpb, dist, C.byref(o)))
+
+
+def tune_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb, ub, dim, nodePerPE,
+                np_size, *, input_remote=None, gin_eps=None, ld_in=0, ld_out=0, row_scale_out=None, relu=False):
+    """The search of the reference's bench_MGG_DSE_dist_ps.py / bench_MGG_DSE_dist_wpb.py in one call: times
+    warpPerBlock x interleaved_dist on this input, returns (warpPerBlock, interleaved_dist, ms) of the fastest and
+    makes later calls with warpPerBlock = interleaved_dist = 0 on the same CSR tensors use it."""
+    import torch
+    o = _AggOpts()
+    o.flags = (AGG_RELU if relu else 0) | (AGG_GIN if gin_eps is not None else 0)
+    o.eps = float(gin_eps or 0.0)
+    o.ld_in = ld_in
+    o.ld_out = ld_out
+    o.d_row_scale_out = row_scale_out.data_ptr() if row_scale_out is not None else None
+    o.in_dtype = BF16 if input.dtype == torch.bfloat16 else F32
+    _pin(row_pointers_l, row_pointers_r)
+    w, d, ms = C.c_int(), C.c_int(), C.c_float()
+    rem = input_remote if input_remote is not None else input
+    _check(lib().mggx_sag_np_div_tune(_dptr(output), _dptr(input), _dptr(rem), _dptr(row_pointers_l), _dptr(column_index_l),
+                                      _dptr(row_pointers_r), _dptr(column_index_r), lb, ub, dim, nodePerPE, np_size,
+                                      C.byref(o), C.byref(w), C.byref(d), C.byref(ms)))
+    return w.value, d.value, ms.value
 
 
 def mgg_SAG_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb, ub, dim,

@@ -141,6 +141,44 @@ def test_library_chosen_knobs(gpu, rmat_graph, dim):
     assert_close_to_oracle(got, want, mag, FP32_TOL, "auto knobs")
 
 
+@pytest.mark.parametrize("dim,gin", [(16, False), (64, True), (41, False)])
+def test_search_of_wpb_and_dist(gpu, rmat_graph, dim, gin):
+    """The one-call search over wpb x dist: leaves a correct result in the output, returns a pair from its grid, and
+    a later call with wpb = dist = 0 on the same CSR tensors runs with that pair (bit-identical to naming it)."""
+    import torch
+    V, ptr, col = rmat_graph
+    x = gpu.fill_normal((V, dim), seed=78)
+    sh = share_of(ptr, col, V, 2, 0)
+    xl = np.ascontiguousarray(x[sh["lb"]:sh["ub"]])
+    R = sh["ub"] - sh["lb"]
+    d = [to_dev(sh[k]) if len(sh[k]) else torch.zeros(1, dtype=torch.int32, device="cuda") for k in ("ptr_l", "col_l", "ptr_r", "col_r")]
+    d_xl, d_x = to_dev(xl), to_dev(x)
+    out = torch.full((R, dim), 7.5, device="cuda")
+    wpb, dist, ms = gpu.tune_np_div(out, d_xl, d[0], d[1], d[2], d[3], sh["lb"], sh["ub"], dim, sh["npp"], 16, input_remote=d_x,
+                                    gin_eps=0.25 if gin else None)
+    assert wpb in (4, 8, 16) and dist in (1, 2, 4, 8, 16) and ms > 0
+    kw = dict(flags=orc.GIN, eps=0.25) if gin else {}
+    want, mag = oracle_agg(sh, xl, x, dim, **kw)
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "result left by the search")
+    call = (lambda o, w, t: gpu.mgg_GIN_np_div(o, d_xl, d[0], d[1], d[2], d[3], sh["lb"], sh["ub"], dim, sh["npp"], 0, 16, w, t, 0.25,
+                                                input_remote=d_x)) if gin else \
+           (lambda o, w, t: gpu.mgg_SAG_np_div(o, d_xl, d[0], d[1], d[2], d[3], sh["lb"], sh["ub"], dim, sh["npp"], 0, 16, w, t,
+                                                input_remote=d_x))
+    auto, named = torch.empty_like(out), torch.empty_like(out)
+    call(auto, 0, 0)
+    assert "block=%d" % (64 * wpb) in gpu.last_agg_kernel()
+    call(named, wpb, dist)
+    gpu.sync()
+    assert torch.equal(auto, named)
+    with pytest.raises(gpu.MggxError):  # repeated runs would add up
+        o = gpu._AggOpts()
+        o.flags = gpu.AGG_ACCUMULATE
+        import ctypes as C
+        gpu._check(gpu.lib().mggx_sag_np_div_tune(gpu._dptr(out), gpu._dptr(d_xl), gpu._dptr(d_x), gpu._dptr(d[0]), gpu._dptr(d[1]),
+                                                  gpu._dptr(d[2]), gpu._dptr(d[3]), sh["lb"], sh["ub"], dim, sh["npp"], 16,
+                                                  C.byref(o), None, None, None))
+
+
 def test_bad_arguments_return_errors_not_faults(gpu, rmat_graph):
     """Shapes the kernels are not built for are refused on the host, with a message, before any launch."""
     import torch
