@@ -224,6 +224,21 @@ typedef struct mggx_dense_opts {
 int mggx_dense_xw(float *d_out, const float *d_x, const float *d_w, int64_t n, int d1, int d2,
                   const mggx_dense_opts *opts);
 
+typedef struct mggx_mlp2_opts {
+    int64_t ld_x;                /* 0 = d1 */
+    int64_t ld_out;              /* 0 = d3 */
+    const float *d_row_scale;    /* [n] multiplies each output row (NULL = 1) */
+    uint32_t relu_mid;           /* max(0,.) between the two products */
+    uint32_t relu_out;           /* max(0,.) on the output */
+} mggx_mlp2_opts;
+
+/* Two consecutive updates in one pass, Out[n x d3] = act(X[n x d1] . Wa[d1 x h]) . Wb[h x d3], fp32 on MFMA: what two
+ * dense_hidden_forward calls (include/gnn_layer.cuh:28-33) compute, without writing and re-reading the n x h
+ * intermediate (a GIN layer's 2-layer MLP).  h <= 64, d3 <= 64 and both matrices must fit in LDS; otherwise
+ * MGGX_ELIMIT is returned and the caller issues two mggx_dense_xw calls. */
+int mggx_mlp2_xw(float *d_out, const float *d_x, const float *d_wa, const float *d_wb, int64_t n, int d1, int h, int d3,
+                 const mggx_mlp2_opts *opts);
+
 /* The same update on the bf16 matrix cores (no counterpart in the reference, which is fp32 only): W is bf16
  * [d1 x d2]; X is fp32 (rounded to bf16, nearest even, inside the kernel) or bf16 (x_dtype); products are
  * accumulated in fp32; Out is fp32 or bf16 (out_dtype).  Strides are in elements of the respective type. */

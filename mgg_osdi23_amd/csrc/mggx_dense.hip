@@ -22,6 +22,7 @@ struct DenseArgs {
     long long ld_x, ld_out;
     int d1, d2;
     int relu;
+    int vec_out;  // rows of out may be written 4 elements at a time (alignment and stride allow it)
 };
 
 // v_mfma_f32_16x16x4_f32 operand layout (wave64):
@@ -45,6 +46,35 @@ __device__ __forceinline__ void load_x4(float (&xv)[4], const float *xrow, int k
     }
 }
 
+// Branch-free form for the resident kernels.  `xrow` is a valid row (callers clamp the row index; results of rows
+// past the end are never stored).  `mode` is the same for the whole wavefront:
+//   0  the 64-wide K group lies inside the row: plain 16-byte loads
+//   1  d1 % 4 == 0: a lane's 4 values are all inside or all outside; load from a clamped offset, zero if outside
+//   2  any d1: four dword loads from clamped offsets, zeroed one by one
+__device__ __forceinline__ void load_x4u(float (&xv)[4], const float *xrow, int kb, int d1, int mode)
+{
+    if (mode == 0) {
+        float4 t4;
+        __builtin_memcpy(&t4, xrow + kb, 16);
+        xv[0] = t4.x; xv[1] = t4.y; xv[2] = t4.z; xv[3] = t4.w;
+    } else if (mode == 1) {
+        float4 t4;
+        __builtin_memcpy(&t4, xrow + min(kb, d1 - 4), 16);
+        const bool in = kb < d1;
+        xv[0] = in ? t4.x : 0.f; xv[1] = in ? t4.y : 0.f; xv[2] = in ? t4.z : 0.f; xv[3] = in ? t4.w : 0.f;
+    } else {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float v = xrow[min(kb + t, d1 - 1)];
+            xv[t] = kb + t < d1 ? v : 0.f;
+        }
+    }
+}
+__device__ __forceinline__ int x_group_mode(int k_first, int width, int d1, int chunk)
+{
+    return k_first + width <= d1 ? 0 : (d1 % chunk == 0 ? 1 : 2);
+}
+
 template <int NB>
 __device__ __forceinline__ void store_tile_f32(const DenseArgs &a, const v4f (&acc)[NB], long long row_base, int c0, int i)
 {
@@ -66,11 +96,103 @@ __device__ __forceinline__ void store_tile_f32(const DenseArgs &a, const v4f (&a
     }
 }
 
-// W kept whole in LDS (zero padded to a multiple of 64 rows); the 8 wavefronts of a workgroup walk over 16-row
-// tiles of X.  X is read four 16-wide K steps at a time, one group ahead of the matrix cores.
+// The resident kernels form every product transposed -- W as the A operand, X as the B operand (both operand layouts
+// give lane L the element (L % 16, L / 16), so the loads are the same) -- which leaves lane L with
+// D[row L % 16][16 nb + 4 (L / 16) + r], r = 0..3: four consecutive columns of one output row, one 16-byte store.
+template <int NB, bool OUT_BF16>
+__device__ __forceinline__ void store_rows(void *out, long long ld_out, int d2, float scale, int relu, int vec_out,
+                                           const v4f (&acc)[NB], long long row, bool row_ok, int c0, int kq)
+{
+    if (!row_ok) return;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int c = c0 + nb * 16 + 4 * kq;
+        if (c >= d2) continue;
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            v[r] = acc[nb][r] * scale;
+            if (relu) v[r] = fmaxf(v[r], 0.f);
+        }
+        if constexpr (OUT_BF16) {
+            __bf16 *o = static_cast<__bf16 *>(out) + row * ld_out + c;
+            const v2bf p0 = __builtin_convertvector((v2f){v[0], v[1]}, v2bf);
+            const v2bf p1 = __builtin_convertvector((v2f){v[2], v[3]}, v2bf);
+            if (vec_out && c + 3 < d2) {
+                const __bf16 q[4] = {p0[0], p0[1], p1[0], p1[1]};
+                __builtin_memcpy(__builtin_assume_aligned(o, 8), q, 8);
+            } else {
+                o[0] = p0[0];
+                if (c + 1 < d2) o[1] = p0[1];
+                if (c + 2 < d2) o[2] = p1[0];
+                if (c + 3 < d2) o[3] = p1[1];
+            }
+        } else {
+            float *o = static_cast<float *>(out) + row * ld_out + c;
+            if (vec_out && c + 3 < d2) {
+                *reinterpret_cast<float4 *>(o) = make_float4(v[0], v[1], v[2], v[3]);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (c + r < d2) o[r] = v[r];
+            }
+        }
+    }
+}
+
+// W kept whole in LDS; the 8 wavefronts of a workgroup walk over 16-row tiles of X.  K is cut into groups of 64.
+// FULL (d1 >= 64): every group is a whole 64 wide -- the last one is shifted back to [d1 - 64, d1) and the W rows
+// it shares with the group before are zero in LDS, so every X load is a plain in-row 16-byte load with no tail
+// handling.  !FULL (d1 < 64): one group, loads clamped and masked.  X is read one group ahead of the matrix cores;
+// the group after the last one of a tile is the first one of the wavefront's next tile.
 constexpr int RES_THREADS = 512;
-template <int NB>
-__global__ void __launch_bounds__(RES_THREADS) k_dense_xw_resident(const DenseArgs a)
+
+// K index held by LDS row r (-1: a zero row)
+template <bool FULL>
+__device__ __forceinline__ int lds_row_k(int r, int ngroups, int d1)
+{
+    if constexpr (FULL) {
+        const int g = r >> 6;
+        if (g < ngroups - 1) return r;
+        const int k = d1 - 64 + (r & 63);
+        return k >= 64 * g ? k : -1;
+    } else {
+        return r < d1 ? r : -1;
+    }
+}
+
+template <bool FULL>
+__device__ __forceinline__ void load_group(float (&x)[4][4], const float *xrow, int g, int ngroups, int d1, int kq)
+{
+    if constexpr (FULL) {
+        const int ks = (g == ngroups - 1 ? d1 - 64 : 64 * g) + 4 * kq;
+#pragma unroll
+        for (int gg = 0; gg < 4; ++gg) load_x4u(x[gg], xrow, ks + 16 * gg, d1, 0);
+    } else {
+        const int mode = d1 % 4 == 0 ? 1 : 2;
+#pragma unroll
+        for (int gg = 0; gg < 4; ++gg) load_x4u(x[gg], xrow, 16 * gg + 4 * kq, d1, mode);
+    }
+}
+
+// acc[nb] += Wt-block^T . X-group, transposed product (see store_rows)
+template <int NB, int RS>
+__device__ __forceinline__ void mfma_group(v4f (&acc)[NB], const float *wt_group, const float (&x)[4][4], int i, int kq)
+{
+#pragma unroll
+    for (int gg = 0; gg < 4; ++gg) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float *wrow = wt_group + (16 * gg + 4 * kq + t) * RS + i;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(wrow[nb * 16], x[gg][t], acc[nb], 0, 0, 0);
+        }
+    }
+}
+
+template <int NB, bool FULL>
+__global__ void __launch_bounds__(RES_THREADS, 4) k_dense_xw_resident(const DenseArgs a)
 {
     constexpr int RS = NB * 16 + 4;  // LDS row stride in floats; the +4 keeps the four K groups on distinct banks
     constexpr int WAVES = RES_THREADS / 64;
@@ -79,46 +201,152 @@ __global__ void __launch_bounds__(RES_THREADS) k_dense_xw_resident(const DenseAr
     const int wave = (int)(threadIdx.x >> 6);
     const int i = lane & 15, kq = lane >> 4;
     const int c0 = (int)blockIdx.y * (NB * 16);
-    const int d1p = (a.d1 + 63) & ~63;
+    const int ngroups = (a.d1 + 63) >> 6;
     const float *w = static_cast<const float *>(a.w);
-    for (int idx = (int)threadIdx.x; idx < d1p * NB * 16; idx += RES_THREADS) {
-        const int k = idx / (NB * 16), j = idx % (NB * 16);
-        wt[k * RS + j] = (k < a.d1 && c0 + j < a.d2) ? w[(long long)k * a.d2 + c0 + j] : 0.f;
+    for (int idx = (int)threadIdx.x; idx < ngroups * 64 * NB * 16; idx += RES_THREADS) {
+        const int r = idx / (NB * 16), j = idx % (NB * 16);
+        const int k = lds_row_k<FULL>(r, ngroups, a.d1);
+        wt[r * RS + j] = (k >= 0 && c0 + j < a.d2) ? w[(long long)k * a.d2 + c0 + j] : 0.f;
+    }
+    __syncthreads();
+
+    // One flat loop over (tile, K group): the loads of the next item are issued first and may not sink below the
+    // scheduling barrier, so they fly while the matrix cores work on the current item.
+    const long long tiles = (a.n + 15) / 16;
+    const long long stride = (long long)gridDim.x * WAVES;
+    long long tile = (long long)blockIdx.x * WAVES + wave;
+    if (tile >= tiles) return;
+    const float *x = static_cast<const float *>(a.x);
+    float xv[4][4], xn[4][4];
+    float scale = 1.0f, scale_next = 1.0f;
+    {
+        const long long row = min(tile * 16 + i, a.n - 1);
+        load_group<FULL>(xv, x + row * a.ld_x, 0, ngroups, a.d1, kq);
+        if (a.rs) scale = a.rs[row];
+    }
+    v4f acc[NB];
+    int g = 0;
+    for (;;) {
+        const bool last_g = g + 1 == ngroups;
+        const long long ntile = last_g ? tile + stride : tile;
+        const int ng = last_g ? 0 : g + 1;
+        {
+            const long long nrow = min(ntile * 16 + i, a.n - 1);
+            load_group<FULL>(xn, x + nrow * a.ld_x, ng, ngroups, a.d1, kq);
+            scale_next = scale;
+            if (last_g && a.rs) scale_next = a.rs[nrow];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (g == 0) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) acc[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
+        }
+        mfma_group<NB, RS>(acc, wt + g * 64 * RS, xv, i, kq);
+        if (last_g) {
+            const long long row = tile * 16 + i;
+            store_rows<NB, false>(a.out, a.ld_out, a.d2, scale, a.relu, a.vec_out, acc, row, row < a.n, c0, kq);
+        }
+#pragma unroll
+        for (int gg = 0; gg < 4; ++gg)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) xv[gg][t] = xn[gg][t];
+        scale = scale_next;
+        tile = ntile;
+        g = ng;
+        if (tile >= tiles) break;
+    }
+}
+
+// Two updates in one pass, Out = act(X . Wa) . Wb, both weight matrices resident in LDS (h <= 64, d3 <= 64).
+// The transposed first product leaves lane L with T[row L % 16][16 nb + 4 (L / 16) + r], r = 0..3: four consecutive
+// K values of one row of the intermediate, which is exactly the operand the second product wants.  The
+// intermediate never leaves the registers.
+struct MlpArgs {
+    float *out;
+    const float *x, *wa, *wb, *rs;
+    long long n, ld_x, ld_out;
+    int d1, h, d3;
+    int relu_mid, relu_out, vec_out;
+};
+
+template <int NB1, int NB2, bool FULL>
+__global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_resident(const MlpArgs a)
+{
+    constexpr int RS1 = NB1 * 16 + 4, RS2 = NB2 * 16 + 4;
+    constexpr int WAVES = RES_THREADS / 64;
+    extern __shared__ float wt[];
+    const int lane = (int)(threadIdx.x & 63u);
+    const int wave = (int)(threadIdx.x >> 6);
+    const int i = lane & 15, kq = lane >> 4;
+    const int ngroups = (a.d1 + 63) >> 6;
+    float *wta = wt, *wtb = wt + ngroups * 64 * RS1;
+    for (int idx = (int)threadIdx.x; idx < ngroups * 64 * NB1 * 16; idx += RES_THREADS) {
+        const int r = idx / (NB1 * 16), j = idx % (NB1 * 16);
+        const int k = lds_row_k<FULL>(r, ngroups, a.d1);
+        wta[r * RS1 + j] = (k >= 0 && j < a.h) ? a.wa[(long long)k * a.h + j] : 0.f;
+    }
+    for (int idx = (int)threadIdx.x; idx < NB1 * 16 * NB2 * 16; idx += RES_THREADS) {
+        const int k = idx / (NB2 * 16), j = idx % (NB2 * 16);
+        wtb[k * RS2 + j] = (k < a.h && j < a.d3) ? a.wb[(long long)k * a.d3 + j] : 0.f;
     }
     __syncthreads();
 
     const long long tiles = (a.n + 15) / 16;
-    for (long long tile = (long long)blockIdx.x * WAVES + wave; tile < tiles; tile += (long long)gridDim.x * WAVES) {
-        const long long row = tile * 16 + i;
-        const bool row_ok = row < a.n;
-        const float *xrow = static_cast<const float *>(a.x) + (row_ok ? row : 0) * a.ld_x;
-        v4f acc[NB];
+    const long long stride = (long long)gridDim.x * WAVES;
+    long long tile = (long long)blockIdx.x * WAVES + wave;
+    if (tile >= tiles) return;
+    float xv[4][4], xn[4][4];
+    float scale = 1.0f, scale_next = 1.0f;
+    {
+        const long long row = min(tile * 16 + i, a.n - 1);
+        load_group<FULL>(xv, a.x + row * a.ld_x, 0, ngroups, a.d1, kq);
+        if (a.rs) scale = a.rs[row];
+    }
+    v4f acc1[NB1];
+    int g = 0;
+    for (;;) {
+        const bool last_g = g + 1 == ngroups;
+        const long long ntile = last_g ? tile + stride : tile;
+        const int ng = last_g ? 0 : g + 1;
+        {
+            const long long nrow = min(ntile * 16 + i, a.n - 1);
+            load_group<FULL>(xn, a.x + nrow * a.ld_x, ng, ngroups, a.d1, kq);
+            scale_next = scale;
+            if (last_g && a.rs) scale_next = a.rs[nrow];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (g == 0) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) acc[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
-        float xv[4][4], xn[4][4];
+            for (int nb = 0; nb < NB1; ++nb) acc1[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
+        }
+        mfma_group<NB1, RS1>(acc1, wta + g * 64 * RS1, xv, i, kq);
+        if (last_g) {
+            v4f acc2[NB2];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) load_x4(xv[g], xrow, 16 * g + 4 * kq, a.d1, row_ok);
-        for (int k0 = 0; k0 < d1p; k0 += 64) {
-            if (k0 + 64 < d1p) {
+            for (int nb = 0; nb < NB2; ++nb) acc2[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int g = 0; g < 4; ++g) load_x4(xn[g], xrow, k0 + 64 + 16 * g + 4 * kq, a.d1, row_ok);
-            }
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
+            for (int nb = 0; nb < NB1; ++nb) {
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    const float *wrow = wt + (k0 + 16 * g + 4 * kq + t) * RS + i;
+                    float tv = acc1[nb][t];
+                    if (a.relu_mid) tv = fmaxf(tv, 0.f);
+                    const float *wrow = wtb + (16 * nb + 4 * kq + t) * RS2 + i;
 #pragma unroll
-                    for (int nb = 0; nb < NB; ++nb)
-                        acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[g][t], wrow[nb * 16], acc[nb], 0, 0, 0);
+                    for (int nb2 = 0; nb2 < NB2; ++nb2)
+                        acc2[nb2] = __builtin_amdgcn_mfma_f32_16x16x4f32(wrow[nb2 * 16], tv, acc2[nb2], 0, 0, 0);
                 }
             }
-#pragma unroll
-            for (int g = 0; g < 4; ++g)
-#pragma unroll
-                for (int t = 0; t < 4; ++t) xv[g][t] = xn[g][t];
+            const long long row = tile * 16 + i;
+            store_rows<NB2, false>(a.out, a.ld_out, a.d3, scale, a.relu_out, a.vec_out, acc2, row, row < a.n, 0, kq);
         }
-        store_tile_f32<NB>(a, acc, tile * 16 + 4 * kq, c0, i);
+#pragma unroll
+        for (int gg = 0; gg < 4; ++gg)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) xv[gg][t] = xn[gg][t];
+        scale = scale_next;
+        tile = ntile;
+        g = ng;
+        if (tile >= tiles) break;
     }
 }
 
@@ -173,6 +401,63 @@ __global__ void __launch_bounds__(256) k_dense_xw(const DenseArgs a)
 // W (bf16, [d1][d2]) is kept transposed in LDS, Wt[column][k], so a lane's 8 K values are one 16-byte read.
 // X is fp32 (rounded to bf16, nearest even, on the fly) or bf16; the accumulator and the epilogue are fp32; the
 // output is fp32 or bf16.
+// 8 consecutive K values of one row as bf16, branch-free; `mode` as in load_x4u with chunks of 8 (wavefront-uniform).
+template <bool X_F32>
+__device__ __forceinline__ v8bf load_x8_bf16(const void *xbase, long long row, long long ld_x, int k, int d1, int mode)
+{
+    v8bf av;
+    if constexpr (X_F32) {
+        const float *xrow = static_cast<const float *>(xbase) + row * ld_x;
+        float f[8];
+        if (mode <= 1) {
+            const int kc = mode == 0 ? k : min(k, d1 - 8);
+            float4 t0, t1;
+            __builtin_memcpy(&t0, xrow + kc, 16);
+            __builtin_memcpy(&t1, xrow + kc + 4, 16);
+            f[0] = t0.x; f[1] = t0.y; f[2] = t0.z; f[3] = t0.w;
+            f[4] = t1.x; f[5] = t1.y; f[6] = t1.z; f[7] = t1.w;
+            if (mode == 1) {
+                const bool in = k < d1;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) f[t] = in ? f[t] : 0.f;
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const float v = xrow[min(k + t, d1 - 1)];
+                f[t] = k + t < d1 ? v : 0.f;
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const v2bf p = __builtin_convertvector((v2f){f[2 * t], f[2 * t + 1]}, v2bf);
+            av[2 * t] = p[0];
+            av[2 * t + 1] = p[1];
+        }
+    } else {
+        const unsigned short *xrow = static_cast<const unsigned short *>(xbase) + row * ld_x;
+        unsigned short h[8];
+        if (mode <= 1) {
+            __builtin_memcpy(h, xrow + (mode == 0 ? k : min(k, d1 - 8)), 16);
+            if (mode == 1) {
+                const bool in = k < d1;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) h[t] = in ? h[t] : (unsigned short)0;
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const unsigned short v = xrow[min(k + t, d1 - 1)];
+                h[t] = k + t < d1 ? v : (unsigned short)0;
+            }
+        }
+        __builtin_memcpy(&av, h, 16);
+    }
+    return av;
+}
+
+// Like the fp32 kernels the product is formed transposed (W as the A operand), so a lane ends up with four
+// consecutive columns of one output row; X is read one K step (32 values per row) ahead, across tile boundaries.
 template <int NB, bool X_F32, bool OUT_BF16>
 __global__ void __launch_bounds__(256) k_dense_xw_bf16(const DenseArgs a)
 {
@@ -193,83 +478,47 @@ __global__ void __launch_bounds__(256) k_dense_xw_bf16(const DenseArgs a)
     __syncthreads();
 
     const long long tiles = (a.n + 15) / 16;
-    for (long long tile = (long long)blockIdx.x * 4 + wave; tile < tiles; tile += (long long)gridDim.x * 4) {
-        const long long row = tile * 16 + i;
-        const bool row_ok = row < a.n;
-        v4f acc[NB];
+    const long long stride = (long long)gridDim.x * 4;
+    long long tile = (long long)blockIdx.x * 4 + wave;
+    if (tile >= tiles) return;
+    float scale = 1.0f, scale_next = 1.0f;
+    v8bf av;
+    {
+        const long long row = min(tile * 16 + i, a.n - 1);
+        av = load_x8_bf16<X_F32>(a.x, row, a.ld_x, 8 * kb, a.d1, x_group_mode(0, 32, a.d1, 8));
+        if (a.rs) scale = a.rs[row];
+    }
+    v4f acc[NB];
+    int k0 = 0;
+    for (;;) {  // flat loop over (tile, K step of 32); the next step's X is in flight during the MFMAs
+        const bool last_k = k0 + 32 >= d1p;
+        const long long ntile = last_k ? tile + stride : tile;
+        const int nk = last_k ? 0 : k0 + 32;
+        const long long nrow = min(ntile * 16 + i, a.n - 1);
+        const v8bf an = load_x8_bf16<X_F32>(a.x, nrow, a.ld_x, nk + 8 * kb, a.d1, x_group_mode(nk, 32, a.d1, 8));
+        scale_next = scale;
+        if (last_k && a.rs) scale_next = a.rs[nrow];
+        __builtin_amdgcn_sched_barrier(0);
+        if (k0 == 0) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) acc[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
-        for (int k0 = 0; k0 < d1p; k0 += 32) {
-            const int k = k0 + 8 * kb;
-            v8bf av;
-            if constexpr (X_F32) {
-                const float *xrow = static_cast<const float *>(a.x) + (row_ok ? row : 0) * a.ld_x;
-                float f[8];
-#pragma unroll
-                for (int t = 0; t < 8; ++t) f[t] = 0.f;
-                if (row_ok) {
-                    if (k + 7 < a.d1) {
-                        float4 t0, t1;
-                        __builtin_memcpy(&t0, xrow + k, 16);
-                        __builtin_memcpy(&t1, xrow + k + 4, 16);
-                        f[0] = t0.x; f[1] = t0.y; f[2] = t0.z; f[3] = t0.w;
-                        f[4] = t1.x; f[5] = t1.y; f[6] = t1.z; f[7] = t1.w;
-                    } else {
-#pragma unroll
-                        for (int t = 0; t < 8; ++t)
-                            if (k + t < a.d1) f[t] = xrow[k + t];
-                    }
-                }
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const v2bf p = __builtin_convertvector((v2f){f[2 * t], f[2 * t + 1]}, v2bf);
-                    av[2 * t] = p[0];
-                    av[2 * t + 1] = p[1];
-                }
-            } else {
-                const unsigned short *xrow = static_cast<const unsigned short *>(a.x) + (row_ok ? row : 0) * a.ld_x;
-                unsigned short h[8];
-#pragma unroll
-                for (int t = 0; t < 8; ++t) h[t] = 0;
-                if (row_ok) {
-                    if (k + 7 < a.d1) {
-                        __builtin_memcpy(h, xrow + k, 16);
-                    } else {
-#pragma unroll
-                        for (int t = 0; t < 8; ++t)
-                            if (k + t < a.d1) h[t] = xrow[k + t];
-                    }
-                }
-                __builtin_memcpy(&av, h, 16);
-            }
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                v8bf bv;
-                __builtin_memcpy(&bv, wt + (size_t)(nb * 16 + i) * KP + k, 16);
-                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, acc[nb], 0, 0, 0);
-            }
+            for (int nb = 0; nb < NB; ++nb) acc[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
         }
-        const long long row_base = tile * 16 + 4 * kb;
+        const int k = k0 + 8 * kb;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const long long orow = row_base + r;
-            if (orow >= a.n) continue;
-            const float scale = a.rs ? a.rs[orow] : 1.0f;
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                const int c = c0 + nb * 16 + i;
-                if (c < a.d2) {
-                    float v = acc[nb][r] * scale;
-                    if (a.relu) v = fmaxf(v, 0.f);
-                    if constexpr (OUT_BF16) {
-                        const v2bf p = __builtin_convertvector((v2f){v, 0.f}, v2bf);
-                        static_cast<__bf16 *>(a.out)[orow * a.ld_out + c] = p[0];
-                    } else {
-                        static_cast<float *>(a.out)[orow * a.ld_out + c] = v;
-                    }
-                }
-            }
+        for (int nb = 0; nb < NB; ++nb) {
+            v8bf bv;
+            __builtin_memcpy(&bv, wt + (size_t)(nb * 16 + i) * KP + k, 16);
+            acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, av, acc[nb], 0, 0, 0);
         }
+        if (last_k) {
+            const long long row = tile * 16 + i;
+            store_rows<NB, OUT_BF16>(a.out, a.ld_out, a.d2, scale, a.relu, a.vec_out, acc, row, row < a.n, c0, kb);
+        }
+        av = an;
+        scale = scale_next;
+        tile = ntile;
+        k0 = nk;
+        if (tile >= tiles) break;
     }
 }
 
@@ -360,8 +609,13 @@ template <int NB>
 struct LaunchResident {
     static void run(dim3 grid, size_t lds, hipStream_t s, const DenseArgs &a)
     {
-        allow_lds(k_dense_xw_resident<NB>, lds);
-        k_dense_xw_resident<NB><<<grid, dim3(RES_THREADS), lds, s>>>(a);
+        if (a.d1 >= 64) {
+            allow_lds(k_dense_xw_resident<NB, true>, lds);
+            k_dense_xw_resident<NB, true><<<grid, dim3(RES_THREADS), lds, s>>>(a);
+        } else {
+            allow_lds(k_dense_xw_resident<NB, false>, lds);
+            k_dense_xw_resident<NB, false><<<grid, dim3(RES_THREADS), lds, s>>>(a);
+        }
     }
 };
 template <int NB>
@@ -415,6 +669,7 @@ MGGX_EXPORT int mggx_dense_xw(float *d_out, const float *d_x, const float *d_w, 
     a.d1 = d1;
     a.d2 = d2;
     a.relu = o.relu != 0;
+    a.vec_out = a.ld_out % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0;
     if (a.ld_x < d1 || a.ld_out < d2) return fail(MGGX_EINVAL, "dense_xw: row stride smaller than width");
     hipStream_t stream = mggx::state().stream;
     const int nb = mggx::pick_nb(d2);
@@ -430,6 +685,76 @@ MGGX_EXPORT int mggx_dense_xw(float *d_out, const float *d_x, const float *d_w, 
         mggx::dispatch_nb<mggx::LaunchChunked>(nb, dim3((unsigned)gx, (unsigned)gy), 0, stream, a);
         MGGX_LAUNCH_CHECK("k_dense_xw");
     }
+    return MGGX_OK;
+}
+
+namespace mggx {
+namespace {
+template <int NB1, int NB2>
+void launch_mlp2(dim3 grid, size_t lds, hipStream_t s, const MlpArgs &a)
+{
+    if (a.d1 >= 64) {
+        allow_lds(k_mlp2_resident<NB1, NB2, true>, lds);
+        k_mlp2_resident<NB1, NB2, true><<<grid, dim3(RES_THREADS), lds, s>>>(a);
+    } else {
+        allow_lds(k_mlp2_resident<NB1, NB2, false>, lds);
+        k_mlp2_resident<NB1, NB2, false><<<grid, dim3(RES_THREADS), lds, s>>>(a);
+    }
+}
+template <int NB1>
+void launch_mlp2_nb2(int nb2, dim3 grid, size_t lds, hipStream_t s, const MlpArgs &a)
+{
+    switch (nb2) {
+        case 1: launch_mlp2<NB1, 1>(grid, lds, s, a); break;
+        case 2: launch_mlp2<NB1, 2>(grid, lds, s, a); break;
+        case 3: launch_mlp2<NB1, 3>(grid, lds, s, a); break;
+        default: launch_mlp2<NB1, 4>(grid, lds, s, a); break;
+    }
+}
+}  // namespace
+}  // namespace mggx
+
+MGGX_EXPORT int mggx_mlp2_xw(float *d_out, const float *d_x, const float *d_wa, const float *d_wb, int64_t n, int d1,
+                             int h, int d3, const mggx_mlp2_opts *opts)
+{
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    if (n < 0 || d1 < 1 || h < 1 || d3 < 1) return fail(MGGX_EINVAL, "mlp2_xw: n=%lld d1=%d h=%d d3=%d", (long long)n, d1, h, d3);
+    if (h > 64 || d3 > 64) return fail(MGGX_ELIMIT, "mlp2_xw: h=%d and d3=%d must be <= 64 (use two mggx_dense_xw calls)", h, d3);
+    if (n == 0) return MGGX_OK;
+    if (!d_out || !d_x || !d_wa || !d_wb) return fail(MGGX_EINVAL, "mlp2_xw: NULL pointer");
+    if (d_out == d_x) return fail(MGGX_EINVAL, "mlp2_xw: in-place update is not supported");
+    mggx_mlp2_opts o{};
+    if (opts) o = *opts;
+    mggx::MlpArgs a{};
+    a.out = d_out;
+    a.x = d_x;
+    a.wa = d_wa;
+    a.wb = d_wb;
+    a.rs = o.d_row_scale;
+    a.n = n;
+    a.ld_x = o.ld_x ? o.ld_x : d1;
+    a.ld_out = o.ld_out ? o.ld_out : d3;
+    a.d1 = d1;
+    a.h = h;
+    a.d3 = d3;
+    a.relu_mid = o.relu_mid != 0;
+    a.relu_out = o.relu_out != 0;
+    a.vec_out = a.ld_out % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0;
+    if (a.ld_x < d1 || a.ld_out < d3) return fail(MGGX_EINVAL, "mlp2_xw: row stride smaller than width");
+    const int nb1 = (h + 15) / 16, nb2 = (d3 + 15) / 16;
+    const size_t lds = ((size_t)((d1 + 63) & ~63) * (nb1 * 16 + 4) + (size_t)nb1 * 16 * (nb2 * 16 + 4)) * sizeof(float);
+    if (lds > mggx::LDS_RESIDENT_LIMIT) return fail(MGGX_ELIMIT, "mlp2_xw: weights of %zu bytes do not fit in LDS (d1 <= ~%d at h = %d)", lds,
+                                                    (int)(mggx::LDS_RESIDENT_LIMIT / 4 / (nb1 * 16 + 4)) - 64, h);
+    const dim3 grid(mggx::persistent_blocks(n));
+    hipStream_t stream = mggx::state().stream;
+    switch (nb1) {
+        case 1: mggx::launch_mlp2_nb2<1>(nb2, grid, lds, stream, a); break;
+        case 2: mggx::launch_mlp2_nb2<2>(nb2, grid, lds, stream, a); break;
+        case 3: mggx::launch_mlp2_nb2<3>(nb2, grid, lds, stream, a); break;
+        default: mggx::launch_mlp2_nb2<4>(nb2, grid, lds, stream, a); break;
+    }
+    MGGX_LAUNCH_CHECK("k_mlp2_resident");
     return MGGX_OK;
 }
 
@@ -457,6 +782,7 @@ MGGX_EXPORT int mggx_dense_xw_bf16(void *d_out, const void *d_x, const void *d_w
     a.d1 = d1;
     a.d2 = d2;
     a.relu = o.relu != 0;
+    a.vec_out = a.ld_out % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & (out_dtype == MGGX_BF16 ? 7u : 15u)) == 0;
     if (a.ld_x < d1 || a.ld_out < d2) return fail(MGGX_EINVAL, "dense_xw_bf16: row stride smaller than width");
     const int nb = mggx::pick_nb(d2);
     const int gy = ((d2 + 15) / 16 + nb - 1) / nb;

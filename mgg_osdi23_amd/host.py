@@ -36,6 +36,11 @@ class _DenseOpts(C.Structure):
     _fields_ = [("ld_x", C.c_int64), ("ld_out", C.c_int64), ("d_row_scale", C.c_void_p), ("relu", C.c_uint32)]
 
 
+class _Mlp2Opts(C.Structure):
+    _fields_ = [("ld_x", C.c_int64), ("ld_out", C.c_int64), ("d_row_scale", C.c_void_p), ("relu_mid", C.c_uint32),
+                ("relu_out", C.c_uint32)]
+
+
 _lib = None
 
 # every symbol include/mggx.h declares
@@ -45,7 +50,7 @@ EXPORTS = [
     "mggx_timer_create", "mggx_timer_start", "mggx_timer_stop", "mggx_timer_elapsed_ms", "mggx_timer_destroy",
     "mggx_release_cached", "mggx_range_partition", "mggx_split_csr", "mggx_build_part", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
-    "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_spmm",
+    "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_mlp2_xw", "mggx_spmm",
     "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
 ]
 
@@ -351,6 +356,18 @@ def dense_forward(out, x, w, n, d1, d2, ld_x=0, ld_out=0, row_scale=None, relu=F
     o.d_row_scale = row_scale.data_ptr() if row_scale is not None else None
     o.relu = int(relu)
     _check(lib().mggx_dense_xw(_dptr(out), _dptr(x), _dptr(w), C.c_int64(n), d1, d2, C.byref(o)))
+
+
+def mlp2_forward(out, x, wa, wb, n, d1, h, d3, ld_x=0, ld_out=0, row_scale=None, relu_mid=True, relu_out=False):
+    """Out = act(X . Wa) . Wb in one pass (h, d3 <= 64): two dense_hidden_forward calls without the round trip of the
+    intermediate through memory."""
+    o = _Mlp2Opts()
+    o.ld_x = ld_x
+    o.ld_out = ld_out
+    o.d_row_scale = row_scale.data_ptr() if row_scale is not None else None
+    o.relu_mid = int(relu_mid)
+    o.relu_out = int(relu_out)
+    _check(lib().mggx_mlp2_xw(_dptr(out), _dptr(x), _dptr(wa), _dptr(wb), C.c_int64(n), d1, h, d3, C.byref(o)))
 
 
 def dense_forward_bf16(out, x, w_bf16, n, d1, d2, ld_x=0, ld_out=0, row_scale=None, relu=False):

@@ -435,6 +435,39 @@ def test_dense_closed_forms_and_epilogue(gpu):
     assert np.all(got[:, 41:] == 9.0)
 
 
+@pytest.mark.parametrize("n,d1,h,d3,relu_mid", [(1000, 64, 64, 64, True), (777, 64, 64, 47, True), (130, 100, 33, 5, False),
+                                                 (17, 7, 16, 64, True), (4099, 200, 48, 17, True)])
+def test_fused_two_layer_update(gpu, n, d1, h, d3, relu_mid):
+    """act(X.Wa).Wb in one pass against the oracle's two dense updates (and against two library calls)."""
+    import torch
+    x = gpu.fill_normal((n, d1), seed=60)
+    wa = gpu.glorot(d1, h, seed=61)
+    wb = gpu.glorot(h, d3, seed=62)
+    s = gpu.fill_uniform((n,), 0.5, 1.5, seed=63)
+    ldo = d3 + 3
+    out = torch.full((n, ldo), 9.0, device="cuda")
+    gpu.mlp2_forward(out, to_dev(x), to_dev(wa), to_dev(wb), n, d1, h, d3, ld_out=ldo, row_scale=to_dev(s), relu_mid=relu_mid)
+    gpu.sync()
+    t = orc.dense(x, wa, f64=True)
+    mag_t = np.abs(x).astype(np.float64) @ np.abs(wa).astype(np.float64)
+    if relu_mid:
+        t = np.maximum(t, 0)
+    want = (t @ wb.astype(np.float64)) * s[:, None]
+    mag = (mag_t @ np.abs(wb).astype(np.float64)) * s[:, None]
+    got = out.cpu().numpy()
+    assert_close_to_oracle(got[:, :d3], want, mag, 2 * FP32_TOL, "fused two-layer update")
+    assert np.all(got[:, d3:] == 9.0)
+    # the two-call form of the same thing
+    mid = torch.empty(n, h, device="cuda")
+    two = torch.empty(n, d3, device="cuda")
+    gpu.dense_forward(mid, to_dev(x), to_dev(wa), n, d1, h, relu=relu_mid)
+    gpu.dense_forward(two, mid, to_dev(wb), n, h, d3, row_scale=to_dev(s))
+    gpu.sync()
+    assert_close_to_oracle(two.cpu().numpy(), want, mag, 2 * FP32_TOL, "two calls")
+    with pytest.raises(gpu.MggxError):
+        gpu.mlp2_forward(out, to_dev(x), to_dev(wa), to_dev(wb), n, d1, 65, d3)
+
+
 @pytest.mark.parametrize("n,c", [(1000, 41), (333, 47), (64, 1), (10, 200), (5, 64)])
 def test_softmax_rows(gpu, n, c):
     import torch
