@@ -92,15 +92,22 @@ def load_traffic(kernel_key, args):
     return {"traffic": nbytes, "traffic_measured_at": "ps=16 wpb=%d dist=%d" % (w, d)}
 
 
-def pick_knobs(args, tune):
-    """(wpb, dist) for one aggregation shape: the command line's, or, when both are 0 and tuning is on, the pair the
-    library's search measures fastest on this input (once, before the timed region; the reference fixes its pair per
-    dataset from the same kind of sweep, bench_MGG_DSE_*.py)."""
-    if args.wpb == 0 and args.dist == 0 and not args.no_tune:
-        w, d, ms = tune()
-        log("tuned: wpb=%d dist=%d (%.4f ms)" % (w, d, ms))
-        return w, d
-    return args.wpb, args.dist
+class Knobs:
+    """(ps, wpb, dist, column blocking) of one aggregation shape: the command line's, or, where --wpb and --dist are 0
+    and the search is on, what the library's search measures fastest on this input (once, before the timed region; the
+    reference fixes its setting per dataset from the same kind of sweep, bench_MGG_DSE_*.py)."""
+
+    def __init__(self, args, tune):
+        self.ps, self.wpb, self.dist, self.blk = args.ps, args.wpb, args.dist, args.col_block_rows
+        if args.wpb == 0 and args.dist == 0 and not args.no_tune:
+            k, ms = tune(args.ps, args.col_block_rows)
+            self.ps, self.wpb, self.dist, self.blk = k["ps"], k["wpb"], k["dist"], k["col_block_rows"]
+            log("search: %s (%.4f ms)" % (self, ms))
+
+    def __str__(self):
+        return "ps=%d wpb=%d dist=%d %s" % (self.ps, self.wpb, self.dist,
+                                            "column blocks of %d ids" % self.blk if self.blk > 0 else
+                                            ("plain order" if self.blk < 0 else "order by rule"))
 
 
 def bench_gcn2(args, torch, host):
@@ -141,17 +148,17 @@ def bench_gcn2(args, torch, host):
 
     d_Y1.zero_()
     d_Y2.zero_()
-    wpb1, dist1 = pick_knobs(args, lambda: host.tune_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, ps,
-                                                           row_scale_out=d_s))
-    wpb2, dist2 = pick_knobs(args, lambda: host.tune_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, ps,
-                                                           row_scale_out=d_s))
+    k1 = Knobs(args, lambda ps, blk: host.tune_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, ps,
+                                                      row_scale_out=d_s, col_block_rows=blk))
+    k2 = Knobs(args, lambda ps, blk: host.tune_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, ps,
+                                                      row_scale_out=d_s, col_block_rows=blk))
     stages = [
         lambda: host.dense_forward(d_Y1, d_X, d_W1, V, in_dim, hidden, row_scale=d_s),
-        lambda: host.mgg_SAG_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, ps, wpb1, dist1,
-                                    row_scale_out=d_s),
+        lambda: host.mgg_SAG_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, k1.ps, k1.wpb, k1.dist,
+                                    row_scale_out=d_s, col_block_rows=k1.blk),
         lambda: host.dense_forward(d_Y2, d_H1, d_W2, V, hidden, ldo, row_scale=d_s),
-        lambda: host.mgg_SAG_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, 0, ps, wpb2, dist2,
-                                    row_scale_out=d_s),
+        lambda: host.mgg_SAG_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, 0, k2.ps, k2.wpb, k2.dist,
+                                    row_scale_out=d_s, col_block_rows=k2.blk),
         lambda: host.softmax_forward(d_P, d_H2, V, out_dim, ld_in=ldo),
     ]
     names = ["dense1", "agg1", "dense2", "agg2", "softmax"]
@@ -198,10 +205,10 @@ def bench_gcn2(args, torch, host):
     d_W2u = torch.from_numpy(W2).to(dev)
     alt = [
         lambda: host.dense_forward(d_Y1, d_X, d_W1, V, in_dim, hidden, row_scale=d_s),
-        lambda: host.mgg_SAG_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, ps, wpb1, dist1,
-                                    row_scale_out=d_s2),
-        lambda: host.mgg_SAG_np_div(d_G, d_H1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, ps, wpb1, dist1,
-                                    row_scale_out=d_s),
+        lambda: host.mgg_SAG_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, k1.ps, k1.wpb, k1.dist,
+                                    row_scale_out=d_s2, col_block_rows=k1.blk),
+        lambda: host.mgg_SAG_np_div(d_G, d_H1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, k1.ps, k1.wpb, k1.dist,
+                                    row_scale_out=d_s, col_block_rows=k1.blk),
         lambda: host.dense_forward(d_Y2b, d_G, d_W2u, V, hidden, out_dim),
         lambda: host.softmax_forward(d_P2, d_Y2b, V, out_dim),
     ]
@@ -241,8 +248,7 @@ def bench_gcn2(args, torch, host):
         "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: 2-layer GCN forward, RMAT(a=.57,b=.19,c=.19) V=%d nnz=%d (self loops, sym-norm), "
-                               "602->16->41 fp32, ps=%d, (wpb, dist) = (%d, %d) at width 16 and (%d, %d) at width 41"
-                               % (V, nnz, ps, wpb1, dist1, wpb2, dist2)},
+                               "602->16->41 fp32; width 16: %s; width 41: %s" % (V, nnz, k1, k2)},
         "roofline": roofline, "cpu_baseline": cpu, "parity": parity, "detail": extra,
     }
 
@@ -264,10 +270,12 @@ def bench_share(args, torch, host):
     d_xl = torch.from_numpy(np.ascontiguousarray(x_remote[lb:ub])).to(dev)  # separate allocation
     d = [torch.from_numpy(a).to(dev) if len(a) else torch.zeros(1, dtype=torch.int32, device=dev) for a in (lp, lc, rp, rc)]
     d_out = torch.empty(R, dim, device=dev)
-    wpb, dist = pick_knobs(args, lambda: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, ps, input_remote=d_xr))
+    kn = Knobs(args, lambda ps, blk: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, ps, input_remote=d_xr,
+                                                      col_block_rows=blk))
 
     def call():
-        host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, ps, wpb, dist, input_remote=d_xr)
+        host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, kn.ps, kn.wpb, kn.dist, input_remote=d_xr,
+                            col_block_rows=kn.blk)
 
     for _ in range(args.warmup):
         call()
@@ -296,7 +304,7 @@ def bench_share(args, torch, host):
         "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[3]: rank-0 1/8 share of RMAT V=%d (ids scrambled), rows=%d nnz=%d (local %d, remote %d), "
-                               "fp32 dim %d, ps=%d wpb=%d dist=%d" % (V, R, nnz, len(lc), len(rc), dim, ps, wpb, dist)},
+                               "fp32 dim %d, %s" % (V, R, nnz, len(lc), len(rc), dim, kn)},
         "roofline": {"bound": "hbm", "kernel": "k_agg (dim 16, local+remote)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      **load_traffic("share_agg", args), "algorithmic_bytes": nbytes, "avg_launch_ms": round(ms, 4)},
@@ -335,11 +343,12 @@ def bench_gin(args, torch, host):
     d_P = torch.empty(V, out_dim, device=dev)
 
     d_Y.zero_()
-    wpb, dist = pick_knobs(args, lambda: host.tune_np_div(d_H, d_Y, d_ptr, d_col, zp, zc, 0, V, hidden, V, ps, gin_eps=eps))
+    kn = Knobs(args, lambda ps, blk: host.tune_np_div(d_H, d_Y, d_ptr, d_col, zp, zc, 0, V, hidden, V, ps, gin_eps=eps, col_block_rows=blk))
     stages, names = [lambda: host.dense_forward(d_Y, d_X, d_W0, V, in_dim, hidden)], ["dense0"]
     for l in range(L):
         last = l == L - 1
-        stages.append(lambda: host.mgg_GIN_np_div(d_H, d_Y, d_ptr, d_col, zp, zc, 0, V, hidden, V, 0, ps, wpb, dist, eps))
+        stages.append(lambda: host.mgg_GIN_np_div(d_H, d_Y, d_ptr, d_col, zp, zc, 0, V, hidden, V, 0, kn.ps, kn.wpb, kn.dist, eps,
+                                                  col_block_rows=kn.blk))
         if args.unfused_mlp:
             stages.append(lambda l=l: host.dense_forward(d_T, d_H, d_Wa[l], V, hidden, hidden, relu=True))
             if last:
@@ -395,7 +404,7 @@ def bench_gin(args, torch, host):
         "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[2]: 5-layer GIN forward, RMAT V=%d nnz=%d, 100->64->47, 2-layer MLP per layer (%s), eps=0, "
-                               "ps=%d wpb=%d dist=%d" % (V, nnz, "two kernels" if args.unfused_mlp else "one fused kernel", ps, wpb, dist)},
+                               "%s" % (V, nnz, "two kernels" if args.unfused_mlp else "one fused kernel", kn)},
         "roofline": {"bound": "hbm", "kernel": "k_agg (GIN, dim 64)", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("gin_agg", args),
                      "algorithmic_bytes": nbytes, "avg_launch_ms": round(agg_ms, 4)},
@@ -427,9 +436,11 @@ def bench_big(args, torch, host):
     W = host.glorot(dim, dim, seed=6)
     d_W = torch.from_numpy(W).to(dev).to(torch.bfloat16)
     d_next = torch.empty(R, dim, device=dev, dtype=torch.bfloat16)
-    wpb, dist = pick_knobs(args, lambda: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, ps, input_remote=d_xr))
+    kn = Knobs(args, lambda ps, blk: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, ps, input_remote=d_xr,
+                                                      col_block_rows=blk))
     stages = [
-        lambda: host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, ps, wpb, dist, input_remote=d_xr),
+        lambda: host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, kn.ps, kn.wpb, kn.dist, input_remote=d_xr,
+                                    col_block_rows=kn.blk),
         lambda: host.dense_forward_bf16(d_next, d_out, d_W, R, dim, dim),
     ]
     for _ in range(args.warmup):
@@ -484,8 +495,8 @@ def bench_big(args, torch, host):
         "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[4] / 2^%d: rank-0 1/8 share of RMAT V=%d (scrambled), rows=%d nnz=%d (local %d, remote %d), "
-                               "bf16 dim %d, fp32 accumulate, then %dx%d bf16 MFMA update; ps=%d wpb=%d dist=%d"
-                               % (k, V, R, nnz, len(lc), len(rc), dim, dim, dim, ps, wpb, dist)},
+                               "bf16 dim %d, fp32 accumulate, then %dx%d bf16 MFMA update; %s"
+                               % (k, V, R, nnz, len(lc), len(rc), dim, dim, dim, kn)},
         "roofline": {"bound": "hbm", "kernel": "k_agg (bf16 dim 128, local+remote)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("big_agg", args),
                      "algorithmic_bytes": nbytes, "avg_launch_ms": round(avg["agg"], 4)},
@@ -521,7 +532,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="gcn2", choices=["gcn2", "share", "gin", "big", "copy"])
-    ap.add_argument("--ps", type=int, default=16)
+    ap.add_argument("--ps", type=int, default=16, help="partSize; 0 = let the library choose (the search then tries 16 and 32)")
+    ap.add_argument("--col-block-rows", type=int, default=0, help="column-blocked partition order: 0 = library decides, -1 = off, "
+                         "N = blocks of N neighbor ids")
     ap.add_argument("--wpb", type=int, default=0, help="wavefronts per workgroup; 0 = let the library choose")
     ap.add_argument("--dist", type=int, default=0, help="interleaved_dist; 0 = let the library choose.  With --wpb 0 --dist 0 (the default) the "
                          "library's search picks the pair once per aggregation shape before the timed region")

@@ -159,7 +159,13 @@ typedef struct mggx_agg_opts {
     int64_t ld_out;              /* row stride of out in elements; 0 = dim */
     const float *d_row_scale_out;/* [ub-lb] multiplies each finished sum (NULL = 1) */
     int in_dtype;                /* MGGX_F32 or MGGX_BF16 (out is always fp32) */
+    int col_block_rows;          /* column-blocked order: 0 = library decides, -1 = off, > 0 = neighbor ids per block */
 } mggx_agg_opts;
+
+typedef struct mggx_agg_knobs {
+    int ps, wpb, dist;           /* partSize / warpPerBlock / interleaved_dist */
+    int col_block_rows;          /* > 0: column-blocked with that many ids per block; -1: plain order */
+} mggx_agg_knobs;
 
 /* mgg_SAG_np_div / mgg_GIN_np_div (include/neighbor_utils.cuh:787-841, 902-958;
  * kernels :1351-1460, :1554-1667):
@@ -171,8 +177,12 @@ typedef struct mggx_agg_opts {
  * ps/wpb/dist are MGG's partSize / warpPerBlock / interleaved_dist: partitions
  * of <= ps neighbors of one row, wpb 64-lane wavefronts per workgroup, dist
  * consecutive partition rounds per wavefront.  They change speed, never the
- * mathematical result.  wpb = 0 and/or dist = 0 let the library choose them from the
- * partition count per row.  opts may be NULL (fp32, overwrite, ld == dim).
+ * mathematical result.  ps = 0, wpb = 0 and/or dist = 0 let the library choose (by rule, or
+ * what mggx_sag_np_div_tune measured on the same arrays).  opts may be NULL (fp32, overwrite, ld == dim).
+ * Column-blocked order (opts->col_block_rows): for a local-only CSR whose rows are sorted by neighbor id and long
+ * (>= 20 neighbors per block and row), the partitions are walked block by block of neighbor ids, so the part of the
+ * feature table in use at any time is small enough to stay in cache; each block leaves a partial row in library
+ * scratch and a second kernel sums them in block order and applies the epilogue.  Same result up to summation order.
  * The partition plan of (d_ptr_l, d_ptr_r, rows, ps) is built on first use and
  * cached by pointer identity: the CSR arrays must not be rewritten in place
  * while cached (mggx_release_cached() drops the cache). */
@@ -182,15 +192,17 @@ int mggx_sag_np_div(float *d_out, const void *d_in_local, const void *d_in_remot
                     int ps, int wpb, int dist, const mggx_agg_opts *opts);
 
 /* The design-space search of bench_MGG_DSE_dist_ps.py:12-42 / bench_MGG_DSE_dist_wpb.py (one process launch per
- * setting there) as one call: runs the aggregation of mggx_sag_np_div with wpb in {4, 8, 16} x dist in {1, 2, 4, 8, 16}
- * (three runs each, the faster of the last two counts), returns the fastest pair and its time, and remembers it in
- * the cached plan, so later mggx_sag_np_div calls on the same CSR arrays with the same dim and in_dtype and
- * wpb = dist = 0 use it.  d_out holds a valid result afterwards.  Synchronises; not for stream capture.
- * MGGX_AGG_ACCUMULATE is rejected (the repeated runs would add up).  Any out-pointer may be NULL. */
+ * setting there) as one call: runs the aggregation of mggx_sag_np_div over ps (as given, or {16, 32} when 0) x plain /
+ * column-blocked order (where the rows are long enough, unless opts fixes it) x wpb in {4, 8, 16} x dist in
+ * {1, 2, 4, 8, 16}, three runs each (the faster of the last two counts), returns the fastest setting and its time, and
+ * remembers it, so later mggx_sag_np_div calls on the same CSR arrays with the same dim and in_dtype that leave
+ * wpb = dist = col_block_rows = 0 (and ps = 0 or the winning ps) use it.  d_out holds a valid result afterwards.
+ * Synchronises; not for stream capture.  MGGX_AGG_ACCUMULATE is rejected (the repeated runs would add up).
+ * Either out-pointer may be NULL. */
 int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const void *d_in_remote,
                          const int *d_ptr_l, const int *d_col_l, const int *d_ptr_r, const int *d_col_r,
                          int lb, int ub, int dim, int nodes_per_pe, int ps, const mggx_agg_opts *opts,
-                         int *wpb_best, int *dist_best, float *ms_best);
+                         mggx_agg_knobs *best, float *ms_best);
 
 /* SAG_host / SAG_cuda_kernel (include/neighbor_utils.cuh:463-506, 2373-2447) and
  * the local half of SAG_host_fused_interleaved (:593-676, 2598-2688): explicit

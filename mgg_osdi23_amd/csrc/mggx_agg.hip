@@ -540,6 +540,17 @@ __global__ void __launch_bounds__(256) k_agg_empty_rows(const AggArgs a, const i
     finish_elem(a, r, d, 0.0f);
 }
 
+// Column-blocked plans: out[v] = epilogue(sum over blocks c of P[c * rows + v]), blocks summed in order.
+__global__ void __launch_bounds__(256) k_agg_block_reduce(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp)
+{
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long long)rows * a.dim) return;
+    const int v = (int)(idx / a.dim), d = (int)(idx % a.dim);
+    float total = 0.0f;
+    for (int c = 0; c < blocks; ++c) total += part[((long long)c * rows + v) * ldp + d];
+    finish_elem(a, v, d, total);
+}
+
 int pow2_ceil(int x)
 {
     int p = 1;
@@ -580,6 +591,7 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     if (ld_in < dim || ld_out < dim) return fail(MGGX_EINVAL, "aggregation: row stride smaller than dim");
     if (plan->rows == 0) return MGGX_OK;
     if (!d_out || !d_in_l) return fail(MGGX_EINVAL, "aggregation: NULL feature pointer");
+    const bool blocked = plan->blocks > 1;
     if (plan->nnz_r > 0 && (!d_in_r || !d_col_r)) return fail(MGGX_EINVAL, "aggregation: remote edges but no remote table");
     if (plan->nnz_l > 0 && !d_col_l) return fail(MGGX_EINVAL, "aggregation: local edges but no column array");
 
@@ -591,8 +603,8 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         mode = MODE_BF16_VEC8;
         lpr = pow2_ceil(dim / 8);
     } else if (o.in_dtype == MGGX_F32) {
-        const bool vec = dim % 4 == 0 && ld_in % 4 == 0 && ld_out % 4 == 0 && aligned16(d_in_l) &&
-                         (!d_in_r || aligned16(d_in_r)) && aligned16(d_out);
+        const bool out_ok = blocked || (ld_out % 4 == 0 && aligned16(d_out));  // blocked plans write their own partial rows
+        const bool vec = dim % 4 == 0 && ld_in % 4 == 0 && out_ok && aligned16(d_in_l) && (!d_in_r || aligned16(d_in_r));
         mode = vec ? MODE_F32_VEC4 : MODE_F32_STRIDED;
         lpr = pow2_ceil((dim + 3) / 4);
     } else {
@@ -602,9 +614,6 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     // 0 = let the library choose (from sweeps on the benchmark graphs): 8 wavefronts; with few slots per wavefront
     // (wide rows) 16 rounds, so a workgroup still covers a few thousand neighbors; otherwise a workgroup tile of
     // about 8 rows' worth of partitions (most rows then finish inside one workgroup), between 1 and 16 rounds.
-    if (wpb == 0 && dist == 0)
-        for (const Plan::Tuned &t : plan->tuned)
-            if (t.dim == dim && t.dtype == o.in_dtype) { wpb = t.wpb; dist = t.dist; }
     if (wpb == 0) wpb = 8;
     if (dist == 0) {
         if (slots <= 4) {
@@ -622,6 +631,7 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     const int cpad = (dim + 3) & ~3;
 
     AggArgs a{};
+    const int ldp = (dim + 3) & ~3;  // row stride of the per-block partial sums of a column-blocked plan
     a.out = d_out;
     a.in_l = d_in_l;
     a.in_r = d_in_r ? d_in_r : d_in_l;
@@ -629,9 +639,9 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     a.col_r = d_col_r;
     a.desc = plan->d_desc;
     a.off = plan->d_off;
-    a.rs_out = o.d_row_scale_out;
+    a.rs_out = blocked ? nullptr : o.d_row_scale_out;
     a.ld_in = ld_in;
-    a.ld_out = ld_out;
+    a.ld_out = blocked ? ldp : ld_out;
     a.num_parts = plan->num_parts;
     a.nnz_l = (int)plan->nnz_l;
     a.nnz_r = (int)plan->nnz_r;
@@ -641,7 +651,7 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     a.dist = dist;
     a.cpad = cpad;
     a.parts_per_wg = (int)parts_per_wg;
-    a.flags = o.flags;
+    a.flags = blocked ? 0u : o.flags;
     a.eps = o.eps;
     a.in_is_bf16 = o.in_dtype == MGGX_BF16;
 
@@ -654,14 +664,14 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     bool buf = false;
     {
         const unsigned long long pl = reinterpret_cast<uintptr_t>(a.in_l), pr = reinterpret_cast<uintptr_t>(a.in_r);
-        const unsigned long long el = pl + (unsigned long long)plan->rows * ld_bytes;
+        const unsigned long long el = pl + (unsigned long long)plan->real_rows * ld_bytes;
         const bool has_r = plan->nnz_r > 0;
         const unsigned long long er = has_r ? pr + ((unsigned long long)plan->max_col_r + 1) * ld_bytes : el;
         const unsigned long long lo = has_r ? (pl < pr ? pl : pr) : pl;
         const unsigned long long hi = el > er ? el : er;
         const unsigned long long win = hi - lo;
         const unsigned long long sentinel = (win + ld_bytes - 1) / ld_bytes;
-        if (win < 0x7FF00000ull && ld_bytes < (1ull << 24) && sentinel < (1ull << 24) - 1 && plan->rows < (1 << 24) &&
+        if (win < 0x7FF00000ull && ld_bytes < (1ull << 24) && sentinel < (1ull << 24) - 1 && plan->real_rows < (1 << 24) &&
             (!has_r || plan->max_col_r < (1 << 24) - 1) && st.gather_addressing == 0) {
             buf = true;
             a.win_base = reinterpret_cast<const void *>(static_cast<uintptr_t>(lo));
@@ -676,10 +686,15 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         const size_t hdr_bytes = (size_t)num_wg * 2 * sizeof(int2);
         const size_t hdr_pad = (hdr_bytes + 255) & ~(size_t)255;
         void *ws = nullptr;
-        int rc = workspace(hdr_pad + (size_t)num_wg * 2 * cpad * sizeof(float), &ws);
+        const size_t carry_bytes = (hdr_pad + (size_t)num_wg * 2 * cpad * sizeof(float) + 255) & ~(size_t)255;
+        const size_t part_bytes = blocked ? (size_t)plan->rows * ldp * sizeof(float) : 0;
+        int rc = workspace(carry_bytes + part_bytes, &ws);
         if (rc) return rc;
         a.c_hdr = static_cast<int2 *>(ws);
         a.c_val = reinterpret_cast<float *>(static_cast<char *>(ws) + hdr_pad);
+        if (blocked) {
+            a.out = reinterpret_cast<float *>(static_cast<char *>(ws) + carry_bytes);
+        }
         const size_t lds_bytes = (size_t)wpb * 2 * sizeof(int2) + (size_t)wpb * 2 * cpad * sizeof(float);
         const dim3 grid((unsigned)num_wg), block((unsigned)(64 * wpb));
         if (buf) {
@@ -701,14 +716,25 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
             MGGX_LAUNCH_CHECK("k_agg_fixup");
         }
     }
-    const bool touch_empty = !(o.flags & MGGX_AGG_ACCUMULATE) || (o.flags & (MGGX_AGG_GIN | MGGX_AGG_RELU));
+    const bool touch_empty = blocked || !(o.flags & MGGX_AGG_ACCUMULATE) || (o.flags & (MGGX_AGG_GIN | MGGX_AGG_RELU));
     if (plan->num_empty > 0 && touch_empty) {
         const long long n = (long long)plan->num_empty * dim;
         k_agg_empty_rows<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(a, plan->d_empty_rows, plan->num_empty);
         MGGX_LAUNCH_CHECK("k_agg_empty_rows");
     }
-    snprintf(st.last_kernel, sizeof(st.last_kernel), "k_agg<%d,%d,%d> grid=%lld block=%d parts=%d", lpr, mode, (int)buf, num_wg, 64 * wpb,
-             plan->num_parts);
+    if (blocked) {
+        AggArgs r = a;  // the real output and epilogue
+        const float *part = a.out;
+        r.out = d_out;
+        r.ld_out = ld_out;
+        r.rs_out = o.d_row_scale_out;
+        r.flags = o.flags;
+        const long long n = (long long)plan->real_rows * dim;
+        k_agg_block_reduce<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(r, part, plan->real_rows, plan->blocks, ldp);
+        MGGX_LAUNCH_CHECK("k_agg_block_reduce");
+    }
+    snprintf(st.last_kernel, sizeof(st.last_kernel), "k_agg<%d,%d,%d> grid=%lld block=%d parts=%d blocks=%d", lpr, mode, (int)buf, num_wg,
+             64 * wpb, plan->num_parts, plan->blocks);
     return MGGX_OK;
 }
 
@@ -717,73 +743,140 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
 
 using mggx::fail;
 
+namespace mggx {
+namespace {
+
+constexpr int DEFAULT_BLOCK_ROWS = 48 * 1024;  // neighbor ids per column block (sweeps on the 233 K-node benchmark graph)
+
+// A column-blocked plan re-reads and re-writes a partial output row per block: it pays off when rows are long.
+bool blocking_eligible(const GraphInfo &g, int block_rows)
+{
+    if (g.nnz_r > 0 || g.rows < 2 * (long long)block_rows) return false;
+    const long long blocks = ((long long)g.rows + block_rows - 1) / block_rows;
+    return g.nnz_l >= 20 * blocks * (long long)g.rows;
+}
+
+struct Knobs {
+    int ps, wpb, dist, block_rows;  // block_rows: > 0 column-blocked, -1 plain
+};
+
+// Fills in the knobs the caller left at 0: from the search's result for this CSR, width and element type, else by rule.
+Knobs resolve_knobs(const GraphInfo &g, int dim, int dtype, int ps, int wpb, int dist, int block_rows)
+{
+    const GraphInfo::Tuned *t = nullptr;
+    for (const GraphInfo::Tuned &e : g.tuned)
+        if (e.dim == dim && e.dtype == dtype) t = &e;
+    Knobs k{ps, wpb, dist, block_rows};
+    if (t && (ps == 0 || ps == t->ps) && wpb == 0 && dist == 0 && block_rows == 0) return Knobs{t->ps, t->wpb, t->dist, t->block_rows};
+    if (k.ps == 0) k.ps = 16;
+    if (k.block_rows == 0) k.block_rows = blocking_eligible(g, DEFAULT_BLOCK_ROWS) ? DEFAULT_BLOCK_ROWS : -1;
+    return k;
+}
+
+int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in_local, const void *d_in_remote, const int *d_ptr_l,
+              const int *d_col_l, const int *d_ptr_r, const int *d_col_r, int lb, int ub, int dim, const mggx_agg_opts &o)
+{
+    Plan *plan = nullptr;
+    int rc;
+    if (k.block_rows > 0 && g.nnz_r == 0 && ub - lb >= 2 * (long long)k.block_rows) {
+        rc = plan_get_blocked(d_ptr_l, d_col_l, ub - lb, lb, k.ps, k.block_rows, &plan);
+        if (rc) return rc;
+        if (plan->unsuitable) plan = nullptr;
+    }
+    if (!plan) {
+        rc = plan_get(d_ptr_l, d_ptr_r, d_col_r, ub - lb, k.ps, &plan);
+        if (rc) return rc;
+    }
+    return run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, k.wpb, k.dist, o);
+}
+
+int check_np_div_args(const char *who, const int *d_ptr_l, int lb, int ub, int nodes_per_pe, int &ps, int block_rows)
+{
+    if (ub < lb || !d_ptr_l) return fail(MGGX_EINVAL, "%s: bad row range [%d,%d) or NULL row pointers", who, lb, ub);
+    if (ps < 0) return fail(MGGX_EINVAL, "%s: ps %d must not be negative (0 = choose)", who, ps);
+    if (nodes_per_pe < ub - lb) return fail(MGGX_EINVAL, "%s: nodes_per_pe %d smaller than the row range", who, nodes_per_pe);
+    if (block_rows < -1) return fail(MGGX_EINVAL, "%s: col_block_rows %d (0 = choose, -1 = off)", who, block_rows);
+    if (ps > (int)DESC_LEN_MASK) ps = (int)DESC_LEN_MASK;  // longer than any row: same partitions
+    return MGGX_OK;
+}
+
+}  // namespace
+}  // namespace mggx
+
 MGGX_EXPORT int mggx_sag_np_div(float *d_out, const void *d_in_local, const void *d_in_remote, const int *d_ptr_l,
                                 const int *d_col_l, const int *d_ptr_r, const int *d_col_r, int lb, int ub, int dim,
                                 int nodes_per_pe, int ps, int wpb, int dist, const mggx_agg_opts *opts)
 {
     int rc = mggx::ensure_init();
     if (rc) return rc;
-    if (ub < lb || !d_ptr_l) return fail(MGGX_EINVAL, "sag_np_div: bad row range [%d,%d) or NULL row pointers", lb, ub);
-    if (ps < 1) return fail(MGGX_EINVAL, "sag_np_div: ps %d must be positive", ps);
-    if (nodes_per_pe < ub - lb) return fail(MGGX_EINVAL, "sag_np_div: nodes_per_pe %d smaller than the row range", nodes_per_pe);
-    if (ps > (int)mggx::DESC_LEN_MASK) ps = (int)mggx::DESC_LEN_MASK;  // longer than any row: same partitions
     mggx_agg_opts o{};
     if (opts) o = *opts;
-    mggx::Plan *plan = nullptr;
-    rc = mggx::plan_get(d_ptr_l, d_ptr_r, d_col_r, ub - lb, ps, &plan);
+    rc = mggx::check_np_div_args("sag_np_div", d_ptr_l, lb, ub, nodes_per_pe, ps, o.col_block_rows);
     if (rc) return rc;
-    return mggx::run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, wpb, dist, o);
+    mggx::GraphInfo *g = nullptr;
+    rc = mggx::graph_info(d_ptr_l, d_ptr_r, ub - lb, &g);
+    if (rc) return rc;
+    const mggx::Knobs k = mggx::resolve_knobs(*g, dim, o.in_dtype, ps, wpb, dist, o.col_block_rows);
+    return mggx::run_knobs(*g, k, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o);
 }
 
 MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const void *d_in_remote, const int *d_ptr_l,
                                      const int *d_col_l, const int *d_ptr_r, const int *d_col_r, int lb, int ub, int dim,
-                                     int nodes_per_pe, int ps, const mggx_agg_opts *opts, int *wpb_best, int *dist_best,
-                                     float *ms_best)
+                                     int nodes_per_pe, int ps, const mggx_agg_opts *opts, mggx_agg_knobs *best_out, float *ms_best)
 {
     int rc = mggx::ensure_init();
     if (rc) return rc;
-    if (ub < lb || !d_ptr_l) return fail(MGGX_EINVAL, "sag_np_div_tune: bad row range [%d,%d) or NULL row pointers", lb, ub);
-    if (ps < 1) return fail(MGGX_EINVAL, "sag_np_div_tune: ps %d must be positive", ps);
-    if (nodes_per_pe < ub - lb) return fail(MGGX_EINVAL, "sag_np_div_tune: nodes_per_pe %d smaller than the row range", nodes_per_pe);
-    if (ps > (int)mggx::DESC_LEN_MASK) ps = (int)mggx::DESC_LEN_MASK;
     mggx_agg_opts o{};
     if (opts) o = *opts;
+    rc = mggx::check_np_div_args("sag_np_div_tune", d_ptr_l, lb, ub, nodes_per_pe, ps, o.col_block_rows);
+    if (rc) return rc;
     if (o.flags & MGGX_AGG_ACCUMULATE) return fail(MGGX_EINVAL, "sag_np_div_tune: repeated runs would accumulate; clear MGGX_AGG_ACCUMULATE");
-    mggx::Plan *plan = nullptr;
-    rc = mggx::plan_get(d_ptr_l, d_ptr_r, d_col_r, ub - lb, ps, &plan);
+    mggx::GraphInfo *g = nullptr;
+    rc = mggx::graph_info(d_ptr_l, d_ptr_r, ub - lb, &g);
     if (rc) return rc;
     mggx::State &st = mggx::state();
     hipEvent_t e0, e1;
     MGGX_HIP(hipEventCreate(&e0));
     MGGX_HIP(hipEventCreate(&e1));
+    // the grid: ps as given, or {16, 32}; plain and, where rows are long enough, column-blocked; wpb x dist
+    int pss[2] = {ps, 0}, n_ps = 1;
+    if (ps == 0) { pss[0] = 16; pss[1] = 32; n_ps = 2; }
+    int blks[2] = {-1, 0}, n_blk = 1;
+    if (o.col_block_rows > 0) blks[0] = o.col_block_rows;
+    else if (o.col_block_rows == 0 && mggx::blocking_eligible(*g, mggx::DEFAULT_BLOCK_ROWS)) { blks[1] = mggx::DEFAULT_BLOCK_ROWS; n_blk = 2; }
     static const int wpbs[] = {8, 4, 16}, dists[] = {1, 2, 4, 8, 16};
     float best = -1.f;
-    int bw = 8, bd = 1;
-    rc = mggx::run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, 8, 1, o);  // warm caches and workspace
-    for (int wi = 0; wi < 3 && !rc; ++wi)
-        for (int di = 0; di < 5 && !rc; ++di) {
-            float ms_min = -1.f;
-            for (int rep = 0; rep < 3 && !rc; ++rep) {
-                hipError_t e = hipEventRecord(e0, st.stream);
-                rc = mggx::run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, wpbs[wi], dists[di], o);
-                if (e == hipSuccess) e = hipEventRecord(e1, st.stream);
-                if (e == hipSuccess) e = hipEventSynchronize(e1);
-                float ms = 0.f;
-                if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-                if (e != hipSuccess && !rc) rc = fail(MGGX_EHIP, "sag_np_div_tune: timing failed: %s", hipGetErrorString(e));
-                if (!rc && rep > 0 && (ms_min < 0.f || ms < ms_min)) ms_min = ms;  // the first run of a setting is untimed
-            }
-            if (!rc && (best < 0.f || ms_min < best)) { best = ms_min; bw = wpbs[wi]; bd = dists[di]; }
-        }
+    mggx::Knobs bk{pss[0], 8, 1, blks[0]};
+    rc = mggx::run_knobs(*g, bk, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o);  // warm-up
+    for (int pi = 0; pi < n_ps && !rc; ++pi)
+        for (int bi = 0; bi < n_blk && !rc; ++bi)
+            for (int wi = 0; wi < 3 && !rc; ++wi)
+                for (int di = 0; di < 5 && !rc; ++di) {
+                    const mggx::Knobs k{pss[pi], wpbs[wi], dists[di], blks[bi]};
+                    float ms_min = -1.f;
+                    for (int rep = 0; rep < 3 && !rc; ++rep) {
+                        hipError_t e = hipEventRecord(e0, st.stream);
+                        rc = mggx::run_knobs(*g, k, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o);
+                        if (e == hipSuccess) e = hipEventRecord(e1, st.stream);
+                        if (e == hipSuccess) e = hipEventSynchronize(e1);
+                        float ms = 0.f;
+                        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+                        if (e != hipSuccess && !rc) rc = fail(MGGX_EHIP, "sag_np_div_tune: timing failed: %s", hipGetErrorString(e));
+                        if (!rc && rep > 0 && (ms_min < 0.f || ms < ms_min)) ms_min = ms;  // the first run of a setting is untimed
+                    }
+                    if (!rc && (best < 0.f || ms_min < best)) { best = ms_min; bk = k; }
+                }
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     if (rc) return rc;
+    // leave the winner's result in d_out and remember it
+    rc = mggx::run_knobs(*g, bk, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o);
+    if (rc) return rc;
     bool found = false;
-    for (mggx::Plan::Tuned &t : plan->tuned)
-        if (t.dim == dim && t.dtype == o.in_dtype) { t.wpb = bw; t.dist = bd; found = true; }
-    if (!found) plan->tuned.push_back({dim, o.in_dtype, bw, bd});
-    if (wpb_best) *wpb_best = bw;
-    if (dist_best) *dist_best = bd;
+    for (mggx::GraphInfo::Tuned &t : g->tuned)
+        if (t.dim == dim && t.dtype == o.in_dtype) { t.ps = bk.ps; t.wpb = bk.wpb; t.dist = bk.dist; t.block_rows = bk.block_rows; found = true; }
+    if (!found) g->tuned.push_back({dim, o.in_dtype, bk.ps, bk.wpb, bk.dist, bk.block_rows});
+    if (best_out) { best_out->ps = bk.ps; best_out->wpb = bk.wpb; best_out->dist = bk.dist; best_out->col_block_rows = bk.block_rows; }
     if (ms_best) *ms_best = best;
     return MGGX_OK;
 }

@@ -53,8 +53,24 @@ struct Plan {
     int num_empty = 0;
     int64_t nnz_l = 0, nnz_r = 0;
     int max_col_r = -1;        // largest remote neighbor id (bounds the remote table)
-    // (wpb, dist) measured best by mggx_sag_np_div_tune for a row width and element type; used when a call passes 0/0
-    struct Tuned { int dim, dtype, wpb, dist; };
+    // Column-blocked plans: the neighbor ids [lb, lb + real_rows) are cut into `blocks` ranges of `block_rows` ids and
+    // `rows` = blocks * real_rows virtual rows; virtual row c * real_rows + v holds row v's neighbors inside block c,
+    // so the descriptor order walks the feature table block by block.  Plain plans: blocks == 1, rows == real_rows.
+    const int *d_col_l = nullptr;  // cache key of blocked plans (they depend on the column values)
+    int real_rows = 0;
+    int block_rows = 0;
+    int blocks = 1;
+    bool unsuitable = false;   // blocked plan asked for, but the rows are not sorted by neighbor id
+};
+
+// What is known about a CSR the aggregation has been called with (keyed by pointer identity).
+struct GraphInfo {
+    const int *d_ptr_l = nullptr;
+    const int *d_ptr_r = nullptr;
+    int rows = 0;
+    int64_t nnz_l = 0, nnz_r = 0;
+    // knobs measured best by mggx_sag_np_div_tune for a row width and element type; used where a call passes 0
+    struct Tuned { int dim, dtype, ps, wpb, dist, block_rows; };
     std::vector<Tuned> tuned;
 };
 
@@ -64,6 +80,7 @@ struct State {
     void *ws = nullptr;
     size_t ws_bytes = 0;
     std::vector<Plan *> plans;
+    std::vector<GraphInfo> graphs;
     char last_kernel[160] = "";
     int gather_addressing = 0;  // 0 = choose per call, 1 = always 64-bit addresses
 };
@@ -78,6 +95,9 @@ int workspace(size_t bytes, void **p);
 int exclusive_scan_i32(const int *d_in, int *d_out, int n, long long *total_host);
 
 int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int rows, int ps, Plan **out);
+// Column-blocked plan of a local-only CSR; (*out)->unsuitable is set when the rows are not sorted by neighbor id.
+int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int ps, int block_rows, Plan **out);
+int graph_info(const int *d_ptr_l, const int *d_ptr_r, int rows, GraphInfo **out);
 int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows,
                       int num_parts, int ps, Plan **out);
 void plan_free(Plan *p);

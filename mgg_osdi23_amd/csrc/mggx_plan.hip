@@ -100,14 +100,16 @@ __global__ void __launch_bounds__(SCAN_THREADS) k_scan_apply(const int *__restri
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x == SCAN_THREADS - 1) out[n] = (int)run;
 }
 
-// parts of one CSR side per row: ceil(deg/ps); both sides summed when ptr_r != NULL
-__global__ void __launch_bounds__(256) k_count_parts(const int *__restrict__ ptr_l, const int *__restrict__ ptr_r, int rows,
+// parts of one CSR side per row: ceil(deg/ps); both sides summed when beg_r != NULL.  Row r spans edges
+// [beg[r], end[r]) (a CSR passes end = ptr + 1).
+__global__ void __launch_bounds__(256) k_count_parts(const int *__restrict__ beg_l, const int *__restrict__ end_l,
+                                                     const int *__restrict__ beg_r, const int *__restrict__ end_r, int rows,
                                                      int ps, int *__restrict__ cnt)
 {
     const int r = blockIdx.x * 256 + threadIdx.x;
     if (r >= rows) return;
-    long long c = ((long long)ptr_l[r + 1] - ptr_l[r] + ps - 1) / ps;
-    if (ptr_r) c += ((long long)ptr_r[r + 1] - ptr_r[r] + ps - 1) / ps;
+    long long c = ((long long)end_l[r] - beg_l[r] + ps - 1) / ps;
+    if (beg_r) c += ((long long)end_r[r] - beg_r[r] + ps - 1) / ps;
     cnt[r] = (int)c;
 }
 
@@ -123,8 +125,9 @@ __device__ __forceinline__ int row_of_part(const int *__restrict__ off, int rows
     return lo;
 }
 
-__global__ void __launch_bounds__(256) k_fill_desc(const int *__restrict__ off, const int *__restrict__ ptr_l,
-                                                   const int *__restrict__ ptr_r, int rows, int ps, int num_parts,
+__global__ void __launch_bounds__(256) k_fill_desc(const int *__restrict__ off, const int *__restrict__ beg_l,
+                                                   const int *__restrict__ end_l, const int *__restrict__ beg_r,
+                                                   const int *__restrict__ end_r, int rows, int ps, int num_parts,
                                                    int4 *__restrict__ desc)
 {
     const int q = blockIdx.x * 256 + threadIdx.x;
@@ -132,21 +135,54 @@ __global__ void __launch_bounds__(256) k_fill_desc(const int *__restrict__ off, 
     const int r = row_of_part(off, rows, q);
     const int j = q - off[r];
     const int total = off[r + 1] - off[r];
-    const int nl = (int)(((long long)ptr_l[r + 1] - ptr_l[r] + ps - 1) / ps);
+    const int nl = (int)(((long long)end_l[r] - beg_l[r] + ps - 1) / ps);
     unsigned start, len;
     if (j < nl) {
-        const long long beg = (long long)ptr_l[r] + (long long)j * ps;
+        const long long beg = (long long)beg_l[r] + (long long)j * ps;
         start = (unsigned)beg;
-        len = (unsigned)min((long long)ps, (long long)ptr_l[r + 1] - beg);
+        len = (unsigned)min((long long)ps, (long long)end_l[r] - beg);
     } else {
-        const long long beg = (long long)ptr_r[r] + (long long)(j - nl) * ps;
+        const long long beg = (long long)beg_r[r] + (long long)(j - nl) * ps;
         start = (unsigned)beg | DESC_REMOTE;
-        len = (unsigned)min((long long)ps, (long long)ptr_r[r + 1] - beg);
+        len = (unsigned)min((long long)ps, (long long)end_r[r] - beg);
     }
     unsigned z = len;
     if (j == 0) z |= DESC_FIRST;
     if (j == total - 1) z |= DESC_LAST;
     desc[q] = make_int4((int)start, r, (int)z, 0);
+}
+
+// Column-blocked plans.  One wavefront per row: flag = 1 if some row's neighbor ids are not in non-decreasing order.
+__global__ void __launch_bounds__(256) k_check_sorted(const int *__restrict__ ptr, const int *__restrict__ col, int rows,
+                                                      int *__restrict__ flag)
+{
+    const int r = blockIdx.x * 4 + (int)(threadIdx.x >> 6);
+    if (r >= rows) return;
+    const int lane = (int)(threadIdx.x & 63u);
+    bool bad = false;
+    for (int e = ptr[r] + lane; e + 1 < ptr[r + 1]; e += 64) bad |= col[e] > col[e + 1];
+    if (bad) *flag = 1;
+}
+
+// vbeg[c * rows + v] = first edge of row v whose neighbor id is >= lb + c * block_rows, c = 0..blocks (rows sorted)
+__global__ void __launch_bounds__(256) k_block_bounds(const int *__restrict__ ptr, const int *__restrict__ col, int rows, int lb,
+                                                      int block_rows, int blocks, int *__restrict__ vbeg)
+{
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long long)(blocks + 1) * rows) return;
+    const int c = (int)(idx / rows), v = (int)(idx % rows);
+    int lo = ptr[v], hi = ptr[v + 1];
+    if (c == blocks) {
+        lo = hi;
+    } else if (c > 0) {
+        const long long key = (long long)lb + (long long)c * block_rows;
+        while (lo < hi) {
+            const int mid = (int)(((long long)lo + hi) >> 1);
+            if (col[mid] < key) lo = mid + 1;
+            else hi = mid;
+        }
+    }
+    vbeg[idx] = lo;
 }
 
 // explicit partition arrays (reference layout) -> descriptors; lengths from row_ptr
@@ -341,7 +377,8 @@ int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int row
 {
     State &s = state();
     for (Plan *p : s.plans)
-        if (p->d_ptr_l == d_ptr_l && p->d_ptr_r == d_ptr_r && p->rows == rows && p->ps == ps && !p->d_part_ptr) {
+        if (p->d_ptr_l == d_ptr_l && p->d_ptr_r == d_ptr_r && p->rows == rows && p->ps == ps && !p->d_part_ptr && p->blocks == 1 &&
+            !p->unsuitable) {
             *out = p;
             return MGGX_OK;
         }
@@ -349,6 +386,7 @@ int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int row
     p->d_ptr_l = d_ptr_l;
     p->d_ptr_r = d_ptr_r;
     p->rows = rows;
+    p->real_rows = rows;
     p->ps = ps;
     int rc = MGGX_OK;
     int *d_cnt = nullptr;
@@ -358,7 +396,9 @@ int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int row
             rc = fail(MGGX_ENOMEM, "plan: row arrays for %d rows", rows);
             break;
         }
-        if (rows > 0) k_count_parts<<<(rows + 255) / 256, 256, 0, s.stream>>>(d_ptr_l, d_ptr_r, rows, ps, d_cnt);
+        if (rows > 0)
+            k_count_parts<<<(rows + 255) / 256, 256, 0, s.stream>>>(d_ptr_l, d_ptr_l + 1, d_ptr_r, d_ptr_r ? d_ptr_r + 1 : nullptr, rows, ps,
+                                                                    d_cnt);
         long long total = 0;
         rc = exclusive_scan_i32(d_cnt, p->d_off, rows, &total);
         if (rc) break;
@@ -398,8 +438,9 @@ int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int row
             break;
         }
         if (p->num_parts > 0) {
-            k_fill_desc<<<(p->num_parts + 255) / 256, 256, 0, s.stream>>>(p->d_off, d_ptr_l, d_ptr_r, rows, ps,
-                                                                          p->num_parts, p->d_desc);
+            k_fill_desc<<<(p->num_parts + 255) / 256, 256, 0, s.stream>>>(p->d_off, d_ptr_l, d_ptr_l + 1, d_ptr_r,
+                                                                          d_ptr_r ? d_ptr_r + 1 : nullptr, rows, ps, p->num_parts,
+                                                                          p->d_desc);
             if (hipGetLastError() != hipSuccess) {
                 rc = fail(MGGX_EHIP, "plan: descriptor kernel launch failed");
                 break;
@@ -432,6 +473,7 @@ int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_
     p->d_part_ptr = d_part_ptr;
     p->d_part2node = d_part2node;
     p->rows = rows;
+    p->real_rows = rows;
     p->ps = ps;
     p->num_parts = num_parts;
     int rc = MGGX_OK;
@@ -466,6 +508,119 @@ int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_
     return MGGX_OK;
 }
 
+int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int ps, int block_rows, Plan **out)
+{
+    State &s = state();
+    for (Plan *p : s.plans)
+        if (p->d_ptr_l == d_ptr_l && p->d_col_l == d_col_l && p->real_rows == rows && p->ps == ps && p->block_rows == block_rows &&
+            (p->blocks > 1 || p->unsuitable)) {
+            *out = p;
+            return MGGX_OK;
+        }
+    if (block_rows < 1 || rows < 1) return fail(MGGX_EINVAL, "plan: column blocks of %d rows over %d rows", block_rows, rows);
+    const long long blocks = ((long long)rows + block_rows - 1) / block_rows;
+    const long long vrows = blocks * rows;
+    if (blocks < 2 || vrows + rows > 0x7fffffffLL) return fail(MGGX_ELIMIT, "plan: %lld column blocks over %d rows", blocks, rows);
+    Plan *p = new Plan;
+    p->d_ptr_l = d_ptr_l;
+    p->d_col_l = d_col_l;
+    p->real_rows = rows;
+    p->ps = ps;
+    p->block_rows = block_rows;
+    int rc = MGGX_OK;
+    int *d_cnt = nullptr, *d_vbeg = nullptr, *d_flag = nullptr;
+    do {
+        int flag = 0;
+        if (hipMalloc((void **)&d_flag, sizeof(int)) != hipSuccess) {
+            rc = fail(MGGX_ENOMEM, "plan: scratch");
+            break;
+        }
+        (void)hipMemsetAsync(d_flag, 0, sizeof(int), s.stream);
+        k_check_sorted<<<(rows + 3) / 4, 256, 0, s.stream>>>(d_ptr_l, d_col_l, rows, d_flag);
+        hipError_t e = hipMemcpyAsync(&flag, d_flag, sizeof(int), hipMemcpyDeviceToHost, s.stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(s.stream);
+        if (e != hipSuccess) {
+            rc = fail(MGGX_EHIP, "plan: sortedness check: %s", hipGetErrorString(e));
+            break;
+        }
+        if (flag) {  // remember the answer; the caller falls back to the plain plan
+            p->unsuitable = true;
+            p->rows = rows;
+            break;
+        }
+        p->rows = (int)vrows;
+        p->blocks = (int)blocks;
+        if (hipMalloc((void **)&d_vbeg, sizeof(int) * (size_t)(vrows + rows)) != hipSuccess ||
+            hipMalloc((void **)&d_cnt, sizeof(int) * (size_t)vrows) != hipSuccess ||
+            hipMalloc((void **)&p->d_off, sizeof(int) * ((size_t)vrows + 1)) != hipSuccess) {
+            rc = fail(MGGX_ENOMEM, "plan: arrays for %lld virtual rows", vrows);
+            break;
+        }
+        k_block_bounds<<<(unsigned)((vrows + rows + 255) / 256), 256, 0, s.stream>>>(d_ptr_l, d_col_l, rows, lb, block_rows, (int)blocks,
+                                                                                   d_vbeg);
+        k_count_parts<<<(unsigned)((vrows + 255) / 256), 256, 0, s.stream>>>(d_vbeg, d_vbeg + rows, nullptr, nullptr, (int)vrows, ps, d_cnt);
+        long long total = 0;
+        rc = exclusive_scan_i32(d_cnt, p->d_off, (int)vrows, &total);
+        if (rc) break;
+        p->num_parts = (int)total;
+        int end = 0;
+        if (hipMemcpy(&end, d_ptr_l + rows, sizeof(int), hipMemcpyDeviceToHost) != hipSuccess) {
+            rc = fail(MGGX_EHIP, "plan: reading edge count");
+            break;
+        }
+        p->nnz_l = end;
+        if (hipMalloc((void **)&p->d_desc, sizeof(int4) * (size_t)std::max(p->num_parts, 1)) != hipSuccess) {
+            rc = fail(MGGX_ENOMEM, "plan: %d descriptors", p->num_parts);
+            break;
+        }
+        if (p->num_parts > 0) {
+            k_fill_desc<<<(p->num_parts + 255) / 256, 256, 0, s.stream>>>(p->d_off, d_vbeg, d_vbeg + rows, nullptr, nullptr, (int)vrows, ps,
+                                                                          p->num_parts, p->d_desc);
+            if (hipGetLastError() != hipSuccess) {
+                rc = fail(MGGX_EHIP, "plan: descriptor kernel launch failed");
+                break;
+            }
+        }
+        rc = plan_finish(p);  // synchronises: d_vbeg is no longer in use afterwards
+    } while (0);
+    if (d_cnt) (void)hipFree(d_cnt);
+    if (d_vbeg) (void)hipFree(d_vbeg);
+    if (d_flag) (void)hipFree(d_flag);
+    if (rc) {
+        plan_free(p);
+        return rc;
+    }
+    cache_insert(p);
+    *out = p;
+    return MGGX_OK;
+}
+
+int graph_info(const int *d_ptr_l, const int *d_ptr_r, int rows, GraphInfo **out)
+{
+    State &s = state();
+    for (GraphInfo &g : s.graphs)
+        if (g.d_ptr_l == d_ptr_l && g.d_ptr_r == d_ptr_r && g.rows == rows) {
+            *out = &g;
+            return MGGX_OK;
+        }
+    GraphInfo g;
+    g.d_ptr_l = d_ptr_l;
+    g.d_ptr_r = d_ptr_r;
+    g.rows = rows;
+    int ends[2] = {0, 0};
+    if (rows > 0) {
+        MGGX_HIP(hipStreamSynchronize(s.stream));
+        MGGX_HIP(hipMemcpy(&ends[0], d_ptr_l + rows, sizeof(int), hipMemcpyDeviceToHost));
+        if (d_ptr_r) MGGX_HIP(hipMemcpy(&ends[1], d_ptr_r + rows, sizeof(int), hipMemcpyDeviceToHost));
+    }
+    g.nnz_l = ends[0];
+    g.nnz_r = ends[1];
+    if (s.graphs.size() >= 32) s.graphs.erase(s.graphs.begin());
+    s.graphs.push_back(g);
+    *out = &s.graphs.back();
+    return MGGX_OK;
+}
+
 }  // namespace mggx
 
 using mggx::fail;
@@ -491,7 +646,8 @@ MGGX_EXPORT int mggx_build_part_device(const int *d_indptr, int num_nodes, int p
     long long total = 0;
     do {
         if (num_nodes > 0)
-            mggx::k_count_parts<<<(num_nodes + 255) / 256, 256, 0, s.stream>>>(d_indptr, nullptr, num_nodes, part_size, d_cnt);
+            mggx::k_count_parts<<<(num_nodes + 255) / 256, 256, 0, s.stream>>>(d_indptr, d_indptr + 1, nullptr, nullptr, num_nodes, part_size,
+                                                                               d_cnt);
         rc = mggx::exclusive_scan_i32(d_cnt, d_n2p, num_nodes, &total);
         if (rc) break;
         mggx::k_set_tail<<<1, 1, 0, s.stream>>>(d_n2p, num_nodes);

@@ -204,6 +204,7 @@ MGGX_EXPORT int mggx_release_cached(void)
     if (s.device >= 0) MGGX_HIP(hipStreamSynchronize(s.stream));
     for (mggx::Plan *p : s.plans) mggx::plan_free(p);
     s.plans.clear();
+    s.graphs.clear();
     if (s.ws) {
         MGGX_HIP(hipFree(s.ws));
         s.ws = nullptr;

@@ -29,7 +29,11 @@ class MggxError(RuntimeError):
 
 class _AggOpts(C.Structure):
     _fields_ = [("flags", C.c_uint32), ("eps", C.c_float), ("ld_in", C.c_int64), ("ld_out", C.c_int64),
-                ("d_row_scale_out", C.c_void_p), ("in_dtype", C.c_int)]
+                ("d_row_scale_out", C.c_void_p), ("in_dtype", C.c_int), ("col_block_rows", C.c_int)]
+
+
+class _AggKnobs(C.Structure):
+    _fields_ = [("ps", C.c_int), ("wpb", C.c_int), ("dist", C.c_int), ("col_block_rows", C.c_int)]
 
 
 class _DenseOpts(C.Structure):
@@ -240,7 +244,7 @@ def _pin(*tensors) -> None:
     if key in _pinned:
         return
     _pinned[key] = tensors
-    while len(_pinned) > 32:  # the library keeps at most 16 plans; anything older is already evicted there
+    while len(_pinned) > 256:  # the library remembers at most 16 plans and 32 CSRs; anything older is forgotten there
         _pinned.pop(next(iter(_pinned)))
 
 
@@ -279,7 +283,7 @@ def build_part_device(d_indptr, num_nodes: int, part_size: int, compat: bool = T
 
 
 def _agg(out, in_local, in_remote, ptr_l, col_l, ptr_r, col_r, lb, ub, dim, npp, ps, wpb, dist, flags, eps,
-         ld_in, ld_out, row_scale_out):
+         ld_in, ld_out, row_scale_out, col_block_rows=0):
     import torch
     o = _AggOpts()
     o.flags = flags
@@ -288,16 +292,18 @@ def _agg(out, in_local, in_remote, ptr_l, col_l, ptr_r, col_r, lb, ub, dim, npp,
     o.ld_out = ld_out
     o.d_row_scale_out = row_scale_out.data_ptr() if row_scale_out is not None else None
     o.in_dtype = BF16 if in_local.dtype == torch.bfloat16 else F32
-    _pin(ptr_l, ptr_r)
+    o.col_block_rows = col_block_rows
+    _pin(ptr_l, ptr_r, col_l)
     _check(lib().mggx_sag_np_div(_dptr(out), _dptr(in_local), _dptr(in_remote), _dptr(ptr_l), _dptr(col_l),
                                  _dptr(ptr_r), _dptr(col_r), lb, ub, dim, npp, ps, wpb, dist, C.byref(o)))
 
 
 def tune_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb, ub, dim, nodePerPE,
-                np_size, *, input_remote=None, gin_eps=None, ld_in=0, ld_out=0, row_scale_out=None, relu=False):
+                np_size, *, input_remote=None, gin_eps=None, ld_in=0, ld_out=0, row_scale_out=None, relu=False, col_block_rows=0):
     """The search of the reference's bench_MGG_DSE_dist_ps.py / bench_MGG_DSE_dist_wpb.py in one call: times
-    warpPerBlock x interleaved_dist on this input, returns (warpPerBlock, interleaved_dist, ms) of the fastest and
-    makes later calls with warpPerBlock = interleaved_dist = 0 on the same CSR tensors use it."""
+    partSize (as given, or 16 and 32 when 0) x plain / column-blocked order x warpPerBlock x interleaved_dist on this
+    input, returns ({"ps", "wpb", "dist", "col_block_rows"}, ms) of the fastest and makes later calls that leave the
+    knobs at 0 on the same CSR tensors use it."""
     import torch
     o = _AggOpts()
     o.flags = (AGG_RELU if relu else 0) | (AGG_GIN if gin_eps is not None else 0)
@@ -306,33 +312,34 @@ def tune_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, c
     o.ld_out = ld_out
     o.d_row_scale_out = row_scale_out.data_ptr() if row_scale_out is not None else None
     o.in_dtype = BF16 if input.dtype == torch.bfloat16 else F32
-    _pin(row_pointers_l, row_pointers_r)
-    w, d, ms = C.c_int(), C.c_int(), C.c_float()
+    o.col_block_rows = col_block_rows
+    _pin(row_pointers_l, row_pointers_r, column_index_l)
+    k, ms = _AggKnobs(), C.c_float()
     rem = input_remote if input_remote is not None else input
     _check(lib().mggx_sag_np_div_tune(_dptr(output), _dptr(input), _dptr(rem), _dptr(row_pointers_l), _dptr(column_index_l),
                                       _dptr(row_pointers_r), _dptr(column_index_r), lb, ub, dim, nodePerPE, np_size,
-                                      C.byref(o), C.byref(w), C.byref(d), C.byref(ms)))
-    return w.value, d.value, ms.value
+                                      C.byref(o), C.byref(k), C.byref(ms)))
+    return {"ps": k.ps, "wpb": k.wpb, "dist": k.dist, "col_block_rows": k.col_block_rows}, ms.value
 
 
 def mgg_SAG_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb, ub, dim,
                    nodePerPE, peid, np_size, warpPerBlock, interleaved_dist, *, input_remote=None, accumulate=False,
-                   ld_in=0, ld_out=0, row_scale_out=None, relu=False):
+                   ld_in=0, ld_out=0, row_scale_out=None, relu=False, col_block_rows=0):
     """Argument order of the reference's mgg_SAG_np_div.  `input` is this rank's table; `input_remote` the
     global-id-indexed table the reference reaches with remote GETs (defaults to `input`, the single-GPU case).
     The reference adds into `output`; pass accumulate=True for that, the default overwrites."""
     flags = (AGG_ACCUMULATE if accumulate else 0) | (AGG_RELU if relu else 0)
     _agg(output, input, input_remote if input_remote is not None else input, row_pointers_l, column_index_l,
          row_pointers_r, column_index_r, lb, ub, dim, nodePerPE, np_size, warpPerBlock, interleaved_dist, flags, 0.0,
-         ld_in, ld_out, row_scale_out)
+         ld_in, ld_out, row_scale_out, col_block_rows)
 
 
 def mgg_GIN_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb, ub, dim,
                    nodePerPE, peid, np_size, warpPerBlock, interleaved_dist, eps, *, input_remote=None, ld_in=0,
-                   ld_out=0):
+                   ld_out=0, col_block_rows=0):
     _agg(output, input, input_remote if input_remote is not None else input, row_pointers_l, column_index_l,
          row_pointers_r, column_index_r, lb, ub, dim, nodePerPE, np_size, warpPerBlock, interleaved_dist, AGG_GIN,
-         float(eps), ld_in, ld_out, None)
+         float(eps), ld_in, ld_out, None, col_block_rows)
 
 
 def SAG_host(output, input, row_pointers, column_index, part_pointers, part2Node, lowbound, num_nodes, num_parts,

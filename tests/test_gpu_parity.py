@@ -154,9 +154,10 @@ def test_search_of_wpb_and_dist(gpu, rmat_graph, dim, gin):
     d = [to_dev(sh[k]) if len(sh[k]) else torch.zeros(1, dtype=torch.int32, device="cuda") for k in ("ptr_l", "col_l", "ptr_r", "col_r")]
     d_xl, d_x = to_dev(xl), to_dev(x)
     out = torch.full((R, dim), 7.5, device="cuda")
-    wpb, dist, ms = gpu.tune_np_div(out, d_xl, d[0], d[1], d[2], d[3], sh["lb"], sh["ub"], dim, sh["npp"], 16, input_remote=d_x,
-                                    gin_eps=0.25 if gin else None)
-    assert wpb in (4, 8, 16) and dist in (1, 2, 4, 8, 16) and ms > 0
+    kn, ms = gpu.tune_np_div(out, d_xl, d[0], d[1], d[2], d[3], sh["lb"], sh["ub"], dim, sh["npp"], 16, input_remote=d_x,
+                             gin_eps=0.25 if gin else None)
+    wpb, dist = kn["wpb"], kn["dist"]
+    assert kn["ps"] == 16 and wpb in (4, 8, 16) and dist in (1, 2, 4, 8, 16) and ms > 0 and kn["col_block_rows"] == -1
     kw = dict(flags=orc.GIN, eps=0.25) if gin else {}
     want, mag = oracle_agg(sh, xl, x, dim, **kw)
     assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "result left by the search")
@@ -176,7 +177,93 @@ def test_search_of_wpb_and_dist(gpu, rmat_graph, dim, gin):
         import ctypes as C
         gpu._check(gpu.lib().mggx_sag_np_div_tune(gpu._dptr(out), gpu._dptr(d_xl), gpu._dptr(d_x), gpu._dptr(d[0]), gpu._dptr(d[1]),
                                                   gpu._dptr(d[2]), gpu._dptr(d[3]), sh["lb"], sh["ub"], dim, sh["npp"], 16,
-                                                  C.byref(o), None, None, None))
+                                                  C.byref(o), None, None))
+
+
+@pytest.mark.parametrize("dim,block_rows,flags", [(16, 100, "plain"), (44, 64, "scale"), (41, 37, "gin"), (8, 300, "acc_relu"),
+                                                  (64, 128, "plain")])
+def test_column_blocked_order(gpu, rmat_graph, dim, block_rows, flags):
+    """The column-blocked partition order (whole graph, rows sorted by neighbor id): same sums as the plain order and
+    the oracle, with every epilogue; unsorted rows fall back to the plain order silently."""
+    import torch
+    V, ptr, col = rmat_graph
+    x = gpu.fill_normal((V, dim), seed=91)
+    sh = share_of(ptr, col, V, 1, 0)
+    d_ptr, d_col = to_dev(ptr), to_dev(col)
+    z, zc = torch.zeros(V + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    d_x = to_dev(x)
+    s = gpu.fill_uniform((V,), 0.5, 2.0, seed=92)
+    base = gpu.fill_normal((V, dim), seed=93)
+
+    def run(blk, ps, wpb, dist):
+        out = to_dev(base.copy()) if flags == "acc_relu" else torch.full((V, dim), 7.5, device="cuda")
+        if flags == "gin":
+            gpu.mgg_GIN_np_div(out, d_x, d_ptr, d_col, z, zc, 0, V, dim, V, 0, ps, wpb, dist, 0.5, col_block_rows=blk)
+        else:
+            gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, z, zc, 0, V, dim, V, 0, ps, wpb, dist, col_block_rows=blk,
+                               accumulate=flags == "acc_relu", relu=flags == "acc_relu",
+                               row_scale_out=to_dev(s) if flags == "scale" else None)
+        gpu.sync()
+        return out.cpu().numpy()
+
+    kw = {}
+    if flags == "gin":
+        kw = dict(flags=orc.GIN, eps=0.5)
+    want, mag = oracle_agg(sh, x, x, dim, **kw)
+    if flags == "scale":
+        want, mag = want * s[:, None], mag * s[:, None]
+    if flags == "acc_relu":
+        want, mag = np.maximum(want + base, 0), mag + np.abs(base)
+    for ps, wpb, dist in ((16, 4, 1), (4, 2, 3), (32, 8, 16), (0, 0, 0)):
+        got = run(block_rows, ps, wpb, dist)
+        assert "blocks=%d" % -(-V // block_rows) in gpu.last_agg_kernel()
+        assert_close_to_oracle(got, want, mag, FP32_TOL, "column-blocked ps=%d wpb=%d dist=%d" % (ps, wpb, dist))
+    plain = run(-1, 16, 4, 1)
+    assert "blocks=1" in gpu.last_agg_kernel()
+    assert_close_to_oracle(plain, want, mag, FP32_TOL, "plain order")
+    # rows not sorted by neighbor id: the request is honoured by falling back to the plain order
+    rng = np.random.default_rng(5)
+    col_u = col.copy()
+    for v in range(0, V, 3):
+        rng.shuffle(col_u[ptr[v]:ptr[v + 1]])
+    d_col_u = to_dev(col_u)
+    out = torch.full((V, dim), 7.5, device="cuda")
+    if flags == "plain":
+        gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col_u, z, zc, 0, V, dim, V, 0, 16, 4, 1, col_block_rows=block_rows)
+        gpu.sync()
+        assert "blocks=1" in gpu.last_agg_kernel()
+        assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "unsorted rows")
+
+
+def test_column_blocked_with_empty_rows_and_search(gpu):
+    """Rows without neighbors, rows whose neighbors all fall in one block, and the search over both orders."""
+    import torch
+    V, dim = 5000, 16
+    rng = np.random.default_rng(11)
+    deg = rng.integers(0, 400, V)
+    deg[rng.integers(0, V, 500)] = 0
+    ptr = np.zeros(V + 1, np.int32)
+    ptr[1:] = np.cumsum(deg)
+    col = np.concatenate([np.sort(rng.choice(V if v % 7 else 50, d, replace=d > 50)) for v, d in enumerate(deg)] + [np.zeros(0, np.int64)]).astype(np.int32)
+    x = gpu.fill_normal((V, dim), seed=94)
+    sh = share_of(ptr, col, V, 1, 0)
+    want, mag = oracle_agg(sh, x, x, dim)
+    d_ptr, d_col, d_x = to_dev(ptr), to_dev(col), to_dev(x)
+    z, zc = torch.zeros(V + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    out = torch.full((V, dim), 7.5, device="cuda")
+    gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, z, zc, 0, V, dim, V, 0, 16, 4, 2, col_block_rows=512)
+    gpu.sync()
+    assert "blocks=10" in gpu.last_agg_kernel()
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "column-blocked, empty rows")
+    out.fill_(7.5)
+    kn, ms = gpu.tune_np_div(out, d_x, d_ptr, d_col, z, zc, 0, V, dim, V, 0, col_block_rows=512)
+    assert kn["ps"] in (16, 32) and kn["col_block_rows"] == 512 and ms > 0
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "result left by the search")
+    out.fill_(7.5)
+    gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, z, zc, 0, V, dim, V, 0, 0, 0, 0)
+    gpu.sync()
+    assert "blocks=10" in gpu.last_agg_kernel()   # the remembered setting
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "remembered setting")
 
 
 def test_bad_arguments_return_errors_not_faults(gpu, rmat_graph):
@@ -189,7 +276,7 @@ def test_bad_arguments_return_errors_not_faults(gpu, rmat_graph):
     out = torch.zeros(V, 16, device="cuda")
     call = lambda **kw: gpu.mgg_SAG_np_div(out, x, d_ptr, d_col, z, z, 0, V, kw.get("dim", 16), kw.get("npp", V), 0,
                                            kw.get("ps", 16), kw.get("wpb", 4), kw.get("dist", 1), ld_in=kw.get("ld_in", 0))
-    for bad in (dict(dim=0), dict(dim=300), dict(wpb=17), dict(wpb=-1), dict(dist=-2), dict(ps=0), dict(npp=V - 1), dict(ld_in=8)):
+    for bad in (dict(dim=0), dict(dim=300), dict(wpb=17), dict(wpb=-1), dict(dist=-2), dict(ps=-1), dict(npp=V - 1), dict(ld_in=8)):
         with pytest.raises(gpu.MggxError):
             call(**bad)
     with pytest.raises(gpu.MggxError):
