@@ -29,6 +29,7 @@ struct mgg_runtime_options {
     const void *remote_table = nullptr;  // global-id-indexed feature table; nullptr = the input buffer
     bool accumulate = true;              // mgg_SAG_np_div adds into `output` as the reference does (:1458)
     bool synchronize = true;             // the reference waits for the device after every call (:835)
+    int col_block_rows = 0;              // column-blocked partition order: 0 = library decides, -1 = off, N = ids per block
 };
 inline mgg_runtime_options &mgg_options()
 {
@@ -122,6 +123,7 @@ inline void mgg_SAG_np_div(float *output, const float *input, const nidType *row
     (void)peid;
     mggx_agg_opts o{};
     o.flags = mgg_options().accumulate ? MGGX_AGG_ACCUMULATE : 0;
+    o.col_block_rows = mgg_options().col_block_rows;
     const void *remote = mgg_options().remote_table ? mgg_options().remote_table : input;
     mgg_finish_call(mggx_sag_np_div(output, input, remote, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb,
                                     ub, dim, nodePerPE, np_size, warpPerBlock, interleaved_dist, &o),
@@ -138,10 +140,30 @@ inline void mgg_GIN_np_div(float *output, const float *input, const nidType *row
     mggx_agg_opts o{};
     o.flags = MGGX_AGG_GIN;
     o.eps = eps;
+    o.col_block_rows = mgg_options().col_block_rows;
     const void *remote = mgg_options().remote_table ? mgg_options().remote_table : input;
     mgg_finish_call(mggx_sag_np_div(output, input, remote, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb,
                                     ub, dim, nodePerPE, np_size, warpPerBlock, interleaved_dist, &o),
                     "mgg_GIN_np_div_cuda");
+}
+
+// The reference finds (partSize, warpPerBlock, interleaved_dist) per dataset by launching one run per setting
+// (bench_MGG_DSE_dist_ps.py, bench_MGG_DSE_dist_wpb.py); this does the search on the caller's own buffers in one
+// call.  Later mgg_SAG_np_div calls on the same CSR arrays with warpPerBlock = interleaved_dist = 0 (and np_size 0
+// or the returned one) run with the returned setting.  `output` is overwritten.
+inline mggx_agg_knobs mgg_tune_np_div(float *output, const float *input, const nidType *row_pointers_l,
+                                      const nidType *column_index_l, const nidType *row_pointers_r,
+                                      const nidType *column_index_r, const nidType lb, const nidType ub, const int dim,
+                                      const int nodePerPE, const int np_size, float *best_ms = nullptr)
+{
+    mggx_agg_opts o{};
+    o.col_block_rows = mgg_options().col_block_rows;
+    mggx_agg_knobs k{};
+    const void *remote = mgg_options().remote_table ? mgg_options().remote_table : input;
+    mgg_finish_call(mggx_sag_np_div_tune(output, input, remote, row_pointers_l, column_index_l, row_pointers_r, column_index_r,
+                                         lb, ub, dim, nodePerPE, np_size, &o, &k, best_ms),
+                    "mgg_tune_np_div");
+    return k;
 }
 
 // Explicit partition arrays (from build_part), local rows only:

@@ -286,6 +286,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     if constexpr (BUF) g.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(a.win_base), 0, a.win_bytes, 0x00020000);
     g.zero = reinterpret_cast<const char *>(g_zero_row) + cofs;
     const int pad_id = BUF ? a.sentinel : -1;  // what a slot holds past the end of its partition
+    const bool lane_on = MODE == MODE_F32_STRIDED ? l < a.dim : NV * l < a.dim;
 
     float acc[NV];
 #pragma unroll
@@ -356,11 +357,21 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
                 constexpr int b = decltype(bb)::value;
                 if (__any(len > k0 + b * BATCH)) {
                     float v[BATCH][NV];
+                    int rid[BATCH];
                     static_for<0, BATCH>([&](auto tt) {
                         constexpr int t = decltype(tt)::value;
                         constexpr int k = b * BATCH + t;
-                        g.load(v[t], slot_bcast<LPR, k / IPL>(ids[k % IPL], slot_base));
+                        rid[t] = slot_bcast<LPR, k / IPL>(ids[k % IPL], slot_base);
+#pragma unroll
+                        for (int i = 0; i < NV; ++i) v[t][i] = 0.0f;
                     });
+                    // lanes past the row width issue no load at all: a quad of idle lanes costs the address unit nothing
+                    if (lane_on) {
+                        static_for<0, BATCH>([&](auto tt) {
+                            constexpr int t = decltype(tt)::value;
+                            g.load(v[t], rid[t]);
+                        });
+                    }
                     // keep every load of the batch in flight before the first sum waits on one
                     __builtin_amdgcn_sched_barrier(0);
                     static_for<0, BATCH>([&](auto tt) {
