@@ -89,6 +89,15 @@ int mggx_split_csr(const int *ptr, const int *col, int lb, int ub,
                    int *local_ptr, int *remote_ptr, int *local_col, int *remote_col,
                    int64_t *n_local, int64_t *n_remote);
 
+/* Compact staging of the remote rows of a share (no counterpart in the reference, which issues one nvshmem GET per
+ * remote neighbor, include/neighbor_utils.cuh:1432-1452; this is the list a pre-exchange of remote rows would fetch).
+ * fetch_ids = the distinct ids of remote_col, most referenced first, ties by ascending id; remote_col_compact[e] =
+ * position of remote_col[e] in fetch_ids.  Staging row i of the remote table = feature row fetch_ids[i]
+ * (mggx_gather_rows) and passing remote_col_compact as d_col_r gives the same sums, from a table with one row per
+ * distinct id and the hot rows packed together.  Call with both outputs NULL to get *n_unique first. */
+int mggx_compact_remote(const int *remote_col, int64_t n_remote, int *remote_col_compact, int *fetch_ids,
+                        int64_t *n_unique);
+
 /* build_part<int> (include/neighbor_utils.cuh:411-460).  part_ptr has
  * num_parts+1 entries, part2node num_parts, node2part num_nodes+2 (the
  * reference's layout).  compat != 0 reproduces the reference's terminal entry
@@ -183,7 +192,7 @@ typedef struct mggx_agg_knobs {
  * (>= 20 neighbors per block and row), the partitions are walked block by block of neighbor ids, so the part of the
  * feature table in use at any time is small enough to stay in cache; each block leaves a partial row in library
  * scratch and a second kernel sums them in block order and applies the epilogue.  Same result up to summation order.
- * The partition plan of (d_ptr_l, d_ptr_r, rows, ps) is built on first use and
+ * The partition plan of (d_ptr_l, d_ptr_r, d_col_r, rows, ps) -- and d_col_l for the column-blocked order -- is built on first use and
  * cached by pointer identity: the CSR arrays must not be rewritten in place
  * while cached (mggx_release_cached() drops the cache). */
 int mggx_sag_np_div(float *d_out, const void *d_in_local, const void *d_in_remote,
@@ -261,6 +270,10 @@ int mggx_dense_xw_bf16(void *d_out, const void *d_x, const void *d_w_bf16, int64
  * cudnnSoftmaxForward(ACCURATE, MODE_CHANNEL) on (n, c, 1, 1) == stable row
  * softmax.  In place (d_out == d_in) is allowed. */
 int mggx_softmax_rows(float *d_out, const float *d_in, int64_t n, int c, int64_t ld_in, int64_t ld_out);
+
+/* d_dst row i = d_table row d_ids[i], i < n; rows of row_bytes bytes (a multiple of 16, both tables 16-byte aligned):
+ * stages a compact remote table from a table indexed by global id. */
+int mggx_gather_rows(void *d_dst, const void *d_table, const int *d_ids, int64_t n, size_t row_bytes);
 
 /* fp32 -> bf16 (round to nearest even) for staging bf16 feature tables. */
 int mggx_cast_f32_to_bf16(void *d_dst, const float *d_src, int64_t n);

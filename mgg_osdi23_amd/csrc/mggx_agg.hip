@@ -625,10 +625,13 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     // 0 = let the library choose (from sweeps on the benchmark graphs): 8 wavefronts; with few slots per wavefront
     // (wide rows) 16 rounds, so a workgroup still covers a few thousand neighbors; otherwise a workgroup tile of
     // about 8 rows' worth of partitions (most rows then finish inside one workgroup), between 1 and 16 rounds.
-    if (wpb == 0) wpb = 8;
+    // Column-blocked plans (long rows by construction): 4 wavefronts, 4 rounds for narrow rows.
+    if (wpb == 0) wpb = blocked ? 4 : 8;
     if (dist == 0) {
         if (slots <= 4) {
             dist = 16;
+        } else if (blocked) {
+            dist = 4;
         } else {
             const double per_row = (double)plan->num_parts / (double)plan->rows;
             const long long want = (long long)(8.0 * per_row / (double)(wpb * slots) + 0.999);

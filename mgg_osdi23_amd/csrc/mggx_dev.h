@@ -57,6 +57,7 @@ struct Plan {
     // `rows` = blocks * real_rows virtual rows; virtual row c * real_rows + v holds row v's neighbors inside block c,
     // so the descriptor order walks the feature table block by block.  Plain plans: blocks == 1, rows == real_rows.
     const int *d_col_l = nullptr;  // cache key of blocked plans (they depend on the column values)
+    const int *d_col_r = nullptr;  // cache key of plans with remote edges (max_col_r depends on the values)
     int real_rows = 0;
     int block_rows = 0;
     int blocks = 1;

@@ -89,6 +89,51 @@ MGGX_EXPORT int mggx_split_csr(const int *ptr, const int *col, int lb, int ub,
 }
 
 // ---------------------------------------------------------------------------
+// Compact staging of the remote rows.  The reference fetches every remote neighbor with its own GET
+// (include/neighbor_utils.cuh:1432-1452); a share only ever touches the distinct ids in remote_col, so the staged
+// table needs one row per distinct id.  They are ordered most-referenced first (ties by ascending id), which packs
+// the hot rows into the same cache lines, and remote_col is rewritten to positions in that order.
+MGGX_EXPORT int mggx_compact_remote(const int *remote_col, int64_t n_remote, int *remote_col_compact, int *fetch_ids,
+                                    int64_t *n_unique)
+{
+    if (n_remote < 0 || (n_remote && !remote_col)) return fail(MGGX_EINVAL, "compact_remote: bad remote_col");
+    if (n_remote > std::numeric_limits<int>::max()) return fail(MGGX_ELIMIT, "compact_remote: more than 2^31-1 edges");
+    try {
+        std::vector<int> sorted(remote_col, remote_col + n_remote);
+        __gnu_parallel::sort(sorted.begin(), sorted.end());
+        std::vector<int> ids, cnt;
+        for (int64_t i = 0; i < n_remote;) {
+            int64_t j = i;
+            while (j < n_remote && sorted[j] == sorted[i]) ++j;
+            if (sorted[i] < 0) return fail(MGGX_EFORMAT, "compact_remote: negative neighbor id %d", sorted[i]);
+            ids.push_back(sorted[i]);
+            cnt.push_back((int)(j - i));
+            i = j;
+        }
+        const int64_t u = (int64_t)ids.size();
+        if (n_unique) *n_unique = u;
+        if (!remote_col_compact && !fetch_ids) return MGGX_OK;
+        if (!remote_col_compact || !fetch_ids) return fail(MGGX_EINVAL, "compact_remote: pass both output arrays or neither");
+        std::vector<int> order((size_t)u);
+        for (int64_t i = 0; i < u; ++i) order[(size_t)i] = (int)i;
+        __gnu_parallel::stable_sort(order.begin(), order.end(), [&](int x, int y) { return cnt[(size_t)x] > cnt[(size_t)y]; });
+        std::vector<int> rank((size_t)u);  // position in staging order of the i-th smallest id
+        for (int64_t pos = 0; pos < u; ++pos) {
+            rank[(size_t)order[(size_t)pos]] = (int)pos;
+            fetch_ids[pos] = ids[(size_t)order[(size_t)pos]];
+        }
+#pragma omp parallel for schedule(static)
+        for (int64_t e = 0; e < n_remote; ++e) {
+            const int64_t i = std::lower_bound(ids.begin(), ids.end(), remote_col[e]) - ids.begin();
+            remote_col_compact[e] = rank[(size_t)i];
+        }
+    } catch (const std::bad_alloc &) {
+        return fail(MGGX_ENOMEM, "compact_remote: out of host memory for %lld edges", (long long)n_remote);
+    }
+    return MGGX_OK;
+}
+
+// ---------------------------------------------------------------------------
 // Neighbor-partition arrays (reference: build_part, include/neighbor_utils.cuh:411-460).
 // Partition p of node i covers edges [indptr[i] + k*ps, min(.. + ps, indptr[i+1])).
 // node2part is the exclusive prefix of partition counts with the total repeated

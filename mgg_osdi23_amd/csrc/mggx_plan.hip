@@ -377,14 +377,15 @@ int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int row
 {
     State &s = state();
     for (Plan *p : s.plans)
-        if (p->d_ptr_l == d_ptr_l && p->d_ptr_r == d_ptr_r && p->rows == rows && p->ps == ps && !p->d_part_ptr && p->blocks == 1 &&
-            !p->unsuitable) {
+        if (p->d_ptr_l == d_ptr_l && p->d_ptr_r == d_ptr_r && p->d_col_r == d_col_r && p->rows == rows && p->ps == ps &&
+            !p->d_part_ptr && p->blocks == 1 && !p->unsuitable) {
             *out = p;
             return MGGX_OK;
         }
     Plan *p = new Plan;
     p->d_ptr_l = d_ptr_l;
     p->d_ptr_r = d_ptr_r;
+    p->d_col_r = d_col_r;  // the plan holds the largest remote id
     p->rows = rows;
     p->real_rows = rows;
     p->ps = ps;

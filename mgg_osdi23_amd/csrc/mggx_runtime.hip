@@ -237,6 +237,18 @@ __global__ void __launch_bounds__(256) k_cast_bf16(unsigned short *__restrict__ 
     }
 }
 
+// dst row i = table row ids[i]; rows of v16 16-byte pieces
+__global__ void __launch_bounds__(256) k_gather_rows(int4 *__restrict__ dst, const int4 *__restrict__ table, const int *__restrict__ ids,
+                                                     long long n, int v16)
+{
+    const long long total = n * v16;
+    for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (long long)gridDim.x * 256) {
+        const long long i = idx / v16;
+        const int p = (int)(idx % v16);
+        dst[idx] = table[(long long)ids[i] * v16 + p];
+    }
+}
+
 }  // namespace
 
 MGGX_EXPORT int mggx_copy_bytes(void *d_dst, const void *d_src, size_t n)
@@ -248,6 +260,21 @@ MGGX_EXPORT int mggx_copy_bytes(void *d_dst, const void *d_src, size_t n)
     if (blocks > 256 * 64) blocks = 256 * 64;
     k_copy16<<<dim3((unsigned)blocks), dim3(256), 0, state().stream>>>((int4 *)d_dst, (const int4 *)d_src, n16);
     MGGX_LAUNCH_CHECK("k_copy16");
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_gather_rows(void *d_dst, const void *d_table, const int *d_ids, int64_t n, size_t row_bytes)
+{
+    if (n < 0 || (n && (!d_dst || !d_table || !d_ids)) || row_bytes == 0 || (row_bytes % 16) ||
+        ((reinterpret_cast<uintptr_t>(d_dst) | reinterpret_cast<uintptr_t>(d_table)) & 15u))
+        return fail(MGGX_EINVAL, "gather_rows: NULL pointer, or rows not 16-byte multiples / aligned");
+    if (!n) return MGGX_OK;
+    const long long total = (long long)n * (long long)(row_bytes / 16);
+    long long blocks = (total + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    k_gather_rows<<<dim3((unsigned)blocks), dim3(256), 0, state().stream>>>((int4 *)d_dst, (const int4 *)d_table, d_ids, (long long)n,
+                                                                             (int)(row_bytes / 16));
+    MGGX_LAUNCH_CHECK("k_gather_rows");
     return MGGX_OK;
 }
 

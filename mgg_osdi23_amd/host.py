@@ -52,10 +52,10 @@ EXPORTS = [
     "mggx_last_error", "mggx_version", "mggx_init", "mggx_device_name", "mggx_set_stream", "mggx_sync",
     "mggx_malloc", "mggx_free", "mggx_memset", "mggx_memcpy_h2d", "mggx_memcpy_d2h", "mggx_memcpy_d2d",
     "mggx_timer_create", "mggx_timer_start", "mggx_timer_stop", "mggx_timer_elapsed_ms", "mggx_timer_destroy",
-    "mggx_release_cached", "mggx_range_partition", "mggx_split_csr", "mggx_build_part", "mggx_graph_read",
+    "mggx_release_cached", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
     "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_mlp2_xw", "mggx_spmm",
-    "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
+    "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_gather_rows", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
 ]
 
 
@@ -111,6 +111,23 @@ def split_CSR(ptr: np.ndarray, col: np.ndarray, lb: int, ub: int):
     _check(lib().mggx_split_csr(_iptr(ptr), _iptr(col), lb, ub, _iptr(lp), _iptr(rp), _iptr(lc), _iptr(rc),
                                 C.byref(nl), C.byref(nr)))
     return lp, rp, lc, rc
+
+
+def compact_remote(remote_col: np.ndarray):
+    """-> (remote_col_compact, fetch_ids): the distinct remote ids in staging order (most referenced first) and the
+    column array rewritten to positions in it; stage `table[fetch_ids]` as the remote table."""
+    rc = np.ascontiguousarray(remote_col, dtype=np.int32)
+    nu = C.c_int64()
+    _check(lib().mggx_compact_remote(_iptr(rc), C.c_int64(len(rc)), None, None, C.byref(nu)))
+    out = np.zeros(len(rc), np.int32)
+    ids = np.zeros(nu.value, np.int32)
+    _check(lib().mggx_compact_remote(_iptr(rc), C.c_int64(len(rc)), _iptr(out), _iptr(ids), C.byref(nu)))
+    return out, ids
+
+
+def gather_rows(dst, table, ids, n: int, row_bytes: int) -> None:
+    """dst row i = table row ids[i] on the device (staging a compact remote table)."""
+    _check(lib().mggx_gather_rows(_dptr(dst), _dptr(table), _dptr(ids), C.c_int64(n), C.c_size_t(row_bytes)))
 
 
 def build_part(indptr: np.ndarray, num_nodes: int, part_size: int, compat: bool = True):
@@ -293,7 +310,7 @@ def _agg(out, in_local, in_remote, ptr_l, col_l, ptr_r, col_r, lb, ub, dim, npp,
     o.d_row_scale_out = row_scale_out.data_ptr() if row_scale_out is not None else None
     o.in_dtype = BF16 if in_local.dtype == torch.bfloat16 else F32
     o.col_block_rows = col_block_rows
-    _pin(ptr_l, ptr_r, col_l)
+    _pin(ptr_l, ptr_r, col_l, col_r)
     _check(lib().mggx_sag_np_div(_dptr(out), _dptr(in_local), _dptr(in_remote), _dptr(ptr_l), _dptr(col_l),
                                  _dptr(ptr_r), _dptr(col_r), lb, ub, dim, npp, ps, wpb, dist, C.byref(o)))
 
@@ -313,7 +330,7 @@ def tune_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, c
     o.d_row_scale_out = row_scale_out.data_ptr() if row_scale_out is not None else None
     o.in_dtype = BF16 if input.dtype == torch.bfloat16 else F32
     o.col_block_rows = col_block_rows
-    _pin(row_pointers_l, row_pointers_r, column_index_l)
+    _pin(row_pointers_l, row_pointers_r, column_index_l, column_index_r)
     k, ms = _AggKnobs(), C.c_float()
     rem = input_remote if input_remote is not None else input
     _check(lib().mggx_sag_np_div_tune(_dptr(output), _dptr(input), _dptr(rem), _dptr(row_pointers_l), _dptr(column_index_l),

@@ -256,3 +256,27 @@ def test_generators_are_deterministic_and_well_formed():
     assert abs(float(x.mean())) < 0.01 and abs(float(x.std()) - 1.0) < 0.01
     u = host.fill_uniform((100000,), -1.0, 1.0, seed=2)
     assert u.min() >= -1.0 and u.max() < 1.0 and abs(float(u.mean())) < 0.01
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_compact_remote_staging_order(seed):
+    """The distinct remote ids, most referenced first (ties by ascending id), and the rewritten column array:
+    checked against numpy's unique/argsort and by the round trip fetch_ids[compact] == remote_col."""
+    rng = np.random.default_rng(seed)
+    V = 5000
+    ptr, col = host.gen_rmat(13, V, 60_000, seed=seed, scramble=bool(seed % 2))
+    npp, lb, ub = host.range_partition(V, 4, seed % 4)
+    _, rp, _, rc = host.split_CSR(ptr, col, lb, ub)
+    compact, ids = host.compact_remote(rc)
+    assert np.array_equal(ids[compact], rc)
+    uniq, cnt = np.unique(rc, return_counts=True)
+    order = np.argsort(-cnt, kind="stable")       # ties keep ascending id
+    assert np.array_equal(ids, uniq[order])
+    assert not np.any((ids >= lb) & (ids < ub))   # remote ids only
+    # degenerate inputs
+    c0, i0 = host.compact_remote(np.zeros(0, np.int32))
+    assert len(c0) == 0 and len(i0) == 0
+    c1, i1 = host.compact_remote(np.array([7, 7, 7], np.int32))
+    assert c1.tolist() == [0, 0, 0] and i1.tolist() == [7]
+    with pytest.raises(host.MggxError):
+        host.compact_remote(np.array([3, -1], np.int32))

@@ -266,6 +266,36 @@ def test_column_blocked_with_empty_rows_and_search(gpu):
     assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "remembered setting")
 
 
+@pytest.mark.parametrize("dim,dtype", [(16, "f32"), (44, "f32"), (128, "bf16")])
+def test_compact_remote_table_gives_the_same_sums(gpu, rmat_graph, dim, dtype):
+    """Remote rows staged compactly (one row per distinct remote id, most referenced first) with the column array
+    rewritten to match: bit-identical output to the table indexed by global id, and within tolerance of the oracle."""
+    import torch
+    V, ptr, col = rmat_graph
+    x = gpu.fill_normal((V, dim), seed=70)
+    sh = share_of(ptr, col, V, 4, 2)
+    lb, ub = sh["lb"], sh["ub"]
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    d_x = to_dev(x).to(td)
+    d_xl = d_x[lb:ub].clone()
+    compact, ids = gpu.compact_remote(sh["col_r"])
+    d_ids = to_dev(ids)
+    staged = torch.full((len(ids), dim), 3.0, device="cuda", dtype=td)
+    gpu.gather_rows(staged, d_x, d_ids, len(ids), dim * d_x.element_size())
+    gpu.sync()
+    assert torch.equal(staged, d_x[d_ids.long()])
+    d = [to_dev(sh["ptr_l"]), to_dev(sh["col_l"]), to_dev(sh["ptr_r"])]
+    out_a = torch.full((ub - lb, dim), 7.5, device="cuda")
+    out_b = torch.full((ub - lb, dim), 7.5, device="cuda")
+    gpu.mgg_SAG_np_div(out_a, d_xl, d[0], d[1], d[2], to_dev(sh["col_r"]), lb, ub, dim, sh["npp"], 0, 16, 4, 2, input_remote=d_x)
+    gpu.mgg_SAG_np_div(out_b, d_xl, d[0], d[1], d[2], to_dev(compact), lb, ub, dim, sh["npp"], 0, 16, 4, 2, input_remote=staged)
+    gpu.sync()
+    assert torch.equal(out_a, out_b)
+    xr = d_x.float().cpu().numpy()
+    want, mag = oracle_agg(sh, xr[lb:ub], xr, dim)
+    assert_close_to_oracle(out_b.cpu().numpy(), want, mag, FP32_TOL, "compact remote table")
+
+
 def test_bad_arguments_return_errors_not_faults(gpu, rmat_graph):
     """Shapes the kernels are not built for are refused on the host, with a message, before any launch."""
     import torch
