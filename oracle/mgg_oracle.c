@@ -12,7 +12,7 @@
  * (per-warp partial sums, committed warp by warp) and `*_f64` accumulates in
  * double as the tolerance anchor.
  *
- * How each function is pinned (see tests/test_oracle_*.py):
+ * How each function is pinned (tests/test_cpu_graph_prep.py, tests/test_cpu_oracle_numerics.py):
  *   orc_range_partition  closed form + brute force
  *   orc_split_csr        reference templates compiled into oracle/_ref, golden fixtures, invariants
  *   orc_build_part       same (incl. the missing-sentinel and node2Part+2 quirks)
