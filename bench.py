@@ -140,8 +140,9 @@ def bench_gcn2(args, torch, host):
     deg = np.diff(ptr).astype(np.float64)
     s = (1.0 / np.sqrt(np.maximum(deg, 1.0))).astype(np.float32)
 
-    # Device layout: the 41-wide layer is kept with a row stride of 44 floats (zero padding columns), so its rows
-    # are 16-byte aligned and move as whole dwordx4 loads; bytes and flops are still counted at width 41.
+    # Device layout: the 41-wide layer is computed at width 44 (zero padding columns) in tables with a row pitch of 48
+    # floats, so its rows move as whole dwordx4 loads and start on 64-byte boundaries (a 192-byte row then touches two
+    # 128-byte lines, never three); bytes and flops are still counted at width 41.
     ldo = (out_dim + 3) & ~3
     W2p = np.zeros((hidden, ldo), np.float32)
     W2p[:, :out_dim] = W2
@@ -156,8 +157,9 @@ def bench_gcn2(args, torch, host):
     d_s = torch.from_numpy(s).to(dev)
     d_Y1 = torch.empty(V, hidden, device=dev)
     d_H1 = torch.empty(V, hidden, device=dev)
-    d_Y2 = torch.empty(V, ldo, device=dev)
-    d_H2 = torch.empty(V, ldo, device=dev)
+    pitch = max(ldo, args.pitch41 or 48)  # row pitch of the 41-wide tables in floats
+    d_Y2 = torch.zeros(V, pitch, device=dev)
+    d_H2 = torch.zeros(V, pitch, device=dev)
     d_P = torch.empty(V, out_dim, device=dev)
 
     d_Y1.zero_()
@@ -165,15 +167,15 @@ def bench_gcn2(args, torch, host):
     k1 = Knobs(args, lambda ps, blk: host.tune_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, ps,
                                                       row_scale_out=d_s, col_block_rows=blk))
     k2 = Knobs(args, lambda ps, blk: host.tune_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, ps,
-                                                      row_scale_out=d_s, col_block_rows=blk))
+                                                      row_scale_out=d_s, col_block_rows=blk, ld_in=pitch, ld_out=pitch))
     stages = [
         lambda: host.dense_forward(d_Y1, d_X, d_W1, V, in_dim, hidden, row_scale=d_s),
         lambda: host.mgg_SAG_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, k1.ps, k1.wpb, k1.dist,
                                     row_scale_out=d_s, col_block_rows=k1.blk),
-        lambda: host.dense_forward(d_Y2, d_H1, d_W2, V, hidden, ldo, row_scale=d_s),
+        lambda: host.dense_forward(d_Y2, d_H1, d_W2, V, hidden, ldo, row_scale=d_s, ld_out=pitch),
         lambda: host.mgg_SAG_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, 0, k2.ps, k2.wpb, k2.dist,
-                                    row_scale_out=d_s, col_block_rows=k2.blk),
-        lambda: host.softmax_forward(d_P, d_H2, V, out_dim, ld_in=ldo),
+                                    row_scale_out=d_s, col_block_rows=k2.blk, ld_in=pitch, ld_out=pitch),
+        lambda: host.softmax_forward(d_P, d_H2, V, out_dim, ld_in=pitch),
     ]
     names = ["dense1", "agg1", "dense2", "agg2", "softmax"]
     k1.observe(host, stages[1])
@@ -591,6 +593,7 @@ def main():
     ap.add_argument("--small", action="store_true", help="tiny graph, for a quick functional run")
     ap.add_argument("--big-scale", type=int, default=0, help="--workload big: divide every size by 2^k")
     ap.add_argument("--unfused-mlp", action="store_true", help="--workload gin: run each MLP as two dense updates instead of the fused kernel")
+    ap.add_argument("--pitch41", type=int, default=0, help="--workload gcn2: row pitch in floats of the 41-wide tables (default 48; at least 44)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
