@@ -225,7 +225,8 @@ int mggx_sag_parts(float *d_out, const float *d_in, const int *d_row_ptr, const 
 
 /* SpMM_cuda_kernel via sparse_beg_forward / sparse_hidden_forward
  * (include/gnn_kernel.cuh:9-71, gnn_layer.cuh:86-161): whole graph on one GPU,
- * out[v,:] += sum_{u in N(v)} in[u,:]. */
+ * out[v,:] += sum_{u in N(v)} in[u,:].  ps = 0 / wpb = 0 let the library choose; the rounds per wavefront and the
+ * partition order follow the same rules as mggx_sag_np_div. */
 int mggx_spmm(float *d_out, const float *d_in, const int *d_row_ptr, const int *d_col,
               int num_nodes, int dim, int ps, int wpb);
 

@@ -916,11 +916,13 @@ MGGX_EXPORT int mggx_spmm(float *d_out, const float *d_in, const int *d_row_ptr,
 {
     int rc = mggx::ensure_init();
     if (rc) return rc;
-    if (!d_row_ptr || num_nodes < 0 || ps < 1) return fail(MGGX_EINVAL, "spmm: bad argument");
-    mggx::Plan *plan = nullptr;
-    rc = mggx::plan_get(d_row_ptr, nullptr, nullptr, num_nodes, ps, &plan);
-    if (rc) return rc;
+    if (!d_row_ptr || num_nodes < 0 || ps < 0) return fail(MGGX_EINVAL, "spmm: bad argument");
     mggx_agg_opts o{};
     o.flags = MGGX_AGG_ACCUMULATE;
-    return mggx::run_agg(plan, d_out, d_in, nullptr, d_col, nullptr, 0, dim, wpb, 1, o);
+    mggx::GraphInfo *g = nullptr;
+    rc = mggx::graph_info(d_row_ptr, nullptr, num_nodes, &g);
+    if (rc) return rc;
+    // the whole graph on one GPU: the same knob rules (and column-blocked order for long rows) as mggx_sag_np_div
+    mggx::Knobs k = mggx::resolve_knobs(*g, dim, MGGX_F32, ps, wpb, 0, 0);
+    return mggx::run_knobs(*g, k, d_out, d_in, nullptr, d_row_ptr, d_col, nullptr, nullptr, 0, num_nodes, dim, o);
 }

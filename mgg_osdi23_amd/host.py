@@ -368,7 +368,7 @@ def SAG_host(output, input, row_pointers, column_index, part_pointers, part2Node
 
 
 def SpMM(output, input, row_pointers, column_index, num_nodes, dim, partSize, warpPerBlock):
-    _pin(row_pointers)
+    _pin(row_pointers, column_index)
     _check(lib().mggx_spmm(_dptr(output), _dptr(input), _dptr(row_pointers), _dptr(column_index), num_nodes, dim,
                            partSize, warpPerBlock))
 

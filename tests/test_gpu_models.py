@@ -229,4 +229,14 @@ def test_full_size_whole_graph_gcn_widths(gpu):
     out = torch.empty(V, 16, device="cuda")
     gpu.mgg_SAG_np_div(out, ones, d_ptr, d_col, zp, zc, 0, V, 16, V, 0, 16, 8, 16)
     gpu.sync()
+    assert "blocks=5" in gpu.last_agg_kernel()  # long sorted rows: the library's rule picks the column-blocked order
     assert np.array_equal(out.cpu().numpy()[:, 0], np.diff(ptr).astype(np.float32))
+    gpu.mgg_SAG_np_div(out, ones, d_ptr, d_col, zp, zc, 0, V, 16, V, 0, 16, 8, 16, col_block_rows=-1)
+    gpu.sync()
+    assert "blocks=1 " in gpu.last_agg_kernel() + " "
+    assert np.array_equal(out.cpu().numpy()[:, 0], np.diff(ptr).astype(np.float32))
+    acc = torch.ones(V, 16, device="cuda")  # the single-GPU SpMM entry point adds into its output
+    gpu.SpMM(acc, ones, d_ptr, d_col, V, 16, 16, 8)
+    gpu.sync()
+    assert "blocks=5" in gpu.last_agg_kernel()
+    assert np.array_equal(acc.cpu().numpy()[:, 3], np.diff(ptr).astype(np.float32) + 1.0)
