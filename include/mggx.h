@@ -159,6 +159,11 @@ int mggx_build_part_device(const int *d_indptr, int num_nodes, int part_size, in
 int mggx_split_csr_device(const int *d_ptr, const int *d_col, int lb, int ub, int *d_local_ptr, int *d_remote_ptr,
                           int *d_local_col, int *d_remote_col, int64_t *n_local, int64_t *n_remote);
 
+/* mggx_compact_remote on the GPU (sort, run-length encode, sort by count, remap): d_remote_col is the device copy of
+ * the remote column array; same two-call protocol, bit-identical outputs (device arrays).  Synchronises. */
+int mggx_compact_remote_device(const int *d_remote_col, int64_t n_remote, int *d_remote_col_compact, int *d_fetch_ids,
+                               int64_t *n_unique);
+
 /* ---- aggregation ---- */
 
 typedef struct mggx_agg_opts {

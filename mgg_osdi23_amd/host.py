@@ -54,7 +54,7 @@ EXPORTS = [
     "mggx_timer_create", "mggx_timer_start", "mggx_timer_stop", "mggx_timer_elapsed_ms", "mggx_timer_destroy",
     "mggx_release_cached", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
-    "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_mlp2_xw", "mggx_spmm",
+    "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_compact_remote_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_mlp2_xw", "mggx_spmm",
     "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_gather_rows", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
 ]
 
@@ -123,6 +123,17 @@ def compact_remote(remote_col: np.ndarray):
     ids = np.zeros(nu.value, np.int32)
     _check(lib().mggx_compact_remote(_iptr(rc), C.c_int64(len(rc)), _iptr(out), _iptr(ids), C.byref(nu)))
     return out, ids
+
+
+def compact_remote_device(d_remote_col, n_remote: int):
+    """compact_remote on the GPU -> (remote_col_compact, fetch_ids) as device tensors."""
+    import torch
+    nu = C.c_int64()
+    _check(lib().mggx_compact_remote_device(_dptr(d_remote_col), C.c_int64(n_remote), None, None, C.byref(nu)))
+    out = torch.zeros(max(n_remote, 1), dtype=torch.int32, device=d_remote_col.device)
+    ids = torch.zeros(max(nu.value, 1), dtype=torch.int32, device=d_remote_col.device)
+    _check(lib().mggx_compact_remote_device(_dptr(d_remote_col), C.c_int64(n_remote), _dptr(out), _dptr(ids), C.byref(nu)))
+    return out[:n_remote], ids[: nu.value]
 
 
 def gather_rows(dst, table, ids, n: int, row_bytes: int) -> None:

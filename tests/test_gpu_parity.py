@@ -279,6 +279,8 @@ def test_compact_remote_table_gives_the_same_sums(gpu, rmat_graph, dim, dtype):
     d_x = to_dev(x).to(td)
     d_xl = d_x[lb:ub].clone()
     compact, ids = gpu.compact_remote(sh["col_r"])
+    d_compact, d_ids_dev = gpu.compact_remote_device(to_dev(sh["col_r"]), len(sh["col_r"]))  # the same on the GPU: bit-identical
+    assert np.array_equal(d_compact.cpu().numpy(), compact) and np.array_equal(d_ids_dev.cpu().numpy(), ids)
     d_ids = to_dev(ids)
     staged = torch.full((len(ids), dim), 3.0, device="cuda", dtype=td)
     gpu.gather_rows(staged, d_x, d_ids, len(ids), dim * d_x.element_size())
