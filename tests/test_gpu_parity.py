@@ -516,7 +516,7 @@ def test_split_csr_device_bit_exact(gpu, rmat_graph, num_gpus, pe):
 
 # --------------------------------------------------------------------------- dense update and softmax
 @pytest.mark.parametrize("n,d1,d2", [(1000, 602, 16), (1000, 16, 41), (777, 100, 64), (512, 64, 64), (300, 64, 47),
-                                     (256, 128, 128), (65, 7, 3), (1, 1, 1), (130, 33, 130)])
+                                     (256, 128, 128), (65, 7, 3), (1, 1, 1), (130, 33, 130), (100, 1500, 64), (70, 65, 16)])
 def test_dense_update(gpu, n, d1, d2):
     import torch
     x = gpu.fill_normal((n, d1), seed=20)
@@ -527,6 +527,13 @@ def test_dense_update(gpu, n, d1, d2):
     want = orc.dense(x, w, f64=True)
     mag = np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64)
     assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "dense %dx%dx%d" % (n, d1, d2))
+    # the same rows inside a wider table (row pitch d1 + 3, unaligned rows), poisoned padding
+    xp = np.full((n, d1 + 3), np.nan, np.float32)
+    xp[:, :d1] = x
+    out = torch.full((n, d2), 3.0, device="cuda")
+    gpu.dense_forward(out, to_dev(xp), to_dev(w), n, d1, d2, ld_x=d1 + 3)
+    gpu.sync()
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "dense %dx%dx%d, strided X" % (n, d1, d2))
 
 
 def test_dense_closed_forms_and_epilogue(gpu):
