@@ -20,6 +20,10 @@
  *     always has ld == dim).
  *   - all device work is issued on the stream set by mggx_set_stream()
  *     (default: the null stream) and is asynchronous unless stated.
+ *   - after a first call of the same shape (which builds the cached plan and grows the library's scratch), the
+ *     compute entry points only launch kernels -- no allocation, memset or synchronisation -- and may be captured
+ *     into a HIP graph; the scratch block is reallocated when a later call needs more, so warm up the largest call
+ *     before capturing.  mggx_sag_np_div_tune, the *_device preparation calls and first calls synchronise.
  *   - one host thread per device at a time; the library keeps per-process
  *     state (stream, workspace, plan cache) without locks, as MGG runs one
  *     host thread per GPU.

@@ -59,6 +59,58 @@ def test_gcn_two_layer_forward(gpu, pad):
     assert np.allclose(P.cpu().numpy().sum(1), 1.0, atol=1e-5)
 
 
+def test_forward_replayed_from_a_hip_graph(gpu):
+    """After one eager call has built the plan and sized the workspace, a forward issues kernels only (no
+    allocation, no memset, no synchronisation), so it can be captured into a HIP graph.  Every replay, with eager work
+    of the library between replays, must reproduce the eager result bit for bit."""
+    import torch
+    V, in_dim, hidden, out_dim = 5000, 64, 16, 40
+    ptr, col = gpu.gen_rmat(13, V, 150_000, seed=9)
+    d_ptr, d_col = to_dev(ptr), to_dev(col)
+    zp, zc = zeros_i32(V + 1), zeros_i32()
+    s = to_dev((1.0 / np.sqrt(np.diff(ptr))).astype(np.float32))
+    X = to_dev(gpu.fill_normal((V, in_dim), seed=1))
+    W1, W2 = to_dev(gpu.glorot(in_dim, hidden, seed=2)), to_dev(gpu.glorot(hidden, out_dim, seed=3))
+    Y1, H1 = torch.empty(V, hidden, device="cuda"), torch.empty(V, hidden, device="cuda")
+    Y2, H2 = torch.empty(V, out_dim, device="cuda"), torch.empty(V, out_dim, device="cuda")
+    P = torch.empty(V, out_dim, device="cuda")
+
+    def forward():
+        gpu.dense_forward(Y1, X, W1, V, in_dim, hidden, row_scale=s)
+        gpu.mgg_SAG_np_div(H1, Y1, d_ptr, d_col, zp, zc, 0, V, hidden, V, 0, 16, 4, 2, row_scale_out=s)
+        gpu.dense_forward(Y2, H1, W2, V, hidden, out_dim, row_scale=s)
+        gpu.mgg_SAG_np_div(H2, Y2, d_ptr, d_col, zp, zc, 0, V, out_dim, V, 0, 16, 4, 2, row_scale_out=s)
+        gpu.softmax_forward(P, H2, V, out_dim)
+
+    side = torch.cuda.Stream()
+    try:
+        with torch.cuda.stream(side):
+            gpu.use_torch_stream()
+            # eager first: builds the plans and grows the workspace to the largest size any later call needs
+            # (growing it again would free the block a captured graph still points to)
+            gpu.mgg_SAG_np_div(H2, Y2, d_ptr, d_col, zp, zc, 0, V, out_dim, V, 0, 16, 8, 1)
+            forward()
+            side.synchronize()
+            want = P.clone()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                gpu.use_torch_stream()      # the capturing stream
+                forward()
+            for i in range(3):
+                P.fill_(-1.0)
+                H1.fill_(float(i))
+                graph.replay()
+                side.synchronize()
+                assert torch.equal(P, want), "replay %d differs from the eager forward" % i
+                # eager work of the library between replays (shares the workspace and the plan)
+                gpu.use_torch_stream()
+                gpu.mgg_SAG_np_div(H2, Y2, d_ptr, d_col, zp, zc, 0, V, out_dim, V, 0, 16, 8, 1)
+                side.synchronize()
+    finally:
+        torch.cuda.synchronize()
+        gpu.use_torch_stream()              # back on the default stream for the tests that follow
+
+
 def test_gcn_all_ones_wiring_is_integer_exact(gpu):
     """The reference's own validation design: all-ones X and W make every value an integer (exact in fp32)."""
     import torch
