@@ -209,6 +209,16 @@ def test_harness_programs_validate_and_log(gpu, graph_files, prog, dims, ngpu, p
     assert m and float(m.group(1)) > 0
 
 
+def test_cpp_layer_entry_points(gpu, tmp_path):
+    """mgg_api_check calls every function and class of include/mgg/*.h from C++ (loaders, split_CSR, build_part,
+    mgg_SAG_np_div, mgg_GIN_np_div, SAG_host, SAG_host_fused_interleaved, sparse_*/dense_*/softmax_* layer objects, the
+    knob search) with the reference's all-ones validation and exact comparisons."""
+    exe = os.path.join(BIN, "mgg_api_check")
+    r = subprocess.run([exe, str(tmp_path)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-1000:]
+    assert "0 check(s) failed" in r.stdout and r.stdout.count("[ok]") >= 13 and "[FAIL]" not in r.stdout
+
+
 def test_harness_reports_missing_file(gpu, tmp_path):
     exe = os.path.join(BIN, "mgg_np_div_kernel")
     r = subprocess.run([exe, str(tmp_path / "no_beg.bin"), "x", "y", "1", "16", "4", "1", "16", "16", "16"], capture_output=True,
