@@ -792,7 +792,7 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
 {
     Plan *plan = nullptr;
     int rc;
-    if (k.block_rows > 0 && g.nnz_r == 0 && ub - lb >= 2 * (long long)k.block_rows) {
+    if (k.block_rows > 0 && g.nnz_r == 0 && d_col_l && ub - lb >= 2 * (long long)k.block_rows) {
         rc = plan_get_blocked(d_ptr_l, d_col_l, ub - lb, lb, k.ps, k.block_rows, &plan);
         if (rc) return rc;
         if (plan->unsuitable) plan = nullptr;
