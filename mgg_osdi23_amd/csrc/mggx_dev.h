@@ -60,6 +60,7 @@ struct Plan {
     const int *d_col_r = nullptr;  // cache key of plans with remote edges (max_col_r depends on the values)
     int real_rows = 0;
     int block_rows = 0;
+    int block_lb = 0;          // id of the first row of block 0 (part of the cache key)
     int blocks = 1;
     bool unsuitable = false;   // blocked plan asked for, but the rows are not sorted by neighbor id
 };

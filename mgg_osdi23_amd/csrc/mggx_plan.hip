@@ -513,7 +513,7 @@ int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, i
 {
     State &s = state();
     for (Plan *p : s.plans)
-        if (p->d_ptr_l == d_ptr_l && p->d_col_l == d_col_l && p->real_rows == rows && p->ps == ps && p->block_rows == block_rows &&
+        if (p->d_ptr_l == d_ptr_l && p->d_col_l == d_col_l && p->real_rows == rows && p->ps == ps && p->block_rows == block_rows && p->block_lb == lb &&
             (p->blocks > 1 || p->unsuitable)) {
             *out = p;
             return MGGX_OK;
@@ -528,6 +528,7 @@ int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, i
     p->real_rows = rows;
     p->ps = ps;
     p->block_rows = block_rows;
+    p->block_lb = lb;
     int rc = MGGX_OK;
     int *d_cnt = nullptr, *d_vbeg = nullptr, *d_flag = nullptr;
     do {
