@@ -170,17 +170,25 @@ __device__ __forceinline__ void load_group(float (&x)[4][4], const float *xrow, 
         for (int gg = 0; gg < 4; ++gg) load_x4u(x[gg], xrow, ks + 16 * gg, d1, 0);
     } else {
         const int mode = d1 % 4 == 0 ? 1 : 2;
+        const int ngg = (d1 + 15) >> 4;  // 16-wide K steps that hold anything
 #pragma unroll
-        for (int gg = 0; gg < 4; ++gg) load_x4u(x[gg], xrow, 16 * gg + 4 * kq, d1, mode);
+        for (int gg = 0; gg < 4; ++gg) {
+            if (gg < ngg) {
+                load_x4u(x[gg], xrow, 16 * gg + 4 * kq, d1, mode);
+            } else {
+                x[gg][0] = x[gg][1] = x[gg][2] = x[gg][3] = 0.f;
+            }
+        }
     }
 }
 
 // acc[nb] += Wt-block^T . X-group, transposed product (see store_rows)
 template <int NB, int RS>
-__device__ __forceinline__ void mfma_group(v4f (&acc)[NB], const float *wt_group, const float (&x)[4][4], int i, int kq)
+__device__ __forceinline__ void mfma_group(v4f (&acc)[NB], const float *wt_group, const float (&x)[4][4], int i, int kq, int ngg)
 {
 #pragma unroll
     for (int gg = 0; gg < 4; ++gg) {
+        if (gg >= ngg) break;  // d1 < 64: the remaining 16-wide K steps are all zero
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const float *wrow = wt_group + (16 * gg + 4 * kq + t) * RS + i;
@@ -202,6 +210,7 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_dense_xw_resident(const Dens
     const int i = lane & 15, kq = lane >> 4;
     const int c0 = (int)blockIdx.y * (NB * 16);
     const int ngroups = (a.d1 + 63) >> 6;
+    const int ngg = FULL ? 4 : (a.d1 + 15) >> 4;
     const float *w = static_cast<const float *>(a.w);
     for (int idx = (int)threadIdx.x; idx < ngroups * 64 * NB * 16; idx += RES_THREADS) {
         const int r = idx / (NB * 16), j = idx % (NB * 16);
@@ -241,7 +250,7 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_dense_xw_resident(const Dens
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) acc[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
         }
-        mfma_group<NB, RS>(acc, wt + g * 64 * RS, xv, i, kq);
+        mfma_group<NB, RS>(acc, wt + g * 64 * RS, xv, i, kq, ngg);
         if (last_g) {
             const long long row = tile * 16 + i;
             store_rows<NB, false>(a.out, a.ld_out, a.d2, scale, a.relu, a.vec_out, acc, row, row < a.n, c0, kq);
@@ -279,6 +288,7 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_resident(const MlpArgs 
     const int wave = (int)(threadIdx.x >> 6);
     const int i = lane & 15, kq = lane >> 4;
     const int ngroups = (a.d1 + 63) >> 6;
+    const int ngg = FULL ? 4 : (a.d1 + 15) >> 4;
     float *wta = wt, *wtb = wt + ngroups * 64 * RS1;
     for (int idx = (int)threadIdx.x; idx < ngroups * 64 * NB1 * 16; idx += RES_THREADS) {
         const int r = idx / (NB1 * 16), j = idx % (NB1 * 16);
@@ -319,7 +329,7 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_resident(const MlpArgs 
 #pragma unroll
             for (int nb = 0; nb < NB1; ++nb) acc1[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
         }
-        mfma_group<NB1, RS1>(acc1, wta + g * 64 * RS1, xv, i, kq);
+        mfma_group<NB1, RS1>(acc1, wta + g * 64 * RS1, xv, i, kq, ngg);
         if (last_g) {
             v4f acc2[NB2];
 #pragma unroll
