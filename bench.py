@@ -260,6 +260,20 @@ def bench_gcn2(args, torch, host):
         parity = {"softmax_max_abs_err": float(np.abs(P - P_ref).max()),
                   "h1_max_rel_err": float(np.abs(d_H1.cpu().numpy() - H1_ref).max() / np.abs(H1_ref).max())}
         log("cpu forward %.1f ms on %d threads; parity %s" % (cpu_s * 1e3, th, parity))
+        if orc.have_ref():
+            # The reference's own CPU aggregation (SAG_ref, serial), compiled from its source: first rows of agg1
+            # worth about 20 M edges, on the first layer's output.
+            k = int(np.searchsorted(ptr, 20_000_000))
+            k = max(1, min(k, V))
+            y1 = d_Y1.cpu().numpy()
+            t0 = time.perf_counter()
+            got = orc.ref_sag_ref(y1, ptr[: k + 1], col[: ptr[k]])
+            ref_s = time.perf_counter() - t0
+            mine = d_H1.cpu().numpy()[:k] / s[:k, None]
+            cpu["reference_sag_ref"] = {"m_edges_per_s": round(int(ptr[k]) / ref_s / 1e6, 1), "cores": 1,
+                                        "sample": "rows 0..%d of agg1 (%d edges), width 16" % (k - 1, int(ptr[k])),
+                                        "gpu_m_edges_per_s": round(nnz / (avg["agg1"] * 1e-3) / 1e6, 1),
+                                        "max_rel_diff_vs_gpu": float(np.abs(got - mine).max() / np.abs(got).max())}
 
     return {
         "metric": "gcn_2layer_fwd_ms", "value": round(wall_ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
