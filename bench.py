@@ -1,18 +1,22 @@
 #!/usr/bin/env python3
 """Benchmark of the neighbor-partitioned aggregation path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gcn2|share] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gcn2|share|gin|big|copy|vendor] [--no-cpu]
 
 Default workload (`gcn2`): 2-layer GCN forward on the whole graph -- seeded RMAT
 power-law graph (a=.57 b=.19 c=.19), 233,000 nodes, ~114 M undirected edges,
 self loops, D^-1/2 (A+I) D^-1/2 weighting; fp32 features 602 -> 16 -> 41, Glorot
-weights; ps=16, wpb=8.  One step = dense, aggregate, dense, aggregate, softmax,
-all inputs resident in HBM.  Prints ONE JSON line: forward ms per step, the
-roofline figures of the dominant (aggregation) kernel from HIP events recorded
-inside the timed region, and the CPU oracle timed on this host's cores.
+weights; ps=16, the other knobs from the library's search (run before timing).
+One step = dense, aggregate, dense, aggregate, softmax, all inputs resident in
+HBM.  Prints ONE JSON line: forward ms per step, the roofline figures of the
+dominant (aggregation) kernel from HIP events recorded inside the timed region,
+and the CPU oracle timed on this host's cores.
 
 `share` times the aggregation alone on rank 0's 1/8 share of a 4.2 M-node RMAT
-graph with the remote rows pre-staged in a second HBM table.
+graph with the remote rows pre-staged in a second HBM table; `gin` the 5-layer
+GIN forward; `big` the bf16 large-share aggregation and update; `copy` the
+stream-copy yardstick; `vendor` the library's kernels beside torch.mm and
+torch.sparse.mm on the benchmark shapes.
 """
 from __future__ import annotations
 
@@ -574,6 +578,62 @@ def bench_big(args, torch, host):
     }
 
 
+def bench_vendor(args, torch, host):
+    """The library's kernels beside the vendor libraries torch dispatches to (GEMM behind torch.mm, CSR x dense SpMM
+    behind torch.sparse.mm) on the benchmark shapes.  A yardstick, not a target; nothing of torch's is on the product path."""
+    def timeit(fn, it):
+        fn(); fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(it):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / it
+
+    rows = []
+    for n, d1, d2 in ((233_000, 602, 16), (233_000, 16, 41), (2_450_000, 100, 64), (2_450_000, 64, 64)):
+        x, w = torch.randn(n, d1, device="cuda"), torch.randn(d1, d2, device="cuda")
+        o = torch.empty(n, d2, device="cuda")
+        rows.append({"op": "fp32 update %dx%dx%d" % (n, d1, d2),
+                     "library_ms": round(timeit(lambda: host.dense_forward(o, x, w, n, d1, d2), args.steps), 4),
+                     "vendor_ms": round(timeit(lambda: torch.mm(x, w, out=o), args.steps), 4)})
+    n, d = 2_450_000, 64
+    x, wa, wb = torch.randn(n, d, device="cuda"), torch.randn(d, d, device="cuda"), torch.randn(d, d, device="cuda")
+    o, t = torch.empty(n, d, device="cuda"), torch.empty(n, d, device="cuda")
+
+    def two():
+        torch.mm(x, wa, out=t)
+        torch.relu_(t)
+        torch.mm(t, wb, out=o)
+    rows.append({"op": "fp32 MLP 64->64->64 on %d rows (vendor: mm, relu, mm)" % n,
+                 "library_ms": round(timeit(lambda: host.mlp2_forward(o, x, wa, wb, n, d, d, d), args.steps), 4),
+                 "vendor_ms": round(timeit(two, args.steps), 4)})
+    del x, o, t
+    for name, (scale, V, draws, seed), dims in (("GCN graph", (18, 233_000, 216_000_000, 42), (16, 44)),
+                                                 ("GIN graph", (22, 2_450_000, 64_000_000, 3), (64,))):
+        ptr, col = host.gen_rmat(scale, V, draws, seed=seed)
+        d_ptr, d_col = torch.from_numpy(ptr).cuda(), torch.from_numpy(col).cuda()
+        zp, zc = torch.zeros(V + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+        A = torch.sparse_csr_tensor(d_ptr, d_col, torch.ones(len(col), device="cuda"), size=(V, V))
+        for dim in dims:
+            x, out = torch.randn(V, dim, device="cuda"), torch.empty(V, dim, device="cuda")
+            host.tune_np_div(out, x, d_ptr, d_col, zp, zc, 0, V, dim, V, 16)
+            t1 = timeit(lambda: host.mgg_SAG_np_div(out, x, d_ptr, d_col, zp, zc, 0, V, dim, V, 0, 0, 0, 0), args.steps)
+            t2 = timeit(lambda: torch.sparse.mm(A, x), 3)
+            ref = torch.sparse.mm(A, x)
+            rows.append({"op": "aggregation, %s nnz=%d width %d" % (name, len(col), dim), "library_ms": round(t1, 4),
+                         "vendor_ms": round(t2, 4), "max_diff_over_max": float((out - ref).abs().max() / ref.abs().max())})
+            log(rows[-1])
+        del A
+    worst = min(r["vendor_ms"] / r["library_ms"] for r in rows)
+    return {"metric": "vendor_time_over_library_time_min", "value": round(worst, 3), "unit": "x", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f32", "data": "synthetic", "config": {"workload": "library kernels beside torch.mm / torch.sparse.mm"},
+            "detail": rows}
+
+
 def bench_copy(args, torch, host):
     """Plain device copy of a known size: the stream-copy ceiling, and the yardstick the profiler's FETCH_SIZE /
     WRITE_SIZE counters are scaled against."""
@@ -599,7 +659,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gcn2", choices=["gcn2", "share", "gin", "big", "copy"])
+    ap.add_argument("--workload", default="gcn2", choices=["gcn2", "share", "gin", "big", "copy", "vendor"])
     ap.add_argument("--ps", type=int, default=16, help="partSize; 0 = let the library choose (the search then tries 16 and 32)")
     ap.add_argument("--col-block-rows", type=int, default=0, help="column-blocked partition order: 0 = library decides, -1 = off, "
                          "N = blocks of N neighbor ids")
@@ -627,7 +687,8 @@ def main():
     host.init(0)
     host.use_torch_stream()
     log("device:", host.device_name())
-    res = {"gcn2": bench_gcn2, "share": bench_share, "gin": bench_gin, "big": bench_big, "copy": bench_copy}[args.workload](args, torch, host)
+    res = {"gcn2": bench_gcn2, "share": bench_share, "gin": bench_gin, "big": bench_big, "copy": bench_copy,
+           "vendor": bench_vendor}[args.workload](args, torch, host)
     print(json.dumps(res), flush=True)
 
 
