@@ -235,6 +235,26 @@ def test_column_blocked_order(gpu, rmat_graph, dim, block_rows, flags):
         assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "unsorted rows")
 
 
+def test_column_blocked_order_with_bf16_tables(gpu, rmat_graph):
+    """bf16 feature rows, fp32 partial rows and output: the blocked order must give what the plain order gives."""
+    import torch
+    V, ptr, col = rmat_graph
+    dim = 64
+    x = gpu.fill_normal((V, dim), seed=95)
+    d_x = to_dev(x).to(torch.bfloat16)
+    xr = d_x.float().cpu().numpy()
+    sh = share_of(ptr, col, V, 1, 0)
+    d_ptr, d_col = to_dev(ptr), to_dev(col)
+    z, zc = torch.zeros(V + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    want, mag = oracle_agg(sh, xr, xr, dim, flags=orc.GIN, eps=0.25)
+    for blk in (200, -1):
+        out = torch.full((V, dim), 7.5, device="cuda")
+        gpu.mgg_GIN_np_div(out, d_x, d_ptr, d_col, z, zc, 0, V, dim, V, 0, 16, 4, 2, 0.25, col_block_rows=blk)
+        gpu.sync()
+        assert ("blocks=30" in gpu.last_agg_kernel()) == (blk > 0)
+        assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "bf16 tables, col_block_rows=%d" % blk)
+
+
 def test_column_blocked_with_empty_rows_and_search(gpu):
     """Rows without neighbors, rows whose neighbors all fall in one block, and the search over both orders."""
     import torch
