@@ -562,6 +562,29 @@ __global__ void __launch_bounds__(256) k_agg_block_reduce(const AggArgs a, const
     finish_elem(a, v, d, total);
 }
 
+// The same with four columns per thread, for outputs that take 16-byte stores and epilogues without a read of
+// other tables (row scale and ReLU only).
+__global__ void __launch_bounds__(256) k_agg_block_reduce4(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp)
+{
+    const int q = a.dim >> 2;  // float4 per row
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long long)rows * q) return;
+    const int v = (int)(idx / q), d = 4 * (int)(idx % q);
+    float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int c = 0; c < blocks; ++c) {
+        const float4 p = *reinterpret_cast<const float4 *>(part + ((long long)c * rows + v) * ldp + d);
+        t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
+    }
+    if (a.rs_out) {
+        const float s = a.rs_out[v];
+        t.x *= s; t.y *= s; t.z *= s; t.w *= s;
+    }
+    if (a.flags & MGGX_AGG_RELU) {
+        t.x = fmaxf(t.x, 0.f); t.y = fmaxf(t.y, 0.f); t.z = fmaxf(t.z, 0.f); t.w = fmaxf(t.w, 0.f);
+    }
+    *reinterpret_cast<float4 *>(a.out + (long long)v * a.ld_out + d) = t;
+}
+
 int pow2_ceil(int x)
 {
     int p = 1;
@@ -743,8 +766,14 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         r.ld_out = ld_out;
         r.rs_out = o.d_row_scale_out;
         r.flags = o.flags;
-        const long long n = (long long)plan->real_rows * dim;
-        k_agg_block_reduce<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(r, part, plan->real_rows, plan->blocks, ldp);
+        const bool vec4 = dim % 4 == 0 && ld_out % 4 == 0 && aligned16(d_out) && !(o.flags & (MGGX_AGG_GIN | MGGX_AGG_ACCUMULATE));
+        if (vec4) {
+            const long long n = (long long)plan->real_rows * (dim / 4);
+            k_agg_block_reduce4<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(r, part, plan->real_rows, plan->blocks, ldp);
+        } else {
+            const long long n = (long long)plan->real_rows * dim;
+            k_agg_block_reduce<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(r, part, plan->real_rows, plan->blocks, ldp);
+        }
         MGGX_LAUNCH_CHECK("k_agg_block_reduce");
     }
     snprintf(st.last_kernel, sizeof(st.last_kernel), "k_agg<%d,%d,%d> grid=%lld block=%d parts=%d blocks=%d", lpr, mode, (int)buf, num_wg,
