@@ -189,6 +189,13 @@ __device__ __forceinline__ void finish_elem(const AggArgs &a, int row, int d, fl
     *o = v;
 }
 
+// Output rows are written once and not read again by the aggregation: stored with the streaming hint.
+__device__ __forceinline__ void store_row16(float *p, float x, float y, float z, float w)
+{
+    typedef float v4f_s __attribute__((ext_vector_type(4)));
+    __builtin_nontemporal_store((v4f_s){x, y, z, w}, reinterpret_cast<v4f_s *>(p));
+}
+
 // Finishes this lane's NV elements of a complete row held in registers.
 template <int LPR, int MODE>
 __device__ __forceinline__ void finish_row(const AggArgs &a, int row, int l, const float (&acc)[ModeTraits<MODE>::NV])
@@ -197,16 +204,16 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int row, int l, con
     if constexpr (MODE == MODE_F32_VEC4) {
         if (a.flags == 0 && a.rs_out == nullptr) {
             if (NV * l < a.dim)
-                *reinterpret_cast<float4 *>(a.out + (long long)row * a.ld_out + 4 * l) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+                store_row16(a.out + (long long)row * a.ld_out + 4 * l, acc[0], acc[1], acc[2], acc[3]);
             return;
         }
     }
     if constexpr (MODE == MODE_BF16_VEC8) {
         if (a.flags == 0 && a.rs_out == nullptr) {
             if (NV * l < a.dim) {
-                float4 *o = reinterpret_cast<float4 *>(a.out + (long long)row * a.ld_out + 8 * l);
-                o[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
-                o[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+                float *o = a.out + (long long)row * a.ld_out + 8 * l;
+                store_row16(o, acc[0], acc[1], acc[2], acc[3]);
+                store_row16(o + 4, acc[4], acc[5], acc[6], acc[7]);
             }
             return;
         }
@@ -229,7 +236,7 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int row, int l, con
             if (a.flags & MGGX_AGG_RELU) {
                 v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f);
             }
-            *o = v;
+            store_row16(reinterpret_cast<float *>(o), v.x, v.y, v.z, v.w);
         }
         return;
     }
