@@ -22,7 +22,9 @@ struct DenseArgs {
     long long ld_x, ld_out;
     int d1, d2;
     int relu;
-    int vec_out;  // rows of out may be written 4 elements at a time (alignment and stride allow it)
+    int vec_out;  // bit 0: rows of out may be written 4 elements at a time (alignment and stride allow it);
+                  // bit 1: and they are whole 128-byte lines written once: streaming stores
+    int stream_x; // rows of X are whole 128-byte lines per K group (d1 % 64 == 0, aligned base and pitch)
 };
 
 // v_mfma_f32_16x16x4_f32 operand layout (wave64):
@@ -53,7 +55,11 @@ __device__ __forceinline__ void load_x4(float (&xv)[4], const float *xrow, int k
 //   2  any d1: four dword loads from clamped offsets, zeroed one by one
 __device__ __forceinline__ void load_x4u(float (&xv)[4], const float *xrow, int kb, int d1, int mode)
 {
-    if (mode == 0) {
+    if (mode == 3) {  // as mode 0, and every 64-wide K group of a row is two whole cache lines read once: streaming hint
+        typedef float v4f_u __attribute__((ext_vector_type(4), aligned(16)));
+        const v4f_u t4 = __builtin_nontemporal_load(reinterpret_cast<const v4f_u *>(xrow + kb));
+        xv[0] = t4.x; xv[1] = t4.y; xv[2] = t4.z; xv[3] = t4.w;
+    } else if (mode == 0) {
         float4 t4;
         __builtin_memcpy(&t4, xrow + kb, 16);
         xv[0] = t4.x; xv[1] = t4.y; xv[2] = t4.z; xv[3] = t4.w;
@@ -130,7 +136,8 @@ __device__ __forceinline__ void store_rows(void *out, long long ld_out, int d2, 
         } else {
             float *o = static_cast<float *>(out) + row * ld_out + c;
             if (vec_out && c + 3 < d2) {
-                *reinterpret_cast<float4 *>(o) = make_float4(v[0], v[1], v[2], v[3]);
+                if (vec_out & 2) __builtin_nontemporal_store((v4f){v[0], v[1], v[2], v[3]}, reinterpret_cast<v4f *>(o));
+                else *reinterpret_cast<float4 *>(o) = make_float4(v[0], v[1], v[2], v[3]);
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
@@ -161,13 +168,15 @@ __device__ __forceinline__ int lds_row_k(int r, int ngroups, int d1)
     }
 }
 
-template <bool FULL>
+// KMODE: 0 = d1 < 64, 1 = d1 >= 64, 2 = d1 >= 64 and every K group of a row is whole cache lines (streamed)
+template <int KMODE>
 __device__ __forceinline__ void load_group(float (&x)[4][4], const float *xrow, int g, int ngroups, int d1, int kq)
 {
-    if constexpr (FULL) {
+    if constexpr (KMODE >= 1) {
         const int ks = (g == ngroups - 1 ? d1 - 64 : 64 * g) + 4 * kq;
+        constexpr int mode = KMODE == 2 ? 3 : 0;
 #pragma unroll
-        for (int gg = 0; gg < 4; ++gg) load_x4u(x[gg], xrow, ks + 16 * gg, d1, 0);
+        for (int gg = 0; gg < 4; ++gg) load_x4u(x[gg], xrow, ks + 16 * gg, d1, mode);
     } else {
         const int mode = d1 % 4 == 0 ? 1 : 2;
         const int ngg = (d1 + 15) >> 4;  // 16-wide K steps that hold anything
@@ -199,9 +208,10 @@ __device__ __forceinline__ void mfma_group(v4f (&acc)[NB], const float *wt_group
     }
 }
 
-template <int NB, bool FULL>
+template <int NB, int KMODE>
 __global__ void __launch_bounds__(RES_THREADS, 4) k_dense_xw_resident(const DenseArgs a)
 {
+    constexpr bool FULL = KMODE >= 1;
     constexpr int RS = NB * 16 + 4;  // LDS row stride in floats; the +4 keeps the four K groups on distinct banks
     constexpr int WAVES = RES_THREADS / 64;
     extern __shared__ float wt[];
@@ -230,7 +240,7 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_dense_xw_resident(const Dens
     float scale = 1.0f, scale_next = 1.0f;
     {
         const long long row = min(tile * 16 + i, a.n - 1);
-        load_group<FULL>(xv, x + row * a.ld_x, 0, ngroups, a.d1, kq);
+        load_group<KMODE>(xv, x + row * a.ld_x, 0, ngroups, a.d1, kq);
         if (a.rs) scale = a.rs[row];
     }
     v4f acc[NB];
@@ -241,7 +251,7 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_dense_xw_resident(const Dens
         const int ng = last_g ? 0 : g + 1;
         {
             const long long nrow = min(ntile * 16 + i, a.n - 1);
-            load_group<FULL>(xn, x + nrow * a.ld_x, ng, ngroups, a.d1, kq);
+            load_group<KMODE>(xn, x + nrow * a.ld_x, ng, ngroups, a.d1, kq);
             scale_next = scale;
             if (last_g && a.rs) scale_next = a.rs[nrow];
         }
@@ -275,12 +285,13 @@ struct MlpArgs {
     const float *x, *wa, *wb, *rs;
     long long n, ld_x, ld_out;
     int d1, h, d3;
-    int relu_mid, relu_out, vec_out;
+    int relu_mid, relu_out, vec_out, stream_x;
 };
 
-template <int NB1, int NB2, bool FULL>
+template <int NB1, int NB2, int KMODE>
 __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_resident(const MlpArgs a)
 {
+    constexpr bool FULL = KMODE >= 1;
     constexpr int RS1 = NB1 * 16 + 4, RS2 = NB2 * 16 + 4;
     constexpr int WAVES = RES_THREADS / 64;
     extern __shared__ float wt[];
@@ -309,7 +320,7 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_resident(const MlpArgs 
     float scale = 1.0f, scale_next = 1.0f;
     {
         const long long row = min(tile * 16 + i, a.n - 1);
-        load_group<FULL>(xv, a.x + row * a.ld_x, 0, ngroups, a.d1, kq);
+        load_group<KMODE>(xv, a.x + row * a.ld_x, 0, ngroups, a.d1, kq);
         if (a.rs) scale = a.rs[row];
     }
     v4f acc1[NB1];
@@ -320,7 +331,7 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_resident(const MlpArgs 
         const int ng = last_g ? 0 : g + 1;
         {
             const long long nrow = min(ntile * 16 + i, a.n - 1);
-            load_group<FULL>(xn, a.x + nrow * a.ld_x, ng, ngroups, a.d1, kq);
+            load_group<KMODE>(xn, a.x + nrow * a.ld_x, ng, ngroups, a.d1, kq);
             scale_next = scale;
             if (last_g && a.rs) scale_next = a.rs[nrow];
         }
@@ -619,12 +630,15 @@ template <int NB>
 struct LaunchResident {
     static void run(dim3 grid, size_t lds, hipStream_t s, const DenseArgs &a)
     {
-        if (a.d1 >= 64) {
-            allow_lds(k_dense_xw_resident<NB, true>, lds);
-            k_dense_xw_resident<NB, true><<<grid, dim3(RES_THREADS), lds, s>>>(a);
+        if (a.d1 >= 64 && a.stream_x) {
+            allow_lds(k_dense_xw_resident<NB, 2>, lds);
+            k_dense_xw_resident<NB, 2><<<grid, dim3(RES_THREADS), lds, s>>>(a);
+        } else if (a.d1 >= 64) {
+            allow_lds(k_dense_xw_resident<NB, 1>, lds);
+            k_dense_xw_resident<NB, 1><<<grid, dim3(RES_THREADS), lds, s>>>(a);
         } else {
-            allow_lds(k_dense_xw_resident<NB, false>, lds);
-            k_dense_xw_resident<NB, false><<<grid, dim3(RES_THREADS), lds, s>>>(a);
+            allow_lds(k_dense_xw_resident<NB, 0>, lds);
+            k_dense_xw_resident<NB, 0><<<grid, dim3(RES_THREADS), lds, s>>>(a);
         }
     }
 };
@@ -680,6 +694,8 @@ MGGX_EXPORT int mggx_dense_xw(float *d_out, const float *d_x, const float *d_w, 
     a.d2 = d2;
     a.relu = o.relu != 0;
     a.vec_out = a.ld_out % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0;
+    if (d2 % 32 == 0 && a.ld_out % 32 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 127u) == 0) a.vec_out |= 2;
+    a.stream_x = d1 % 64 == 0 && a.ld_x % 32 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 127u) == 0;
     if (a.ld_x < d1 || a.ld_out < d2) return fail(MGGX_EINVAL, "dense_xw: row stride smaller than width");
     hipStream_t stream = mggx::state().stream;
     const int nb = mggx::pick_nb(d2);
@@ -703,12 +719,15 @@ namespace {
 template <int NB1, int NB2>
 void launch_mlp2(dim3 grid, size_t lds, hipStream_t s, const MlpArgs &a)
 {
-    if (a.d1 >= 64) {
-        allow_lds(k_mlp2_resident<NB1, NB2, true>, lds);
-        k_mlp2_resident<NB1, NB2, true><<<grid, dim3(RES_THREADS), lds, s>>>(a);
+    if (a.d1 >= 64 && a.stream_x) {
+        allow_lds(k_mlp2_resident<NB1, NB2, 2>, lds);
+        k_mlp2_resident<NB1, NB2, 2><<<grid, dim3(RES_THREADS), lds, s>>>(a);
+    } else if (a.d1 >= 64) {
+        allow_lds(k_mlp2_resident<NB1, NB2, 1>, lds);
+        k_mlp2_resident<NB1, NB2, 1><<<grid, dim3(RES_THREADS), lds, s>>>(a);
     } else {
-        allow_lds(k_mlp2_resident<NB1, NB2, false>, lds);
-        k_mlp2_resident<NB1, NB2, false><<<grid, dim3(RES_THREADS), lds, s>>>(a);
+        allow_lds(k_mlp2_resident<NB1, NB2, 0>, lds);
+        k_mlp2_resident<NB1, NB2, 0><<<grid, dim3(RES_THREADS), lds, s>>>(a);
     }
 }
 template <int NB1>
@@ -751,6 +770,8 @@ MGGX_EXPORT int mggx_mlp2_xw(float *d_out, const float *d_x, const float *d_wa, 
     a.relu_mid = o.relu_mid != 0;
     a.relu_out = o.relu_out != 0;
     a.vec_out = a.ld_out % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0;
+    if (d3 % 32 == 0 && a.ld_out % 32 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 127u) == 0) a.vec_out |= 2;
+    a.stream_x = d1 % 64 == 0 && a.ld_x % 32 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 127u) == 0;
     if (a.ld_x < d1 || a.ld_out < d3) return fail(MGGX_EINVAL, "mlp2_xw: row stride smaller than width");
     const int nb1 = (h + 15) / 16, nb2 = (d3 + 15) / 16;
     const size_t lds = ((size_t)((d1 + 63) & ~63) * (nb1 * 16 + 4) + (size_t)nb1 * 16 * (nb2 * 16 + 4)) * sizeof(float);
