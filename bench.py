@@ -82,8 +82,8 @@ class StageTimer:
 MEASURED_TRAFFIC = {
     "gcn2_agg2": (28_216_496_128, (4, 16)),
     "gcn2_agg1": (6_481_731_891, (4, 16)),
-    "gcn2_agg2_blocked": (7_642_250_035, (4, 16)),   # column blocks of 49152 ids: partial rows and their reduction included
-    "gcn2_agg1_blocked": (2_081_738_854, (4, 16)),
+    "gcn2_agg2_blocked": (7_519_810_150, (4, 16)),   # column blocks of 49152 ids: partial rows and their reduction included
+    "gcn2_agg1_blocked": (1_746_502_963, (4, 16)),
     "share_agg": (1_220_807_373, (8, 1)),
     "gin_agg": (25_550_513_561, (16, 1)),
     "big_agg": (60_709_001_216, (4, 16)),
