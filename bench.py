@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the neighbor-partitioned aggregation path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gcn2|share|gin|big|copy|vendor] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gcn2|share|gin|big|copy|gather|vendor] [--no-cpu]
 
 Default workload (`gcn2`): 2-layer GCN forward on the whole graph -- seeded RMAT
 power-law graph (a=.57 b=.19 c=.19), 233,000 nodes, ~114 M undirected edges,
@@ -15,7 +15,8 @@ and the CPU oracle timed on this host's cores.
 `share` times the aggregation alone on rank 0's 1/8 share of a 4.2 M-node RMAT
 graph with the remote rows pre-staged in a second HBM table; `gin` the 5-layer
 GIN forward; `big` the bf16 large-share aggregation and update; `copy` the
-stream-copy yardstick; `vendor` the library's kernels beside torch.mm and
+stream-copy yardstick; `gather` the random-gather yardstick (what the memory system sustains for row gathers from
+tables of the benchmark sizes); `vendor` the library's kernels beside torch.mm and
 torch.sparse.mm on the benchmark shapes.
 """
 from __future__ import annotations
@@ -654,12 +655,45 @@ def bench_copy(args, torch, host):
             "config": {"workload": "k_copy16: %d bytes read + %d bytes written per launch" % (nbytes, nbytes)}}
 
 
+def bench_gather(args, torch, host):
+    """Random row gathers from tables of the benchmark shapes, with no index stream and no reduction: what the memory
+    system sustains for the access pattern of the aggregation at each table size (the ceiling for cache-resident
+    tables, where HBM peak says nothing)."""
+    sink = torch.empty(262144, device="cuda")
+    cases = (("64 B rows, 3 MB table (one column block of the width-16 GCN table)", 49152, 64, 64),
+             ("64 B rows, 15 MB table (whole width-16 GCN table)", 233_000, 64, 64),
+             ("64 B rows, 269 MB table (remote table of the 1/8 share)", 4_200_000, 64, 64),
+             ("176 B of 192 B rows, 3 MB table", 16384, 192, 176),
+             ("176 B of 192 B rows, 9.4 MB table (one column block of the width-41 GCN table)", 49152, 192, 176),
+             ("176 B of 192 B rows, 45 MB table (whole width-41 GCN table)", 233_000, 192, 176),
+             ("256 B rows, 627 MB table (GIN, width 64 fp32)", 2_450_000, 256, 256),
+             ("256 B rows, 4.2 GB table (large share, width 128 bf16, compact staging)", 16_500_000, 256, 256))
+    table = torch.zeros(max(r * ld for _, r, ld, _ in cases), dtype=torch.uint8, device="cuda")
+    n = 228_000_000
+    out = []
+    for name, rows, ld, rb in cases:
+        for _ in range(max(1, args.warmup)):
+            done = host.gather_probe(sink, table, rows, ld, rb, n)
+        torch.cuda.synchronize()
+        timer = StageTimer(torch, ["probe"])
+        for i in range(args.steps):
+            timer.step([lambda: host.gather_probe(sink, table, rows, ld, rb, n, seed=i + 2)])
+        ms = timer.averages()["probe"]
+        out.append({"table": name, "rows_per_s_G": round(done / (ms * 1e-3) / 1e9, 1), "ms": round(ms, 4),
+                    "useful_gbps": round(done * rb / (ms * 1e-3) / 1e9, 1)})
+        log(out[-1])
+    return {"metric": "gather_rows_per_s_G_64B_rows_3MB_table", "value": out[0]["rows_per_s_G"], "unit": "G rows/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": out[0]["ms"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "k_gather_probe: %d random row gathers per launch per table shape" % done}, "detail": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gcn2", choices=["gcn2", "share", "gin", "big", "copy", "vendor"])
+    ap.add_argument("--workload", default="gcn2", choices=["gcn2", "share", "gin", "big", "copy", "gather", "vendor"])
     ap.add_argument("--ps", type=int, default=16, help="partSize; 0 = let the library choose (the search then tries 16 and 32)")
     ap.add_argument("--col-block-rows", type=int, default=0, help="column-blocked partition order: 0 = library decides, -1 = off, "
                          "N = blocks of N neighbor ids")
@@ -688,7 +722,7 @@ def main():
     host.use_torch_stream()
     log("device:", host.device_name())
     res = {"gcn2": bench_gcn2, "share": bench_share, "gin": bench_gin, "big": bench_big, "copy": bench_copy,
-           "vendor": bench_vendor}[args.workload](args, torch, host)
+           "gather": bench_gather, "vendor": bench_vendor}[args.workload](args, torch, host)
     print(json.dumps(res), flush=True)
 
 

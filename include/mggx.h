@@ -292,6 +292,14 @@ int mggx_cast_f32_to_bf16(void *d_dst, const float *d_src, int64_t n);
  * profiler's HBM byte counters are scaled against. */
 int mggx_copy_bytes(void *d_dst, const void *d_src, size_t n);
 
+/* Yardstick for row gathers (no counterpart in the reference): at least n_gathers loads of row_bytes bytes (16..256, in
+ * 16-byte pieces) from rows at pseudo-random indices of a table of `rows` rows with a stride of ld_bytes, eight loads in
+ * flight per lane group, no index array and no reduction; *n_done (optional) receives the exact number issued.  d_sink
+ * must hold 262144 floats (one sum per thread, so the loads are not optimised away).  What this sustains on a table of
+ * a given size is the ceiling the aggregation kernels are measured against where their table is cache resident. */
+int mggx_gather_probe(float *d_sink, const void *d_table, int64_t rows, size_t ld_bytes, size_t row_bytes,
+                      int64_t n_gathers, unsigned seed, int64_t *n_done);
+
 /* How the aggregation kernels address feature rows: 0 (default) picks per call -- 32-bit buffer offsets when both
  * tables lie inside one window of < 2 GiB and < 2^24 rows, 64-bit addresses otherwise; 1 always uses 64-bit
  * addresses.  Results are identical; the switch exists for tests and measurements. */

@@ -249,7 +249,71 @@ __global__ void __launch_bounds__(256) k_gather_rows(int4 *__restrict__ dst, con
     }
 }
 
+// Yardstick for gathers: every slot of LPR lanes loads rows at pseudo-random indices of the table, eight loads in
+// flight, with no index array to read and no reduction structure; each lane sums what it loads and stores the sum.
+typedef unsigned probe_v4u __attribute__((ext_vector_type(4)));
+
+template <int LPR>
+__global__ void __launch_bounds__(256) k_gather_probe(float *__restrict__ sink, const char *__restrict__ table, unsigned rows,
+                                                      unsigned ld_bytes, int lanes_on, int iters, unsigned seed)
+{
+    constexpr int S = 64 / LPR;
+    const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
+    const int slot = lane / LPR, l = lane % LPR;
+    unsigned x = ((((unsigned)blockIdx.x * 4u + (unsigned)wave) * S + (unsigned)slot) + 1u) * 2654435761u ^ seed;
+    x ^= x >> 15; x *= 2246822519u; x ^= x >> 13;
+    const bool on = l < lanes_on;
+    const unsigned cofs = 16u * (unsigned)(on ? l : 0);
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < iters; ++it) {
+        unsigned r[8];
+        probe_v4u v[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            x = x * 1664525u + 1013904223u;
+            r[t] = __umulhi(x ^ (x >> 16), rows);
+            v[t] = (probe_v4u){0u, 0u, 0u, 0u};
+        }
+        if (on) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) v[t] = *reinterpret_cast<const probe_v4u *>(table + (size_t)r[t] * ld_bytes + cofs);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            acc[0] += __uint_as_float(v[t].x); acc[1] += __uint_as_float(v[t].y);
+            acc[2] += __uint_as_float(v[t].z); acc[3] += __uint_as_float(v[t].w);
+        }
+    }
+    sink[(size_t)blockIdx.x * 256 + threadIdx.x] = acc[0] + acc[1] + acc[2] + acc[3];
+}
+
+constexpr int PROBE_BLOCKS = 1024;
+
 }  // namespace
+
+MGGX_EXPORT int mggx_gather_probe(float *d_sink, const void *d_table, int64_t rows, size_t ld_bytes, size_t row_bytes,
+                                  int64_t n_gathers, unsigned seed, int64_t *n_done)
+{
+    if (!d_sink || !d_table || rows < 1 || rows > 0x7fffffffLL || row_bytes < 16 || row_bytes > 256 || (row_bytes % 16) ||
+        ld_bytes < row_bytes || (ld_bytes % 16) || ld_bytes > 0xffffffffull || n_gathers < 1 ||
+        (reinterpret_cast<uintptr_t>(d_table) & 15u))
+        return fail(MGGX_EINVAL, "gather_probe: NULL pointer, rows of 16..256 bytes in 16-byte pieces, or misaligned table");
+    const int lanes_on = (int)(row_bytes / 16);
+    const int lpr = lanes_on <= 4 ? 4 : 16;
+    const long long per_iter = (long long)PROBE_BLOCKS * 4 * (64 / lpr) * 8;
+    long long iters = (n_gathers + per_iter - 1) / per_iter;
+    if (iters > 0x7fffffffLL) return fail(MGGX_ELIMIT, "gather_probe: too many gathers");
+    if (lpr == 4)
+        k_gather_probe<4><<<dim3(PROBE_BLOCKS), dim3(256), 0, state().stream>>>(d_sink, (const char *)d_table, (unsigned)rows,
+                                                                                 (unsigned)ld_bytes, lanes_on, (int)iters, seed);
+    else
+        k_gather_probe<16><<<dim3(PROBE_BLOCKS), dim3(256), 0, state().stream>>>(d_sink, (const char *)d_table, (unsigned)rows,
+                                                                                  (unsigned)ld_bytes, lanes_on, (int)iters, seed);
+    MGGX_LAUNCH_CHECK("k_gather_probe");
+    if (n_done) *n_done = iters * per_iter;
+    return MGGX_OK;
+}
 
 MGGX_EXPORT int mggx_copy_bytes(void *d_dst, const void *d_src, size_t n)
 {

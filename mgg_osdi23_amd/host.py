@@ -55,7 +55,7 @@ EXPORTS = [
     "mggx_release_cached", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
     "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_compact_remote_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_mlp2_xw", "mggx_spmm",
-    "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_gather_rows", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
+    "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_gather_probe", "mggx_gather_rows", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
 ]
 
 
@@ -429,3 +429,11 @@ def softmax_forward(out, x, n, c, ld_in=0, ld_out=0):
 
 def copy_bytes(dst, src, nbytes: int) -> None:
     _check(lib().mggx_copy_bytes(_dptr(dst), _dptr(src), C.c_size_t(nbytes)))
+
+
+def gather_probe(sink, table, rows: int, ld_bytes: int, row_bytes: int, n_gathers: int, seed: int = 1) -> int:
+    """Random row gathers from `table` (rows x ld_bytes bytes); `sink` holds 262144 floats.  Returns the number issued."""
+    done = C.c_int64(0)
+    _check(lib().mggx_gather_probe(_dptr(sink), _dptr(table), C.c_int64(rows), C.c_size_t(ld_bytes), C.c_size_t(row_bytes),
+                                   C.c_int64(n_gathers), C.c_uint(seed), C.byref(done)))
+    return int(done.value)

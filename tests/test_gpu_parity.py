@@ -632,6 +632,24 @@ def test_softmax_rows(gpu, n, c):
     assert np.allclose(t.cpu().numpy(), want, rtol=1e-5, atol=1e-7)
 
 
+@pytest.mark.parametrize("rows,ld,row_bytes", [(1000, 64, 64), (333, 192, 176), (77, 256, 256), (5, 32, 16)])
+def test_gather_yardstick_counts_its_loads(gpu, rows, ld, row_bytes):
+    """On a table of ones every lane that holds a piece of a row sums 4 per load; the other lanes issue none."""
+    import torch
+    table = torch.ones(rows * ld // 4, device="cuda")
+    sink = torch.full((262144,), -1.0, device="cuda")
+    done = gpu.gather_probe(sink, table, rows, ld, row_bytes, 1_000_000)
+    gpu.sync()
+    lanes = 4 if row_bytes <= 64 else 16
+    per_launch = 1024 * 4 * (64 // lanes) * 8
+    assert done >= 1_000_000 and done % per_launch == 0
+    s = sink.cpu().numpy().reshape(-1, lanes)
+    on = row_bytes // 16
+    assert np.all(s[:, :on] == 4.0 * 8 * (done // per_launch)) and np.all(s[:, on:] == 0.0)
+    with pytest.raises(gpu.MggxError):
+        gpu.gather_probe(sink, table, rows, ld, 24, 1000)
+
+
 # --------------------------------------------------------------------------- bf16 tables, fp32 accumulation
 @pytest.mark.parametrize("dim", [8, 64, 128, 256])
 def test_bf16_tables(gpu, rmat_graph, dim):
