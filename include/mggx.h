@@ -79,6 +79,10 @@ int mggx_timer_elapsed_ms(void *timer, float *ms); /* synchronises on the stop e
 int mggx_timer_destroy(void *timer);
 /* Frees the workspace and every cached plan. */
 int mggx_release_cached(void);
+/* Drops what the library remembers about the CSR array at this device address (cached partition plans, search
+ * results): call it before freeing or rewriting an index array that aggregation calls have seen, when the memory is
+ * not released through mggx_free (which does this itself) -- an allocator may hand the same address out again. */
+int mggx_forget(const void *d_ptr);
 
 /* ---- host-side graph preparation (CPU; replaces the host code of the path) ---- */
 
@@ -202,8 +206,8 @@ typedef struct mggx_agg_knobs {
  * feature table in use at any time is small enough to stay in cache; each block leaves a partial row in library
  * scratch and a second kernel sums them in block order and applies the epilogue.  Same result up to summation order.
  * The partition plan of (d_ptr_l, d_ptr_r, d_col_r, rows, ps) -- and d_col_l for the column-blocked order -- is built on first use and
- * cached by pointer identity: the CSR arrays must not be rewritten in place
- * while cached (mggx_release_cached() drops the cache). */
+ * cached by pointer identity: the CSR arrays must not be rewritten in place or freed
+ * while cached (mggx_forget() drops what hangs on one array, mggx_release_cached() everything). */
 int mggx_sag_np_div(float *d_out, const void *d_in_local, const void *d_in_remote,
                     const int *d_ptr_l, const int *d_col_l, const int *d_ptr_r, const int *d_col_r,
                     int lb, int ub, int dim, int nodes_per_pe,

@@ -103,6 +103,7 @@ int graph_info(const int *d_ptr_l, const int *d_ptr_r, int rows, GraphInfo **out
 int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows,
                       int num_parts, int ps, Plan **out);
 void plan_free(Plan *p);
+int forget_pointer(const void *d_ptr);
 
 }  // namespace mggx
 #endif

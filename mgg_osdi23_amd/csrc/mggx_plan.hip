@@ -493,7 +493,8 @@ int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_
             break;
         }
         int end = 0;
-        if (rows > 0 && hipMemcpy(&end, d_row_ptr + rows, sizeof(int), hipMemcpyDeviceToHost) != hipSuccess) {
+        if (rows > 0 && (hipStreamSynchronize(s.stream) != hipSuccess ||
+                         hipMemcpy(&end, d_row_ptr + rows, sizeof(int), hipMemcpyDeviceToHost) != hipSuccess)) {
             rc = fail(MGGX_EHIP, "plan: reading edge count");
             break;
         }
@@ -623,9 +624,41 @@ int graph_info(const int *d_ptr_l, const int *d_ptr_r, int rows, GraphInfo **out
     return MGGX_OK;
 }
 
+// Drops every cached plan and graph record keyed by this device address (an array about to be freed or rewritten).
+int forget_pointer(const void *d_ptr)
+{
+    State &s = state();
+    bool synced = false;
+    for (size_t i = 0; i < s.plans.size();) {
+        Plan *p = s.plans[i];
+        if (p->d_ptr_l == d_ptr || p->d_ptr_r == d_ptr || p->d_col_l == d_ptr || p->d_col_r == d_ptr || p->d_part_ptr == d_ptr ||
+            p->d_part2node == d_ptr) {
+            if (!synced && s.device >= 0) {  // a kernel in flight may still read the plan
+                MGGX_HIP(hipStreamSynchronize(s.stream));
+                synced = true;
+            }
+            plan_free(p);
+            s.plans.erase(s.plans.begin() + (long)i);
+        } else {
+            ++i;
+        }
+    }
+    for (size_t i = 0; i < s.graphs.size();) {
+        if (s.graphs[i].d_ptr_l == d_ptr || s.graphs[i].d_ptr_r == d_ptr) s.graphs.erase(s.graphs.begin() + (long)i);
+        else ++i;
+    }
+    return MGGX_OK;
+}
+
 }  // namespace mggx
 
 using mggx::fail;
+
+MGGX_EXPORT int mggx_forget(const void *d_ptr)
+{
+    if (!d_ptr) return MGGX_OK;
+    return mggx::forget_pointer(d_ptr);
+}
 
 MGGX_EXPORT int mggx_build_part_device(const int *d_indptr, int num_nodes, int part_size, int compat, int *d_part_ptr,
                                        int *d_part2node, int *d_node2part, int *num_parts)

@@ -107,6 +107,8 @@ MGGX_EXPORT int mggx_malloc(void **d_ptr, size_t bytes)
 MGGX_EXPORT int mggx_free(void *d_ptr)
 {
     if (!d_ptr) return MGGX_OK;
+    int rc = mggx::forget_pointer(d_ptr);  // a later allocation may get the same address
+    if (rc) return rc;
     MGGX_HIP(hipFree(d_ptr));
     return MGGX_OK;
 }

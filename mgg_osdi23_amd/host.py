@@ -52,7 +52,7 @@ EXPORTS = [
     "mggx_last_error", "mggx_version", "mggx_init", "mggx_device_name", "mggx_set_stream", "mggx_sync",
     "mggx_malloc", "mggx_free", "mggx_memset", "mggx_memcpy_h2d", "mggx_memcpy_d2h", "mggx_memcpy_d2d",
     "mggx_timer_create", "mggx_timer_start", "mggx_timer_stop", "mggx_timer_elapsed_ms", "mggx_timer_destroy",
-    "mggx_release_cached", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_graph_read",
+    "mggx_release_cached", "mggx_forget", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
     "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_compact_remote_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_mlp2_xw", "mggx_spmm",
     "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_gather_probe", "mggx_gather_rows", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
@@ -272,8 +272,18 @@ def _pin(*tensors) -> None:
     if key in _pinned:
         return
     _pinned[key] = tensors
-    while len(_pinned) > 256:  # the library remembers at most 16 plans and 32 CSRs; anything older is forgotten there
-        _pinned.pop(next(iter(_pinned)))
+    while len(_pinned) > 256:  # before the oldest set may be freed, the library forgets what it cached for it
+        old = _pinned.pop(next(iter(_pinned)))
+        for t in old:
+            if t is not None:
+                _check(lib().mggx_forget(C.c_void_p(t.data_ptr())))
+
+
+def forget(tensor) -> None:
+    """Drops the plans and search results the library keeps for this CSR tensor (call before rewriting it in place)."""
+    _check(lib().mggx_forget(C.c_void_p(tensor.data_ptr())))
+    for key in [k for k in _pinned if tensor.data_ptr() in k]:
+        _pinned.pop(key)
 
 
 def release_cached() -> None:

@@ -362,6 +362,28 @@ def test_plan_cache_eviction_and_release(gpu):
         gpu.release_cached()
 
 
+def test_forget_lets_a_csr_array_be_rewritten(gpu):
+    """The plan cache is keyed by address: after forget(), the same device arrays may hold another graph."""
+    import torch
+    V, dim = 500, 16
+    x = gpu.fill_normal((V, dim), seed=9)
+    d_x = to_dev(x)
+    z = torch.zeros(V + 1, dtype=torch.int32, device="cuda")
+    d_ptr = torch.zeros(V + 1, dtype=torch.int32, device="cuda")
+    d_col = torch.zeros(40000, dtype=torch.int32, device="cuda")
+    for seed in (1, 2):
+        ptr, col = gpu.gen_rmat(9, V, 6000, seed=seed)
+        assert len(col) <= 40000
+        gpu.forget(d_ptr)
+        d_ptr.copy_(torch.from_numpy(ptr))
+        d_col[:len(col)].copy_(torch.from_numpy(col))
+        out = torch.empty(V, dim, device="cuda")
+        gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, z, z, 0, V, dim, V, 0, 16, 4, 2)
+        gpu.sync()
+        want = orc.sag_np_div(x, x, ptr, col, None, None, 0, V, dim, V)
+        assert np.allclose(out.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
+
+
 # --------------------------------------------------------------------------- widths, strides, options
 @pytest.mark.parametrize("dim", [1, 2, 3, 4, 5, 8, 12, 16, 17, 24, 32, 41, 47, 64, 100, 128, 200, 256])
 def test_feature_widths(gpu, rmat_graph, dim):
