@@ -146,24 +146,33 @@ struct Gather {
     unsigned ld_bytes;
     unsigned sofs[4];      // strided mode: byte offsets of this lane's 4 elements inside a row
 
-    __device__ __forceinline__ void load(float (&v)[NV], int row) const
+    // The 16 bytes this lane holds of one row, as loaded (unpacked only when summed, so a batch in flight costs four
+    // registers per row whatever the element type).
+    __device__ __forceinline__ v4u load(int row) const
     {
         if constexpr (BUF) {
             const unsigned off = ((unsigned)row & 0xFFFFFFu) * ld24 + cbase;
             if constexpr (MODE == MODE_F32_STRIDED) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    v[i] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, off + sofs[i], 0, 0));
+                v4u t;
+                t.x = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off + sofs[0], 0, 0);
+                t.y = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off + sofs[1], 0, 0);
+                t.z = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off + sofs[2], 0, 0);
+                t.w = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off + sofs[3], 0, 0);
+                return t;
             } else {
-                unpack16<MODE>(v, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0));
+                return __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
             }
         } else {
             const char *p = row >= 0 ? base + (unsigned long long)(unsigned)row * ld_bytes : zero;
             if constexpr (MODE == MODE_F32_STRIDED) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) v[i] = *reinterpret_cast<const float *>(p + sofs[i]);
+                v4u t;
+                t.x = *reinterpret_cast<const unsigned *>(p + sofs[0]);
+                t.y = *reinterpret_cast<const unsigned *>(p + sofs[1]);
+                t.z = *reinterpret_cast<const unsigned *>(p + sofs[2]);
+                t.w = *reinterpret_cast<const unsigned *>(p + sofs[3]);
+                return t;
             } else {
-                unpack16<MODE>(v, *reinterpret_cast<const v4u *>(p));
+                return *reinterpret_cast<const v4u *>(p);
             }
         }
     }
@@ -375,28 +384,29 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
             static_for<0, CH / BATCH>([&](auto bb) {
                 constexpr int b = decltype(bb)::value;
                 if (__any(len > k0 + b * BATCH)) {
-                    float v[BATCH][NV];
+                    v4u raw[BATCH];
                     int rid[BATCH];
                     static_for<0, BATCH>([&](auto tt) {
                         constexpr int t = decltype(tt)::value;
                         constexpr int k = b * BATCH + t;
                         rid[t] = slot_bcast<LPR, k / IPL>(ids[k % IPL], slot_base);
-#pragma unroll
-                        for (int i = 0; i < NV; ++i) v[t][i] = 0.0f;
+                        raw[t] = (v4u){0u, 0u, 0u, 0u};
                     });
                     // lanes past the row width issue no load at all: a quad of idle lanes costs the address unit nothing
                     if (lane_on) {
                         static_for<0, BATCH>([&](auto tt) {
                             constexpr int t = decltype(tt)::value;
-                            g.load(v[t], rid[t]);
+                            raw[t] = g.load(rid[t]);
                         });
                     }
                     // keep every load of the batch in flight before the first sum waits on one
                     __builtin_amdgcn_sched_barrier(0);
                     static_for<0, BATCH>([&](auto tt) {
                         constexpr int t = decltype(tt)::value;
+                        float v[NV];
+                        unpack16<MODE>(v, raw[t]);
 #pragma unroll
-                        for (int i = 0; i < NV; ++i) acc[i] += v[t][i];
+                        for (int i = 0; i < NV; ++i) acc[i] += v[i];
                     });
                 }
             });
