@@ -113,8 +113,10 @@ MEASURED_TRAFFIC = {
 }
 
 
-def load_traffic(kernel_key, args, blk=-1):
+def load_traffic(kernel_key, args, blk=-1, core=-1):
     """{"traffic": bytes or None, "traffic_measured_at": knobs} for the roofline object."""
+    if core > 0:
+        kernel_key += "_core%d" % core
     if blk > 0:
         if blk != 49152:
             return {"traffic": None}
@@ -123,7 +125,8 @@ def load_traffic(kernel_key, args, blk=-1):
             (kernel_key == "big_agg" and args.big_scale != 0) or kernel_key not in MEASURED_TRAFFIC:
         return {"traffic": None}
     nbytes, (w, d) = MEASURED_TRAFFIC[kernel_key]
-    return {"traffic": nbytes, "traffic_measured_at": "ps=16 wpb=%d dist=%d%s" % (w, d, ", column blocks of 49152 ids" if blk > 0 else "")}
+    return {"traffic": nbytes, "traffic_measured_at": "ps=16 wpb=%d dist=%d%s%s" % (w, d, ", column blocks of 49152 ids" if blk > 0 else "",
+                                                                                 ", dense core of %d rows" % core if core > 0 else "")}
 
 
 class Knobs:
@@ -132,11 +135,13 @@ class Knobs:
     reference fixes its setting per dataset from the same kind of sweep, bench_MGG_DSE_*.py)."""
 
     def __init__(self, args, tune):
-        self.ps, self.wpb, self.dist, self.blk = args.ps, args.wpb, args.dist, args.col_block_rows
+        self.ps, self.wpb, self.dist, self.blk, self.core = args.ps, args.wpb, args.dist, args.col_block_rows, args.core_rows
         if args.wpb == 0 and args.dist == 0 and not args.no_tune:
-            k, ms = tune(args.ps, args.col_block_rows)
-            self.ps, self.wpb, self.dist, self.blk = k["ps"], k["wpb"], k["dist"], k["col_block_rows"]
+            k, ms = tune(args.ps, args.col_block_rows, args.core_rows)
+            self.ps, self.wpb, self.dist, self.blk, self.core = k["ps"], k["wpb"], k["dist"], k["col_block_rows"], k["core_rows"]
             log("search: %s (%.4f ms)" % (self, ms))
+        elif self.core == 0:
+            self.core = -1  # left to the rule: off
 
     def observe(self, host, call):
         """Where the order was left to the library's rule: run the call once and read back which order it used."""
@@ -146,9 +151,10 @@ class Knobs:
             self.blk = 49152 if m and int(m.group(1)) > 1 else -1
 
     def __str__(self):
-        return "ps=%d wpb=%d dist=%d %s" % (self.ps, self.wpb, self.dist,
-                                            "column blocks of %d ids" % self.blk if self.blk > 0 else
-                                            ("plain order" if self.blk < 0 else "order by rule"))
+        return "ps=%d wpb=%d dist=%d %s%s" % (self.ps, self.wpb, self.dist,
+                                              "column blocks of %d ids" % self.blk if self.blk > 0 else
+                                              ("plain order" if self.blk < 0 else "order by rule"),
+                                              ", dense core of %d rows from LDS" % self.core if self.core > 0 else "")
 
 
 def bench_gcn2(args, torch, host):
@@ -191,17 +197,17 @@ def bench_gcn2(args, torch, host):
 
     d_Y1.zero_()
     d_Y2.zero_()
-    k1 = Knobs(args, lambda ps, blk: host.tune_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, ps,
-                                                      row_scale_out=d_s, col_block_rows=blk))
-    k2 = Knobs(args, lambda ps, blk: host.tune_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, ps,
-                                                      row_scale_out=d_s, col_block_rows=blk, ld_in=pitch, ld_out=pitch))
+    k1 = Knobs(args, lambda ps, blk, core: host.tune_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, ps,
+                                                      row_scale_out=d_s, col_block_rows=blk, core_rows=core))
+    k2 = Knobs(args, lambda ps, blk, core: host.tune_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, ps,
+                                                      row_scale_out=d_s, col_block_rows=blk, core_rows=core, ld_in=pitch, ld_out=pitch))
     stages = [
         lambda: host.dense_forward(d_Y1, d_X, d_W1, V, in_dim, hidden, row_scale=d_s),
         lambda: host.mgg_SAG_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, k1.ps, k1.wpb, k1.dist,
-                                    row_scale_out=d_s, col_block_rows=k1.blk),
+                                    row_scale_out=d_s, col_block_rows=k1.blk, core_rows=k1.core),
         lambda: host.dense_forward(d_Y2, d_H1, d_W2, V, hidden, ldo, row_scale=d_s, ld_out=pitch),
         lambda: host.mgg_SAG_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, 0, k2.ps, k2.wpb, k2.dist,
-                                    row_scale_out=d_s, col_block_rows=k2.blk, ld_in=pitch, ld_out=pitch),
+                                    row_scale_out=d_s, col_block_rows=k2.blk, core_rows=k2.core, ld_in=pitch, ld_out=pitch),
         lambda: host.softmax_forward(d_P, d_H2, V, out_dim, ld_in=pitch),
     ]
     names = ["dense1", "agg1", "dense2", "agg2", "softmax"]
@@ -231,7 +237,7 @@ def bench_gcn2(args, torch, host):
     achieved = dom_bytes / (avg[dom] * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "k_agg (%s, dim %d)" % (dom, out_dim if dom == "agg2" else hidden),
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("gcn2_" + dom, args, (k2 if dom == "agg2" else k1).blk),
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("gcn2_" + dom, args, (k2 if dom == "agg2" else k1).blk, (k2 if dom == "agg2" else k1).core),
                 "algorithmic_bytes": dom_bytes, "avg_launch_ms": round(avg[dom], 4)}
     # the table of either aggregation stays in cache (15 / 45 MB): the bound that applies is the L2's gather rate
     roofline["cache_resident_table"] = gather_ceiling(torch, host, (pitch if dom == "agg2" else hidden) * 4,
@@ -254,9 +260,9 @@ def bench_gcn2(args, torch, host):
     alt = [
         lambda: host.dense_forward(d_Y1, d_X, d_W1, V, in_dim, hidden, row_scale=d_s),
         lambda: host.mgg_SAG_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, k1.ps, k1.wpb, k1.dist,
-                                    row_scale_out=d_s2, col_block_rows=k1.blk),
+                                    row_scale_out=d_s2, col_block_rows=k1.blk, core_rows=k1.core),
         lambda: host.mgg_SAG_np_div(d_G, d_H1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, 0, k1.ps, k1.wpb, k1.dist,
-                                    row_scale_out=d_s, col_block_rows=k1.blk),
+                                    row_scale_out=d_s, col_block_rows=k1.blk, core_rows=k1.core),
         lambda: host.dense_forward(d_Y2b, d_G, d_W2u, V, hidden, out_dim),
         lambda: host.softmax_forward(d_P2, d_Y2b, V, out_dim),
     ]
@@ -332,12 +338,12 @@ def bench_share(args, torch, host):
     d_xl = torch.from_numpy(np.ascontiguousarray(x_remote[lb:ub])).to(dev)  # separate allocation
     d = [torch.from_numpy(a).to(dev) if len(a) else torch.zeros(1, dtype=torch.int32, device=dev) for a in (lp, lc, rp, rc)]
     d_out = torch.empty(R, dim, device=dev)
-    kn = Knobs(args, lambda ps, blk: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, ps, input_remote=d_xr,
-                                                      col_block_rows=blk))
+    kn = Knobs(args, lambda ps, blk, core: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, ps, input_remote=d_xr,
+                                                      col_block_rows=blk, core_rows=core))
 
     def call():
         host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, kn.ps, kn.wpb, kn.dist, input_remote=d_xr,
-                            col_block_rows=kn.blk)
+                            col_block_rows=kn.blk, core_rows=kn.core)
 
     kn.observe(host, call)
     for _ in range(args.warmup):
@@ -391,10 +397,10 @@ def compact_variant(args, torch, host, d_out, d_xl, d_xr, d, rc, lb, ub, dim, np
     stage = lambda: host.gather_rows(d_xc, d_xr, d_ids, len(ids), dim * esize)
     stage()
     want = d_out.clone()  # produced from the global-id table by the caller
-    kn = Knobs(args, lambda ps, blk: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d_rcc, lb, ub, dim, npp, ps, input_remote=d_xc,
-                                                      col_block_rows=blk))
+    kn = Knobs(args, lambda ps, blk, core: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d_rcc, lb, ub, dim, npp, ps, input_remote=d_xc,
+                                                      col_block_rows=blk, core_rows=core))
     call = lambda: host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], d_rcc, lb, ub, dim, npp, 0, kn.ps, kn.wpb, kn.dist,
-                                       input_remote=d_xc, col_block_rows=kn.blk)
+                                       input_remote=d_xc, col_block_rows=kn.blk, core_rows=kn.core)
     for _ in range(args.warmup):
         call()
     timer = StageTimer(torch, ["agg", "stage"])
@@ -439,12 +445,12 @@ def bench_gin(args, torch, host):
     d_P = torch.empty(V, out_dim, device=dev)
 
     d_Y.zero_()
-    kn = Knobs(args, lambda ps, blk: host.tune_np_div(d_H, d_Y, d_ptr, d_col, zp, zc, 0, V, hidden, V, ps, gin_eps=eps, col_block_rows=blk))
+    kn = Knobs(args, lambda ps, blk, core: host.tune_np_div(d_H, d_Y, d_ptr, d_col, zp, zc, 0, V, hidden, V, ps, gin_eps=eps, col_block_rows=blk, core_rows=core))
     stages, names = [lambda: host.dense_forward(d_Y, d_X, d_W0, V, in_dim, hidden)], ["dense0"]
     for l in range(L):
         last = l == L - 1
         stages.append(lambda: host.mgg_GIN_np_div(d_H, d_Y, d_ptr, d_col, zp, zc, 0, V, hidden, V, 0, kn.ps, kn.wpb, kn.dist, eps,
-                                                  col_block_rows=kn.blk))
+                                                  col_block_rows=kn.blk, core_rows=kn.core))
         if args.unfused_mlp:
             stages.append(lambda l=l: host.dense_forward(d_T, d_H, d_Wa[l], V, hidden, hidden, relu=True))
             if last:
@@ -532,11 +538,11 @@ def bench_big(args, torch, host):
     W = host.glorot(dim, dim, seed=6)
     d_W = torch.from_numpy(W).to(dev).to(torch.bfloat16)
     d_next = torch.empty(R, dim, device=dev, dtype=torch.bfloat16)
-    kn = Knobs(args, lambda ps, blk: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, ps, input_remote=d_xr,
-                                                      col_block_rows=blk))
+    kn = Knobs(args, lambda ps, blk, core: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, ps, input_remote=d_xr,
+                                                      col_block_rows=blk, core_rows=core))
     stages = [
         lambda: host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, kn.ps, kn.wpb, kn.dist, input_remote=d_xr,
-                                    col_block_rows=kn.blk),
+                                    col_block_rows=kn.blk, core_rows=kn.core),
         lambda: host.dense_forward_bf16(d_next, d_out, d_W, R, dim, dim),
     ]
     for _ in range(args.warmup):
@@ -722,6 +728,8 @@ def main():
     ap.add_argument("--ps", type=int, default=16, help="partSize; 0 = let the library choose (the search then tries 16 and 32)")
     ap.add_argument("--col-block-rows", type=int, default=0, help="column-blocked partition order: 0 = library decides, -1 = off, "
                          "N = blocks of N neighbor ids")
+    ap.add_argument("--core-rows", type=int, default=0, help="dense core served from LDS: 0 = the search decides, -1 = off, "
+                         "N = the N highest-degree rows")
     ap.add_argument("--wpb", type=int, default=0, help="wavefronts per workgroup; 0 = let the library choose")
     ap.add_argument("--dist", type=int, default=0, help="interleaved_dist; 0 = let the library choose.  With --wpb 0 --dist 0 (the default) the "
                          "library's search picks the pair once per aggregation shape before the timed region")

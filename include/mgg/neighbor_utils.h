@@ -30,6 +30,7 @@ struct mgg_runtime_options {
     bool accumulate = true;              // mgg_SAG_np_div adds into `output` as the reference does (:1458)
     bool synchronize = true;             // the reference waits for the device after every call (:835)
     int col_block_rows = 0;              // column-blocked partition order: 0 = library decides, -1 = off, N = ids per block
+    int core_rows = 0;                   // dense core served from LDS: 0 = library decides, -1 = off, N = rows in the core
 };
 inline mgg_runtime_options &mgg_options()
 {
@@ -124,6 +125,7 @@ inline void mgg_SAG_np_div(float *output, const float *input, const nidType *row
     mggx_agg_opts o{};
     o.flags = mgg_options().accumulate ? MGGX_AGG_ACCUMULATE : 0;
     o.col_block_rows = mgg_options().col_block_rows;
+    o.core_rows = mgg_options().core_rows;
     const void *remote = mgg_options().remote_table ? mgg_options().remote_table : input;
     mgg_finish_call(mggx_sag_np_div(output, input, remote, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb,
                                     ub, dim, nodePerPE, np_size, warpPerBlock, interleaved_dist, &o),
@@ -141,6 +143,7 @@ inline void mgg_GIN_np_div(float *output, const float *input, const nidType *row
     o.flags = MGGX_AGG_GIN;
     o.eps = eps;
     o.col_block_rows = mgg_options().col_block_rows;
+    o.core_rows = mgg_options().core_rows;
     const void *remote = mgg_options().remote_table ? mgg_options().remote_table : input;
     mgg_finish_call(mggx_sag_np_div(output, input, remote, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb,
                                     ub, dim, nodePerPE, np_size, warpPerBlock, interleaved_dist, &o),
@@ -158,6 +161,7 @@ inline mggx_agg_knobs mgg_tune_np_div(float *output, const float *input, const n
 {
     mggx_agg_opts o{};
     o.col_block_rows = mgg_options().col_block_rows;
+    o.core_rows = mgg_options().core_rows;
     mggx_agg_knobs k{};
     const void *remote = mgg_options().remote_table ? mgg_options().remote_table : input;
     mgg_finish_call(mggx_sag_np_div_tune(output, input, remote, row_pointers_l, column_index_l, row_pointers_r, column_index_r,

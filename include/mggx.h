@@ -106,6 +106,20 @@ int mggx_split_csr(const int *ptr, const int *col, int lb, int ub,
 int mggx_compact_remote(const int *remote_col, int64_t n_remote, int *remote_col_compact, int *fetch_ids,
                         int64_t *n_unique);
 
+/* Layout of the dense-core path (no counterpart in the reference), exposed for inspection and tests: ranks the rows of
+ * a local CSR by degree (ties by id), takes the first core_rows (rounded down to a multiple of 512) as the core, and
+ * splits the CSR into the core x core block -- as index lists per 64-row slice and tile of tile_cols core columns
+ * (256 in the library), lists of a slice padded with 0xFFFF to the longest, in chunks of 4:
+ * idx[((blk_off[g * ntiles + t] + k / 4) * 64 + lane) * 4 + k % 4] = tile offset of the k-th core neighbor of the row
+ * of rank 64 g + lane inside tile t -- and the remaining CSR (rem_ptr, rem_col: row and edge order kept, ids unchanged).
+ * build returns sizes[5] = {core rows, entries of blk_off, entries of idx, entries of rem_col, edges in the core block};
+ * fetch copies the arrays out (any may be NULL) and releases the handle: order[core], rank[rows] (-1 outside the core),
+ * blk_off, idx, rem_ptr[rows + 1], rem_col. */
+int mggx_core_layout_build(const int *ptr, const int *col, int rows, int lb, int core_rows, int tile_cols, void **handle,
+                           int64_t *sizes);
+int mggx_core_layout_fetch(void *handle, int *order, int *rank, unsigned *blk_off, unsigned short *idx, int *rem_ptr,
+                           int *rem_col);
+
 /* build_part<int> (include/neighbor_utils.cuh:411-460).  part_ptr has
  * num_parts+1 entries, part2node num_parts, node2part num_nodes+2 (the
  * reference's layout).  compat != 0 reproduces the reference's terminal entry
@@ -182,11 +196,13 @@ typedef struct mggx_agg_opts {
     const float *d_row_scale_out;/* [ub-lb] multiplies each finished sum (NULL = 1) */
     int in_dtype;                /* MGGX_F32 or MGGX_BF16 (out is always fp32) */
     int col_block_rows;          /* column-blocked order: 0 = library decides, -1 = off, > 0 = neighbor ids per block */
+    int core_rows;               /* dense core served from LDS: 0 = library decides, -1 = off, > 0 = rows in the core */
 } mggx_agg_opts;
 
 typedef struct mggx_agg_knobs {
     int ps, wpb, dist;           /* partSize / warpPerBlock / interleaved_dist */
     int col_block_rows;          /* > 0: column-blocked with that many ids per block; -1: plain order */
+    int core_rows;               /* > 0: dense core of that many rows; -1: none */
 } mggx_agg_knobs;
 
 /* mgg_SAG_np_div / mgg_GIN_np_div (include/neighbor_utils.cuh:787-841, 902-958;
@@ -205,6 +221,12 @@ typedef struct mggx_agg_knobs {
  * (>= 20 neighbors per block and row), the partitions are walked block by block of neighbor ids, so the part of the
  * feature table in use at any time is small enough to stay in cache; each block leaves a partial row in library
  * scratch and a second kernel sums them in block order and applies the epilogue.  Same result up to summation order.
+ * Dense core (opts->core_rows; fp32, local-only CSR, dim <= 64): the core_rows highest-degree rows (rounded down to a
+ * multiple of 512) are ranked by degree; the edges among them leave the CSR and are summed from LDS -- the feature rows
+ * of 256 core columns at a time staged with whole-line reads, one lane per core row walking an index list -- and the
+ * rest of the CSR runs as usual on top.  Pays on graphs whose high-degree rows hold most edges among themselves; its
+ * plan is built on the host (the CSR is copied back once), so by rule it is off and mggx_sag_np_div_tune turns it on
+ * where it measures faster.  Same result up to summation order.
  * The partition plan of (d_ptr_l, d_ptr_r, d_col_r, rows, ps) -- and d_col_l for the column-blocked order -- is built on first use and
  * cached by pointer identity: the CSR arrays must not be rewritten in place or freed
  * while cached (mggx_forget() drops what hangs on one array, mggx_release_cached() everything). */
@@ -215,10 +237,11 @@ int mggx_sag_np_div(float *d_out, const void *d_in_local, const void *d_in_remot
 
 /* The design-space search of bench_MGG_DSE_dist_ps.py:12-42 / bench_MGG_DSE_dist_wpb.py (one process launch per
  * setting there) as one call: runs the aggregation of mggx_sag_np_div over ps (as given, or {16, 32} when 0) x plain /
- * column-blocked order (where the rows are long enough, unless opts fixes it) x wpb in {4, 8, 16} x dist in
+ * column-blocked order (where the rows are long enough, unless opts fixes it) x without a dense core / with one of
+ * 16, 24 or 32 Ki rows (where eligible, unless opts fixes it) x wpb in {4, 8, 16} x dist in
  * {1, 2, 4, 8, 16}, three runs each (the faster of the last two counts), returns the fastest setting and its time, and
  * remembers it, so later mggx_sag_np_div calls on the same CSR arrays with the same dim and in_dtype that leave
- * wpb = dist = col_block_rows = 0 (and ps = 0 or the winning ps) use it.  d_out holds a valid result afterwards.
+ * wpb = dist = col_block_rows = core_rows = 0 (and ps = 0 or the winning ps) use it.  d_out holds a valid result afterwards.
  * Synchronises; not for stream capture.  MGGX_AGG_ACCUMULATE is rejected (the repeated runs would add up).
  * Either out-pointer may be NULL. */
 int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const void *d_in_remote,

@@ -21,7 +21,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 BUILD = os.path.join(PKG_DIR, "build")
 LIB = os.path.join(PKG_DIR, "libmggx.so")
 
-HIP_SOURCES = ["mggx_runtime.hip", "mggx_plan.hip", "mggx_agg.hip", "mggx_dense.hip", "mggx_prep.hip"]
+HIP_SOURCES = ["mggx_runtime.hip", "mggx_plan.hip", "mggx_agg.hip", "mggx_dense.hip", "mggx_prep.hip", "mggx_core.hip"]
 HOST_SOURCES = ["mggx_host.cpp"]
 HEADERS = [os.path.join(CSRC, "mggx_internal.h"), os.path.join(CSRC, "mggx_dev.h"), os.path.join(ROOT, "include", "mggx.h")]
 

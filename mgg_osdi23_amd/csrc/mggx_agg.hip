@@ -18,6 +18,7 @@
 //   workgroups a row that crosses workgroups leaves two partial rows in a
 //              carry buffer; a small second kernel sums them in a fixed order
 // No atomics anywhere; the summation order depends only on (ps, wpb, dist, dim).
+#include <cstring>
 #include <type_traits>
 
 #include "mggx_dev.h"
@@ -592,7 +593,7 @@ __global__ void __launch_bounds__(256) k_agg_block_reduce(const AggArgs a, const
 }
 
 // The same with four columns per thread, for outputs that take 16-byte stores and epilogues without a read of
-// other tables (row scale and ReLU only).
+// other tables (row scale, accumulation and ReLU only).
 __global__ void __launch_bounds__(256) k_agg_block_reduce4(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp)
 {
     const int q = a.dim >> 2;  // float4 per row
@@ -608,10 +609,15 @@ __global__ void __launch_bounds__(256) k_agg_block_reduce4(const AggArgs a, cons
         const float s = a.rs_out[v];
         t.x *= s; t.y *= s; t.z *= s; t.w *= s;
     }
+    float4 *o = reinterpret_cast<float4 *>(a.out + (long long)v * a.ld_out + d);
+    if (a.flags & MGGX_AGG_ACCUMULATE) {
+        const float4 p = *o;
+        t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
+    }
     if (a.flags & MGGX_AGG_RELU) {
         t.x = fmaxf(t.x, 0.f); t.y = fmaxf(t.y, 0.f); t.z = fmaxf(t.z, 0.f); t.w = fmaxf(t.w, 0.f);
     }
-    *reinterpret_cast<float4 *>(a.out + (long long)v * a.ld_out + d) = t;
+    *o = t;
 }
 
 int pow2_ceil(int x)
@@ -795,7 +801,7 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         r.ld_out = ld_out;
         r.rs_out = o.d_row_scale_out;
         r.flags = o.flags;
-        const bool vec4 = dim % 4 == 0 && ld_out % 4 == 0 && aligned16(d_out) && !(o.flags & (MGGX_AGG_GIN | MGGX_AGG_ACCUMULATE));
+        const bool vec4 = dim % 4 == 0 && ld_out % 4 == 0 && aligned16(d_out) && !(o.flags & MGGX_AGG_GIN);
         if (vec4) {
             const long long n = (long long)plan->real_rows * (dim / 4);
             k_agg_block_reduce4<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(r, part, plan->real_rows, plan->blocks, ldp);
@@ -830,18 +836,28 @@ bool blocking_eligible(const GraphInfo &g, int block_rows)
 
 struct Knobs {
     int ps, wpb, dist, block_rows;  // block_rows: > 0 column-blocked, -1 plain
+    int core_rows;                  // > 0: that many highest-degree rows form a dense core served from LDS, -1: none
 };
 
+// The dense-core path pays for a second pass over the output and a host-built plan: worth trying on a local-only fp32
+// CSR with many rows beyond the core and a mean degree in the hundreds.
+bool core_eligible(const GraphInfo &g, int dim, int dtype, int core_rows)
+{
+    return g.nnz_r == 0 && dtype == MGGX_F32 && dim <= 64 && g.rows >= 2 * (long long)core_rows && g.nnz_l >= 128 * (long long)g.rows;
+}
+
 // Fills in the knobs the caller left at 0: from the search's result for this CSR, width and element type, else by rule.
-Knobs resolve_knobs(const GraphInfo &g, int dim, int dtype, int ps, int wpb, int dist, int block_rows)
+Knobs resolve_knobs(const GraphInfo &g, int dim, int dtype, int ps, int wpb, int dist, int block_rows, int core_rows)
 {
     const GraphInfo::Tuned *t = nullptr;
     for (const GraphInfo::Tuned &e : g.tuned)
         if (e.dim == dim && e.dtype == dtype) t = &e;
-    Knobs k{ps, wpb, dist, block_rows};
-    if (t && (ps == 0 || ps == t->ps) && wpb == 0 && dist == 0 && block_rows == 0) return Knobs{t->ps, t->wpb, t->dist, t->block_rows};
+    Knobs k{ps, wpb, dist, block_rows, core_rows};
+    if (t && (ps == 0 || ps == t->ps) && wpb == 0 && dist == 0 && block_rows == 0 && core_rows == 0)
+        return Knobs{t->ps, t->wpb, t->dist, t->block_rows, t->core_rows};
     if (k.ps == 0) k.ps = 16;
     if (k.block_rows == 0) k.block_rows = blocking_eligible(g, DEFAULT_BLOCK_ROWS) ? DEFAULT_BLOCK_ROWS : -1;
+    if (k.core_rows == 0) k.core_rows = -1;  // by rule: off (its plan is built on the host); the search turns it on where it wins
     return k;
 }
 
@@ -850,6 +866,34 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
 {
     Plan *plan = nullptr;
     int rc;
+    if (k.core_rows > 0 && g.nnz_r == 0 && d_col_l && o.in_dtype == MGGX_F32 && dim <= 64 && d_out && d_in_local) {
+        CorePlan *cp = nullptr;
+        rc = core_plan_get(d_ptr_l, d_col_l, ub - lb, lb, k.core_rows, &cp);
+        if (rc) return rc;
+        if (!cp->unsuitable) {
+            // the core block first: out = (accumulate ? out : 0) + scale * core sums; then what is left of the CSR on top, with
+            // the caller's epilogue (its row scale applies to its own sums, the self term and the ReLU come last)
+            const long long ld_in = o.ld_in ? o.ld_in : dim, ld_out = o.ld_out ? o.ld_out : dim;
+            if (ld_in < dim || ld_out < dim) return fail(MGGX_EINVAL, "aggregation: row stride smaller than dim");
+            rc = run_core(cp, d_out, static_cast<const float *>(d_in_local), dim, ld_in, ld_out, o.d_row_scale_out,
+                          (o.flags & MGGX_AGG_ACCUMULATE) ? 1 : 0);
+            if (rc) return rc;
+            GraphInfo *gr = nullptr;
+            rc = graph_info(cp->d_rem_ptr, nullptr, ub - lb, &gr);
+            if (rc) return rc;
+            mggx_agg_opts o2 = o;
+            o2.flags |= MGGX_AGG_ACCUMULATE;
+            Knobs k2 = k;
+            k2.core_rows = -1;
+            if (k2.block_rows > 0 && !blocking_eligible(*gr, k2.block_rows)) k2.block_rows = -1;
+            rc = run_knobs(*gr, k2, d_out, d_in_local, nullptr, cp->d_rem_ptr, cp->d_rem_col, nullptr, nullptr, lb, ub, dim, o2);
+            if (rc) return rc;
+            State &st = state();
+            const size_t n = strlen(st.last_kernel);
+            snprintf(st.last_kernel + n, sizeof(st.last_kernel) - n, " core=%d", cp->core);
+            return MGGX_OK;
+        }
+    }
     if (k.block_rows > 0 && g.nnz_r == 0 && d_col_l && ub - lb >= 2 * (long long)k.block_rows) {
         rc = plan_get_blocked(d_ptr_l, d_col_l, ub - lb, lb, k.ps, k.block_rows, &plan);
         if (rc) return rc;
@@ -862,8 +906,9 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
     return run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, k.wpb, k.dist, o);
 }
 
-int check_np_div_args(const char *who, const int *d_ptr_l, int lb, int ub, int nodes_per_pe, int &ps, int block_rows)
+int check_np_div_args(const char *who, const int *d_ptr_l, int lb, int ub, int nodes_per_pe, int &ps, int block_rows, int core_rows)
 {
+    if (core_rows < -1) return fail(MGGX_EINVAL, "%s: core_rows %d (0 = choose, -1 = off)", who, core_rows);
     if (ub < lb || !d_ptr_l) return fail(MGGX_EINVAL, "%s: bad row range [%d,%d) or NULL row pointers", who, lb, ub);
     if (ps < 0) return fail(MGGX_EINVAL, "%s: ps %d must not be negative (0 = choose)", who, ps);
     if (nodes_per_pe < ub - lb) return fail(MGGX_EINVAL, "%s: nodes_per_pe %d smaller than the row range", who, nodes_per_pe);
@@ -883,12 +928,12 @@ MGGX_EXPORT int mggx_sag_np_div(float *d_out, const void *d_in_local, const void
     if (rc) return rc;
     mggx_agg_opts o{};
     if (opts) o = *opts;
-    rc = mggx::check_np_div_args("sag_np_div", d_ptr_l, lb, ub, nodes_per_pe, ps, o.col_block_rows);
+    rc = mggx::check_np_div_args("sag_np_div", d_ptr_l, lb, ub, nodes_per_pe, ps, o.col_block_rows, o.core_rows);
     if (rc) return rc;
     mggx::GraphInfo *g = nullptr;
     rc = mggx::graph_info(d_ptr_l, d_ptr_r, ub - lb, &g);
     if (rc) return rc;
-    const mggx::Knobs k = mggx::resolve_knobs(*g, dim, o.in_dtype, ps, wpb, dist, o.col_block_rows);
+    const mggx::Knobs k = mggx::resolve_knobs(*g, dim, o.in_dtype, ps, wpb, dist, o.col_block_rows, o.core_rows);
     return mggx::run_knobs(*g, k, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o);
 }
 
@@ -900,7 +945,7 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
     if (rc) return rc;
     mggx_agg_opts o{};
     if (opts) o = *opts;
-    rc = mggx::check_np_div_args("sag_np_div_tune", d_ptr_l, lb, ub, nodes_per_pe, ps, o.col_block_rows);
+    rc = mggx::check_np_div_args("sag_np_div_tune", d_ptr_l, lb, ub, nodes_per_pe, ps, o.col_block_rows, o.core_rows);
     if (rc) return rc;
     if (o.flags & MGGX_AGG_ACCUMULATE) return fail(MGGX_EINVAL, "sag_np_div_tune: repeated runs would accumulate; clear MGGX_AGG_ACCUMULATE");
     mggx::GraphInfo *g = nullptr;
@@ -916,15 +961,24 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
     int blks[2] = {-1, 0}, n_blk = 1;
     if (o.col_block_rows > 0) blks[0] = o.col_block_rows;
     else if (o.col_block_rows == 0 && mggx::blocking_eligible(*g, mggx::DEFAULT_BLOCK_ROWS)) { blks[1] = mggx::DEFAULT_BLOCK_ROWS; n_blk = 2; }
+    int cores[4] = {-1, 0, 0, 0}, n_core = 1;  // without a dense core and, where it may pay, with one of three sizes
+    if (o.core_rows > 0) {
+        cores[0] = o.core_rows;
+    } else if (o.core_rows == 0) {
+        static const int sizes[] = {16 * 1024, 24 * 1024, 32 * 1024};
+        for (int c : sizes)
+            if (mggx::core_eligible(*g, dim, o.in_dtype, c)) cores[n_core++] = c;
+    }
     static const int wpbs[] = {8, 4, 16}, dists[] = {1, 2, 4, 8, 16};
     float best = -1.f;
-    mggx::Knobs bk{pss[0], 8, 1, blks[0]};
+    mggx::Knobs bk{pss[0], 8, 1, blks[0], cores[0]};
     rc = mggx::run_knobs(*g, bk, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o);  // warm-up
+    for (int ci = 0; ci < n_core && !rc; ++ci)
     for (int pi = 0; pi < n_ps && !rc; ++pi)
         for (int bi = 0; bi < n_blk && !rc; ++bi)
             for (int wi = 0; wi < 3 && !rc; ++wi)
                 for (int di = 0; di < 5 && !rc; ++di) {
-                    const mggx::Knobs k{pss[pi], wpbs[wi], dists[di], blks[bi]};
+                    const mggx::Knobs k{pss[pi], wpbs[wi], dists[di], blks[bi], cores[ci]};
                     float ms_min = -1.f;
                     for (int rep = 0; rep < 3 && !rc; ++rep) {
                         hipError_t e = hipEventRecord(e0, st.stream);
@@ -946,9 +1000,9 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
     if (rc) return rc;
     bool found = false;
     for (mggx::GraphInfo::Tuned &t : g->tuned)
-        if (t.dim == dim && t.dtype == o.in_dtype) { t.ps = bk.ps; t.wpb = bk.wpb; t.dist = bk.dist; t.block_rows = bk.block_rows; found = true; }
-    if (!found) g->tuned.push_back({dim, o.in_dtype, bk.ps, bk.wpb, bk.dist, bk.block_rows});
-    if (best_out) { best_out->ps = bk.ps; best_out->wpb = bk.wpb; best_out->dist = bk.dist; best_out->col_block_rows = bk.block_rows; }
+        if (t.dim == dim && t.dtype == o.in_dtype) { t.ps = bk.ps; t.wpb = bk.wpb; t.dist = bk.dist; t.block_rows = bk.block_rows; t.core_rows = bk.core_rows; found = true; }
+    if (!found) g->tuned.push_back({dim, o.in_dtype, bk.ps, bk.wpb, bk.dist, bk.block_rows, bk.core_rows});
+    if (best_out) { best_out->ps = bk.ps; best_out->wpb = bk.wpb; best_out->dist = bk.dist; best_out->col_block_rows = bk.block_rows; best_out->core_rows = bk.core_rows; }
     if (ms_best) *ms_best = best;
     return MGGX_OK;
 }
@@ -981,6 +1035,6 @@ MGGX_EXPORT int mggx_spmm(float *d_out, const float *d_in, const int *d_row_ptr,
     rc = mggx::graph_info(d_row_ptr, nullptr, num_nodes, &g);
     if (rc) return rc;
     // the whole graph on one GPU: the same knob rules (and column-blocked order for long rows) as mggx_sag_np_div
-    mggx::Knobs k = mggx::resolve_knobs(*g, dim, MGGX_F32, ps, wpb, 0, 0);
+    mggx::Knobs k = mggx::resolve_knobs(*g, dim, MGGX_F32, ps, wpb, 0, 0, 0);
     return mggx::run_knobs(*g, k, d_out, d_in, nullptr, d_row_ptr, d_col, nullptr, nullptr, 0, num_nodes, dim, o);
 }

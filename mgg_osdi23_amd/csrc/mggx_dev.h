@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <list>
 #include <vector>
 
 #include "mggx_internal.h"
@@ -65,6 +66,22 @@ struct Plan {
     bool unsuitable = false;   // blocked plan asked for, but the rows are not sorted by neighbor id
 };
 
+// Dense-core plan of a local-only CSR (layout: CoreLayout in mggx_internal.h), built on the host and kept on the device.
+struct CorePlan {
+    // cache key
+    const int *d_ptr_l = nullptr;
+    const int *d_col_l = nullptr;
+    int rows = 0, lb = 0, asked = 0;
+    // contents
+    int core = 0, ntiles = 0, nseg = 1;
+    int64_t core_nnz = 0, rem_nnz = 0;
+    int *d_order = nullptr, *d_rank = nullptr;
+    unsigned *d_blk_off = nullptr;
+    unsigned short *d_idx = nullptr;
+    int *d_rem_ptr = nullptr, *d_rem_col = nullptr;
+    bool unsuitable = false;  // no core of whole units fits, or the ids do not allow it
+};
+
 // What is known about a CSR the aggregation has been called with (keyed by pointer identity).
 struct GraphInfo {
     const int *d_ptr_l = nullptr;
@@ -72,7 +89,7 @@ struct GraphInfo {
     int rows = 0;
     int64_t nnz_l = 0, nnz_r = 0;
     // knobs measured best by mggx_sag_np_div_tune for a row width and element type; used where a call passes 0
-    struct Tuned { int dim, dtype, ps, wpb, dist, block_rows; };
+    struct Tuned { int dim, dtype, ps, wpb, dist, block_rows, core_rows; };
     std::vector<Tuned> tuned;
 };
 
@@ -82,7 +99,10 @@ struct State {
     void *ws = nullptr;
     size_t ws_bytes = 0;
     std::vector<Plan *> plans;
-    std::vector<GraphInfo> graphs;
+    std::list<GraphInfo> graphs;  // least recently used first; a list, so records stay where they are while others come and go
+    std::vector<CorePlan *> cores;
+    void *core_ws = nullptr;      // staged core table and partial rows of the dense-core path (grow-only)
+    size_t core_ws_bytes = 0;
     char last_kernel[160] = "";
     int gather_addressing = 0;  // 0 = choose per call, 1 = always 64-bit addresses
 };
@@ -104,6 +124,10 @@ int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_
                       int num_parts, int ps, Plan **out);
 void plan_free(Plan *p);
 int forget_pointer(const void *d_ptr);
+int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, CorePlan **out);
+void core_plan_free(CorePlan *p);
+int run_core(CorePlan *p, float *d_out, const float *d_in, int dim, long long ld_in, long long ld_out, const float *d_row_scale,
+             int accumulate);
 
 }  // namespace mggx
 #endif

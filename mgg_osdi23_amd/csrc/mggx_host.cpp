@@ -581,3 +581,132 @@ MGGX_EXPORT int mggx_fill_uniform(float *dst, int64_t n, float lo, float hi, uin
     }
     return MGGX_OK;
 }
+
+
+// ---------------------------------------------------------------------------
+// Dense-core layout (see mggx_internal.h).
+namespace mggx {
+
+int core_layout_build(const int *ptr, const int *col, int rows, int lb, int core, int tc, CoreLayout *out)
+{
+    if (!ptr || rows < 0 || tc < 64 || tc > 4096 || (tc % 64)) return fail(MGGX_EINVAL, "core layout: bad arguments");
+    if (core > rows) core = rows;
+    const int unit = tc > 512 ? tc : 512;  // whole workgroups of 8 slices and whole tiles
+    core = core / unit * unit;
+    if (core < unit || (unit % tc) || (unit % 512)) return fail(MGGX_EINVAL, "core layout: no core of whole %d-row units in %d rows", unit, rows);
+    if (ptr[rows] > 0 && !col) return fail(MGGX_EINVAL, "core layout: NULL column array");
+    CoreLayout &L = *out;
+    L.rows = rows;
+    L.core = core;
+    L.tc = tc;
+    L.ntiles = core / tc;
+    const int ntiles = L.ntiles, nslices = core / 64;
+    // rank by degree, ties by id
+    std::vector<int> ids((size_t)rows);
+    for (int v = 0; v < rows; ++v) ids[v] = v;
+    __gnu_parallel::stable_sort(ids.begin(), ids.end(), [&](int a, int b) { return ptr[a + 1] - ptr[a] > ptr[b + 1] - ptr[b]; });
+    L.order.assign(ids.begin(), ids.begin() + core);
+    L.rank.assign((size_t)rows, -1);
+    for (int i = 0; i < core; ++i) L.rank[L.order[i]] = i;
+    // pass 1: list lengths per (core row, tile); what every row keeps
+    std::vector<unsigned short> cnt((size_t)core * ntiles, 0);
+    L.rem_ptr.assign((size_t)rows + 1, 0);
+    int bad = 0;
+#pragma omp parallel for schedule(dynamic, 256) reduction(| : bad)
+    for (int v = 0; v < rows; ++v) {
+        const int i = L.rank[v];
+        int keep = 0;
+        for (int e = ptr[v]; e < ptr[v + 1]; ++e) {
+            const int u = col[e] - lb;
+            if (u < 0 || u >= rows) { bad = 1; ++keep; continue; }
+            const int j = L.rank[u];
+            if (i >= 0 && j >= 0) {
+                unsigned short &c = cnt[(size_t)i * ntiles + j / tc];
+                if (c == 0xFFFE) { bad = 1; ++keep; continue; }  // a list that long cannot be a simple graph's
+                ++c;
+            } else {
+                ++keep;
+            }
+        }
+        L.rem_ptr[v + 1] = keep;
+    }
+    if (bad) return fail(MGGX_EINVAL, "core layout: a neighbor id outside [lb, lb + rows), or more than 65533 parallel edges");
+    for (int v = 0; v < rows; ++v) L.rem_ptr[v + 1] += L.rem_ptr[v];
+    // block offsets
+    L.blk_off.assign((size_t)nslices * ntiles + 1, 0);
+    uint64_t chunks = 0;
+    for (int g = 0; g < nslices; ++g)
+        for (int t = 0; t < ntiles; ++t) {
+            int w = 0;
+            for (int l = 0; l < 64; ++l) w = std::max<int>(w, cnt[(size_t)(g * 64 + l) * ntiles + t]);
+            L.blk_off[(size_t)g * ntiles + t] = (unsigned)chunks;
+            chunks += (uint64_t)(w + 3) / 4;
+        }
+    if (chunks > 0xFFFFFFFFull / 64) return fail(MGGX_ELIMIT, "core layout: %llu list chunks", (unsigned long long)chunks);
+    L.blk_off[(size_t)nslices * ntiles] = (unsigned)chunks;
+    L.idx.assign((size_t)chunks * 256, (unsigned short)0xFFFF);
+    L.rem_col.assign((size_t)L.rem_ptr[rows], 0);
+    // pass 2: fill
+    int64_t core_nnz = 0;
+#pragma omp parallel reduction(+ : core_nnz)
+    {
+        std::vector<int> cur((size_t)ntiles);
+#pragma omp for schedule(dynamic, 256)
+        for (int v = 0; v < rows; ++v) {
+            const int i = L.rank[v];
+            int w = L.rem_ptr[v];
+            if (i >= 0) std::fill(cur.begin(), cur.end(), 0);
+            for (int e = ptr[v]; e < ptr[v + 1]; ++e) {
+                const int u = col[e] - lb;
+                const int j = L.rank[u];
+                if (i >= 0 && j >= 0) {
+                    const int t = j / tc, k = cur[t]++;
+                    const size_t chunk = (size_t)L.blk_off[(size_t)(i / 64) * ntiles + t] + (size_t)(k / 4);
+                    L.idx[(chunk * 64 + (size_t)(i % 64)) * 4 + (size_t)(k % 4)] = (unsigned short)(j % tc);
+                    ++core_nnz;
+                } else {
+                    L.rem_col[w++] = col[e];
+                }
+            }
+        }
+    }
+    L.core_nnz = core_nnz;
+    return MGGX_OK;
+}
+
+}  // namespace mggx
+
+MGGX_EXPORT int mggx_core_layout_build(const int *ptr, const int *col, int rows, int lb, int core_rows, int tile_cols, void **handle,
+                                       int64_t *sizes)
+{
+    if (!handle || !sizes) return fail(MGGX_EINVAL, "core_layout_build: NULL output");
+    std::unique_ptr<mggx::CoreLayout> L(new (std::nothrow) mggx::CoreLayout);
+    if (!L) return fail(MGGX_ENOMEM, "core_layout_build");
+    int rc;
+    try {
+        rc = mggx::core_layout_build(ptr, col, rows, lb, core_rows, tile_cols, L.get());
+    } catch (const std::bad_alloc &) {
+        return fail(MGGX_ENOMEM, "core_layout_build: out of host memory");
+    }
+    if (rc) return rc;
+    sizes[0] = L->core;
+    sizes[1] = (int64_t)L->blk_off.size();
+    sizes[2] = (int64_t)L->idx.size();
+    sizes[3] = (int64_t)L->rem_col.size();
+    sizes[4] = L->core_nnz;
+    *handle = L.release();
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_core_layout_fetch(void *handle, int *order, int *rank, unsigned *blk_off, unsigned short *idx, int *rem_ptr, int *rem_col)
+{
+    if (!handle) return fail(MGGX_EINVAL, "core_layout_fetch: NULL handle");
+    std::unique_ptr<mggx::CoreLayout> L(static_cast<mggx::CoreLayout *>(handle));
+    if (order) memcpy(order, L->order.data(), L->order.size() * sizeof(int));
+    if (rank) memcpy(rank, L->rank.data(), L->rank.size() * sizeof(int));
+    if (blk_off) memcpy(blk_off, L->blk_off.data(), L->blk_off.size() * sizeof(unsigned));
+    if (idx) memcpy(idx, L->idx.data(), L->idx.size() * sizeof(unsigned short));
+    if (rem_ptr) memcpy(rem_ptr, L->rem_ptr.data(), L->rem_ptr.size() * sizeof(int));
+    if (rem_col && !L->rem_col.empty()) memcpy(rem_col, L->rem_col.data(), L->rem_col.size() * sizeof(int));
+    return MGGX_OK;
+}

@@ -601,9 +601,10 @@ int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, i
 int graph_info(const int *d_ptr_l, const int *d_ptr_r, int rows, GraphInfo **out)
 {
     State &s = state();
-    for (GraphInfo &g : s.graphs)
-        if (g.d_ptr_l == d_ptr_l && g.d_ptr_r == d_ptr_r && g.rows == rows) {
-            *out = &g;
+    for (auto it = s.graphs.begin(); it != s.graphs.end(); ++it)
+        if (it->d_ptr_l == d_ptr_l && it->d_ptr_r == d_ptr_r && it->rows == rows) {
+            s.graphs.splice(s.graphs.end(), s.graphs, it);  // most recently used last; the record itself does not move
+            *out = &*it;
             return MGGX_OK;
         }
     GraphInfo g;
@@ -643,10 +644,19 @@ int forget_pointer(const void *d_ptr)
             ++i;
         }
     }
-    for (size_t i = 0; i < s.graphs.size();) {
-        if (s.graphs[i].d_ptr_l == d_ptr || s.graphs[i].d_ptr_r == d_ptr) s.graphs.erase(s.graphs.begin() + (long)i);
-        else ++i;
+    s.graphs.remove_if([d_ptr](const GraphInfo &g) { return g.d_ptr_l == d_ptr || g.d_ptr_r == d_ptr; });
+    // dense-core plans keyed by the array (freeing one forgets its own remainder arrays in turn: take them out first)
+    std::vector<CorePlan *> gone;
+    for (size_t i = 0; i < s.cores.size();) {
+        if (s.cores[i]->d_ptr_l == d_ptr || s.cores[i]->d_col_l == d_ptr) {
+            gone.push_back(s.cores[i]);
+            s.cores.erase(s.cores.begin() + (long)i);
+        } else {
+            ++i;
+        }
     }
+    if (!gone.empty() && !synced && s.device >= 0) MGGX_HIP(hipStreamSynchronize(s.stream));
+    for (CorePlan *c : gone) core_plan_free(c);
     return MGGX_OK;
 }
 

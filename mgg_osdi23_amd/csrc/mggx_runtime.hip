@@ -204,6 +204,16 @@ MGGX_EXPORT int mggx_release_cached(void)
 {
     mggx::State &s = state();
     if (s.device >= 0) MGGX_HIP(hipStreamSynchronize(s.stream));
+    {   // dense-core plans first: freeing one also forgets the plans of its remainder CSR
+        std::vector<mggx::CorePlan *> cores;
+        cores.swap(s.cores);
+        for (mggx::CorePlan *c : cores) mggx::core_plan_free(c);
+    }
+    if (s.core_ws) {
+        MGGX_HIP(hipFree(s.core_ws));
+        s.core_ws = nullptr;
+        s.core_ws_bytes = 0;
+    }
     for (mggx::Plan *p : s.plans) mggx::plan_free(p);
     s.plans.clear();
     s.graphs.clear();

@@ -29,11 +29,11 @@ class MggxError(RuntimeError):
 
 class _AggOpts(C.Structure):
     _fields_ = [("flags", C.c_uint32), ("eps", C.c_float), ("ld_in", C.c_int64), ("ld_out", C.c_int64),
-                ("d_row_scale_out", C.c_void_p), ("in_dtype", C.c_int), ("col_block_rows", C.c_int)]
+                ("d_row_scale_out", C.c_void_p), ("in_dtype", C.c_int), ("col_block_rows", C.c_int), ("core_rows", C.c_int)]
 
 
 class _AggKnobs(C.Structure):
-    _fields_ = [("ps", C.c_int), ("wpb", C.c_int), ("dist", C.c_int), ("col_block_rows", C.c_int)]
+    _fields_ = [("ps", C.c_int), ("wpb", C.c_int), ("dist", C.c_int), ("col_block_rows", C.c_int), ("core_rows", C.c_int)]
 
 
 class _DenseOpts(C.Structure):
@@ -52,7 +52,7 @@ EXPORTS = [
     "mggx_last_error", "mggx_version", "mggx_init", "mggx_device_name", "mggx_set_stream", "mggx_sync",
     "mggx_malloc", "mggx_free", "mggx_memset", "mggx_memcpy_h2d", "mggx_memcpy_d2h", "mggx_memcpy_d2d",
     "mggx_timer_create", "mggx_timer_start", "mggx_timer_stop", "mggx_timer_elapsed_ms", "mggx_timer_destroy",
-    "mggx_release_cached", "mggx_forget", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_graph_read",
+    "mggx_release_cached", "mggx_forget", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_core_layout_build", "mggx_core_layout_fetch", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
     "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_compact_remote_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_mlp2_xw", "mggx_spmm",
     "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_gather_probe", "mggx_gather_rows", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
@@ -321,7 +321,7 @@ def build_part_device(d_indptr, num_nodes: int, part_size: int, compat: bool = T
 
 
 def _agg(out, in_local, in_remote, ptr_l, col_l, ptr_r, col_r, lb, ub, dim, npp, ps, wpb, dist, flags, eps,
-         ld_in, ld_out, row_scale_out, col_block_rows=0):
+         ld_in, ld_out, row_scale_out, col_block_rows=0, core_rows=0):
     import torch
     o = _AggOpts()
     o.flags = flags
@@ -331,16 +331,18 @@ def _agg(out, in_local, in_remote, ptr_l, col_l, ptr_r, col_r, lb, ub, dim, npp,
     o.d_row_scale_out = row_scale_out.data_ptr() if row_scale_out is not None else None
     o.in_dtype = BF16 if in_local.dtype == torch.bfloat16 else F32
     o.col_block_rows = col_block_rows
+    o.core_rows = core_rows
     _pin(ptr_l, ptr_r, col_l, col_r)
     _check(lib().mggx_sag_np_div(_dptr(out), _dptr(in_local), _dptr(in_remote), _dptr(ptr_l), _dptr(col_l),
                                  _dptr(ptr_r), _dptr(col_r), lb, ub, dim, npp, ps, wpb, dist, C.byref(o)))
 
 
 def tune_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb, ub, dim, nodePerPE,
-                np_size, *, input_remote=None, gin_eps=None, ld_in=0, ld_out=0, row_scale_out=None, relu=False, col_block_rows=0):
+                np_size, *, input_remote=None, gin_eps=None, ld_in=0, ld_out=0, row_scale_out=None, relu=False, col_block_rows=0,
+                core_rows=0):
     """The search of the reference's bench_MGG_DSE_dist_ps.py / bench_MGG_DSE_dist_wpb.py in one call: times
-    partSize (as given, or 16 and 32 when 0) x plain / column-blocked order x warpPerBlock x interleaved_dist on this
-    input, returns ({"ps", "wpb", "dist", "col_block_rows"}, ms) of the fastest and makes later calls that leave the
+    partSize (as given, or 16 and 32 when 0) x plain / column-blocked order x without / with a dense core x warpPerBlock x
+    interleaved_dist on this input, returns ({"ps", "wpb", "dist", "col_block_rows", "core_rows"}, ms) of the fastest and makes later calls that leave the
     knobs at 0 on the same CSR tensors use it."""
     import torch
     o = _AggOpts()
@@ -351,33 +353,34 @@ def tune_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, c
     o.d_row_scale_out = row_scale_out.data_ptr() if row_scale_out is not None else None
     o.in_dtype = BF16 if input.dtype == torch.bfloat16 else F32
     o.col_block_rows = col_block_rows
+    o.core_rows = core_rows
     _pin(row_pointers_l, row_pointers_r, column_index_l, column_index_r)
     k, ms = _AggKnobs(), C.c_float()
     rem = input_remote if input_remote is not None else input
     _check(lib().mggx_sag_np_div_tune(_dptr(output), _dptr(input), _dptr(rem), _dptr(row_pointers_l), _dptr(column_index_l),
                                       _dptr(row_pointers_r), _dptr(column_index_r), lb, ub, dim, nodePerPE, np_size,
                                       C.byref(o), C.byref(k), C.byref(ms)))
-    return {"ps": k.ps, "wpb": k.wpb, "dist": k.dist, "col_block_rows": k.col_block_rows}, ms.value
+    return {"ps": k.ps, "wpb": k.wpb, "dist": k.dist, "col_block_rows": k.col_block_rows, "core_rows": k.core_rows}, ms.value
 
 
 def mgg_SAG_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb, ub, dim,
                    nodePerPE, peid, np_size, warpPerBlock, interleaved_dist, *, input_remote=None, accumulate=False,
-                   ld_in=0, ld_out=0, row_scale_out=None, relu=False, col_block_rows=0):
+                   ld_in=0, ld_out=0, row_scale_out=None, relu=False, col_block_rows=0, core_rows=0):
     """Argument order of the reference's mgg_SAG_np_div.  `input` is this rank's table; `input_remote` the
     global-id-indexed table the reference reaches with remote GETs (defaults to `input`, the single-GPU case).
     The reference adds into `output`; pass accumulate=True for that, the default overwrites."""
     flags = (AGG_ACCUMULATE if accumulate else 0) | (AGG_RELU if relu else 0)
     _agg(output, input, input_remote if input_remote is not None else input, row_pointers_l, column_index_l,
          row_pointers_r, column_index_r, lb, ub, dim, nodePerPE, np_size, warpPerBlock, interleaved_dist, flags, 0.0,
-         ld_in, ld_out, row_scale_out, col_block_rows)
+         ld_in, ld_out, row_scale_out, col_block_rows, core_rows)
 
 
 def mgg_GIN_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb, ub, dim,
                    nodePerPE, peid, np_size, warpPerBlock, interleaved_dist, eps, *, input_remote=None, ld_in=0,
-                   ld_out=0, col_block_rows=0):
+                   ld_out=0, col_block_rows=0, core_rows=0):
     _agg(output, input, input_remote if input_remote is not None else input, row_pointers_l, column_index_l,
          row_pointers_r, column_index_r, lb, ub, dim, nodePerPE, np_size, warpPerBlock, interleaved_dist, AGG_GIN,
-         float(eps), ld_in, ld_out, None, col_block_rows)
+         float(eps), ld_in, ld_out, None, col_block_rows, core_rows)
 
 
 def SAG_host(output, input, row_pointers, column_index, part_pointers, part2Node, lowbound, num_nodes, num_parts,
@@ -447,3 +450,22 @@ def gather_probe(sink, table, rows: int, ld_bytes: int, row_bytes: int, n_gather
     _check(lib().mggx_gather_probe(_dptr(sink), _dptr(table), C.c_int64(rows), C.c_size_t(ld_bytes), C.c_size_t(row_bytes),
                                    C.c_int64(n_gathers), C.c_uint(seed), C.byref(done)))
     return int(done.value)
+
+
+def core_layout(ptr: np.ndarray, col: np.ndarray, lb: int, core_rows: int, tile_cols: int = 256):
+    """The dense-core layout of a local CSR as the library builds it -> dict(core, ntiles, core_nnz, order, rank,
+    blk_off, idx, rem_ptr, rem_col)."""
+    ptr = np.ascontiguousarray(ptr, dtype=np.int32)
+    col = np.ascontiguousarray(col, dtype=np.int32)
+    rows = len(ptr) - 1
+    h = C.c_void_p()
+    sizes = (C.c_int64 * 5)()
+    _check(lib().mggx_core_layout_build(_iptr(ptr), _iptr(col), rows, lb, core_rows, tile_cols, C.byref(h), sizes))
+    core = int(sizes[0])
+    order, rank = np.zeros(core, np.int32), np.zeros(rows, np.int32)
+    blk_off, idx = np.zeros(int(sizes[1]), np.uint32), np.zeros(int(sizes[2]), np.uint16)
+    rem_ptr, rem_col = np.zeros(rows + 1, np.int32), np.zeros(int(sizes[3]), np.int32)
+    _check(lib().mggx_core_layout_fetch(h, _iptr(order), _iptr(rank), blk_off.ctypes.data_as(C.c_void_p),
+                                        idx.ctypes.data_as(C.c_void_p), _iptr(rem_ptr), _iptr(rem_col)))
+    return dict(core=core, ntiles=core // tile_cols, core_nnz=int(sizes[4]), order=order, rank=rank, blk_off=blk_off, idx=idx,
+                rem_ptr=rem_ptr, rem_col=rem_col)

@@ -280,3 +280,63 @@ def test_compact_remote_staging_order(seed):
     assert c1.tolist() == [0, 0, 0] and i1.tolist() == [7]
     with pytest.raises(host.MggxError):
         host.compact_remote(np.array([3, -1], np.int32))
+
+
+@pytest.mark.parametrize("lb,core_rows,tile", [(0, 1024, 256), (0, 1700, 256), (300, 512, 64)])
+def test_dense_core_layout(lb, core_rows, tile):
+    """The core x core block as index lists plus the remaining CSR, against numpy: ranks by degree (ties by id), every
+    core edge exactly once in the list of its (slice, tile) block at the right tile offset in edge order, padding
+    only behind the entries, everything else left in the CSR in its order."""
+    V = 4000
+    ptr, col = host.gen_rmat(12, V, 120_000, seed=4)
+    col = (col + lb).astype(np.int32)  # a share whose rows start at lb: ids are global
+    L = host.core_layout(ptr, col, lb, core_rows, tile)
+    core = L["core"]
+    assert core == core_rows // 512 * 512 and L["ntiles"] == core // tile
+    deg = np.diff(ptr)
+    order = np.argsort(-deg, kind="stable")[:core]
+    assert np.array_equal(L["order"], order)
+    rank = np.full(V, -1, np.int32)
+    rank[order] = np.arange(core)
+    assert np.array_equal(L["rank"], rank)
+    rows = np.repeat(np.arange(V), deg)
+    in_core = (rank[rows] >= 0) & (rank[col - lb] >= 0)
+    assert L["core_nnz"] == int(in_core.sum())
+    # the remainder
+    keep = ~in_core
+    assert np.array_equal(L["rem_col"], col[keep])
+    rp = np.zeros(V + 1, np.int64)
+    np.add.at(rp, rows[keep] + 1, 1)
+    assert np.array_equal(L["rem_ptr"], np.cumsum(rp))
+    # the lists
+    ntiles, off, idx = L["ntiles"], L["blk_off"].astype(np.int64), L["idx"]
+    assert len(off) == core // 64 * ntiles + 1 and len(idx) == off[-1] * 256 and np.all(np.diff(off) >= 0)
+    seen = 0
+    for i in (list(range(0, core, 37)) + [core - 1]):
+        v = order[i]
+        nb = rank[col[ptr[v]:ptr[v + 1]] - lb]
+        nb = nb[nb >= 0]
+        for t in range(ntiles):
+            want = nb[nb // tile == t] % tile
+            b0, b1 = off[(i // 64) * ntiles + t], off[(i // 64) * ntiles + t + 1]
+            got = idx[b0 * 256:b1 * 256].reshape(-1, 64, 4)[:, i % 64, :].reshape(-1)
+            assert len(want) <= len(got)
+            assert np.array_equal(got[:len(want)], want) and np.all(got[len(want):] == 0xFFFF)
+            seen += len(want)
+    assert seen > 0
+    # every block is as long as its longest list, rounded up to 4
+    cnt = np.zeros((core, ntiles), np.int64)
+    rc, cc = rank[rows[in_core]], rank[col[in_core] - lb]
+    np.add.at(cnt, (rc, cc // tile), 1)
+    width = (cnt.reshape(core // 64, 64, ntiles).max(axis=1) + 3) // 4
+    assert np.array_equal(np.diff(off), width.reshape(-1))
+
+
+def test_dense_core_layout_rejects_what_it_cannot_hold():
+    ptr, col = host.gen_rmat(10, 900, 9000, seed=1)
+    with pytest.raises(host.MggxError):
+        host.core_layout(ptr, col, 0, 400, 256)        # less than one 512-row unit
+    with pytest.raises(host.MggxError):
+        host.core_layout(ptr, col, 5, 512, 256)        # ids below lb
+    with pytest.raises(host.MggxError):
+        host.core_layout(ptr, col, 0, 512, 100)        # tile not a multiple of 64

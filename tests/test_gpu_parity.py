@@ -235,6 +235,99 @@ def test_column_blocked_order(gpu, rmat_graph, dim, block_rows, flags):
         assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "unsorted rows")
 
 
+@pytest.mark.parametrize("dim,core_rows,flags", [(16, 1024, "plain"), (44, 512, "scale"), (41, 2048, "gin"), (8, 1500, "acc_relu"),
+                                                 (64, 1024, "plain"), (5, 512, "scale")])
+def test_dense_core_from_lds(gpu, rmat_graph, dim, core_rows, flags):
+    """The dense-core path (core x core block summed from LDS tiles, the rest of the CSR on top): same sums as the
+    ordinary path and the oracle with every epilogue, with padded row strides, and together with the column-blocked
+    order of what is left."""
+    import torch
+    V, ptr, col = rmat_graph
+    x = gpu.fill_normal((V, dim), seed=191)
+    sh = share_of(ptr, col, V, 1, 0)
+    d_ptr, d_col = to_dev(ptr), to_dev(col)
+    z, zc = torch.zeros(V + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    ld = dim + 3 if dim == 5 else dim
+    d_x = torch.zeros(V, ld, device="cuda")
+    d_x[:, :dim] = to_dev(x)
+    s = gpu.fill_uniform((V,), 0.5, 2.0, seed=192)
+    base = gpu.fill_normal((V, dim), seed=193)
+
+    def run(core, blk, ps, wpb, dist):
+        out = torch.full((V, ld), 7.5, device="cuda")
+        if flags == "acc_relu":
+            out[:, :dim] = to_dev(base)
+        if flags == "gin":
+            gpu.mgg_GIN_np_div(out, d_x, d_ptr, d_col, z, zc, 0, V, dim, V, 0, ps, wpb, dist, 0.5, col_block_rows=blk, core_rows=core,
+                               ld_in=ld, ld_out=ld)
+        else:
+            gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, z, zc, 0, V, dim, V, 0, ps, wpb, dist, col_block_rows=blk, core_rows=core,
+                               accumulate=flags == "acc_relu", relu=flags == "acc_relu",
+                               row_scale_out=to_dev(s) if flags == "scale" else None, ld_in=ld, ld_out=ld)
+        gpu.sync()
+        got = out.cpu().numpy()
+        assert np.all(got[:, dim:] == 7.5)  # the padding of the output rows is not touched
+        return got[:, :dim]
+
+    kw = {}
+    if flags == "gin":
+        kw = dict(flags=orc.GIN, eps=0.5)
+    want, mag = oracle_agg(sh, x, x, dim, **kw)
+    if flags == "scale":
+        want, mag = want * s[:, None], mag * s[:, None]
+    if flags == "acc_relu":
+        want, mag = np.maximum(want + base, 0), mag + np.abs(base)
+    for blk, ps, wpb, dist in ((-1, 16, 4, 1), (-1, 4, 2, 3), (300, 32, 8, 16), (0, 0, 0, 0)):
+        got = run(core_rows, blk, ps, wpb, dist)
+        assert "core=%d" % (core_rows // 512 * 512) in gpu.last_agg_kernel()
+        assert_close_to_oracle(got, want, mag, FP32_TOL, "dense core, blk=%d ps=%d wpb=%d dist=%d" % (blk, ps, wpb, dist))
+    got = run(-1, -1, 16, 4, 1)
+    assert "core=" not in gpu.last_agg_kernel()
+    assert_close_to_oracle(got, want, mag, FP32_TOL, "without a core")
+    # closed form: all ones give the degree exactly, core or not
+    ones = torch.ones(V, ld, device="cuda")
+    out = torch.zeros(V, ld, device="cuda")
+    gpu.mgg_SAG_np_div(out, ones, d_ptr, d_col, z, zc, 0, V, dim, V, 0, 16, 4, 1, core_rows=core_rows, ld_in=ld, ld_out=ld)
+    gpu.sync()
+    assert np.array_equal(out.cpu().numpy()[:, :dim], np.repeat(np.diff(ptr).astype(np.float32)[:, None], dim, 1))
+
+
+def test_dense_core_falls_back_and_is_searched(gpu, rmat_graph):
+    """A core the graph cannot hold (fewer rows than one unit), bf16 tables and remote edges fall back to the ordinary
+    path; the search returns a setting with or without a core and later calls reuse it."""
+    import torch
+    V, ptr, col = rmat_graph
+    dim = 16
+    x = gpu.fill_normal((V, dim), seed=195)
+    sh = share_of(ptr, col, V, 1, 0)
+    want, mag = oracle_agg(sh, x, x, dim)
+    z, zc = torch.zeros(V + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    d_ptr, d_col, d_x = to_dev(ptr), to_dev(col), to_dev(x)
+    out = torch.full((V, dim), 7.5, device="cuda")
+    gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, z, zc, 0, V, dim, V, 0, 16, 4, 1, core_rows=300)
+    gpu.sync()
+    assert "core=" not in gpu.last_agg_kernel()
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "core smaller than a unit")
+    kn, ms = gpu.tune_np_div(out, d_x, d_ptr, d_col, z, zc, 0, V, dim, V, 16, core_rows=1024)
+    gpu.sync()
+    assert kn["core_rows"] == 1024 and ms > 0
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "after the search")
+    out.fill_(7.5)
+    gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, z, zc, 0, V, dim, V, 0, 0, 0, 0)
+    gpu.sync()
+    assert "core=1024" in gpu.last_agg_kernel()
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "searched setting reused")
+    # a share with remote edges: the request is ignored
+    sh2 = share_of(ptr, col, V, 2, 0)
+    got = torch.full((sh2["ub"] - sh2["lb"], dim), 7.5, device="cuda")
+    gpu.mgg_SAG_np_div(got, to_dev(x[sh2["lb"]:sh2["ub"]]), to_dev(sh2["ptr_l"]), to_dev(sh2["col_l"]), to_dev(sh2["ptr_r"]),
+                       to_dev(sh2["col_r"]), sh2["lb"], sh2["ub"], dim, sh2["npp"], 0, 16, 4, 1, input_remote=d_x, core_rows=512)
+    gpu.sync()
+    assert "core=" not in gpu.last_agg_kernel()
+    w2, m2 = oracle_agg(sh2, x[sh2["lb"]:sh2["ub"]], x, dim)
+    assert_close_to_oracle(got.cpu().numpy(), w2, m2, FP32_TOL, "share with remote edges")
+
+
 def test_column_blocked_order_with_bf16_tables(gpu, rmat_graph):
     """bf16 feature rows, fp32 partial rows and output: the blocked order must give what the plain order gives."""
     import torch
