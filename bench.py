@@ -107,6 +107,8 @@ MEASURED_TRAFFIC = {
     "gcn2_agg1": (6_481_731_891, (4, 16)),
     "gcn2_agg2_blocked": (7_519_810_150, (4, 16)),   # column blocks of 49152 ids: partial rows and their reduction included
     "gcn2_agg1_blocked": (1_746_502_963, (4, 16)),
+    "gcn2_agg2_core24576_blocked": (6_971_496_140, (4, 16)),   # dense core of 24576 rows from LDS, the rest column-blocked
+    "gcn2_agg1_core24576_blocked": (1_700_438_118, (4, 16)),
     "share_agg": (1_220_807_373, (8, 1)),
     "gin_agg": (25_550_513_561, (16, 1)),
     "big_agg": (60_511_998_361, (4, 16)),
@@ -235,7 +237,8 @@ def bench_gcn2(args, torch, host):
     dom = "agg2" if avg["agg2"] >= avg["agg1"] else "agg1"
     dom_bytes = b2 if dom == "agg2" else b1
     achieved = dom_bytes / (avg[dom] * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": "k_agg (%s, dim %d)" % (dom, out_dim if dom == "agg2" else hidden),
+    kdom = k2 if dom == "agg2" else k1
+    roofline = {"bound": "hbm", "kernel": "%sk_agg (%s, dim %d)" % ("k_core_sell + " if kdom.core > 0 else "", dom, out_dim if dom == "agg2" else hidden),
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("gcn2_" + dom, args, (k2 if dom == "agg2" else k1).blk, (k2 if dom == "agg2" else k1).core),
                 "algorithmic_bytes": dom_bytes, "avg_launch_ms": round(avg[dom], 4)}
