@@ -223,7 +223,7 @@ int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int 
         delete p;
         return rc;
     }
-    if (s.cores.size() >= 2) {  // these plans are large: keep two
+    if (s.cores.size() >= 4) {  // these plans are large (about 3 bytes per edge): keep the four the search of one graph goes through
         core_plan_free(s.cores.front());
         s.cores.erase(s.cores.begin());
     }
