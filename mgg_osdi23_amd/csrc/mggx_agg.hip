@@ -866,7 +866,8 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
 {
     Plan *plan = nullptr;
     int rc;
-    if (k.core_rows > 0 && g.nnz_r == 0 && d_col_l && o.in_dtype == MGGX_F32 && dim <= 64 && d_out && d_in_local) {
+    if (k.core_rows > 0 && ub - lb >= 1024 && g.nnz_r == 0 && g.nnz_l > 0 && d_col_l && o.in_dtype == MGGX_F32 && dim >= 1 && dim <= 64 && d_out &&
+        d_in_local) {
         CorePlan *cp = nullptr;
         rc = core_plan_get(d_ptr_l, d_col_l, ub - lb, lb, k.core_rows, &cp);
         if (rc) return rc;
