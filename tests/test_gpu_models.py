@@ -297,6 +297,17 @@ def test_full_size_whole_graph_gcn_widths(gpu):
     gpu.sync()
     assert "blocks=1 " in gpu.last_agg_kernel() + " "
     assert np.array_equal(out.cpu().numpy()[:, 0], np.diff(ptr).astype(np.float32))
+    # the dense core of this graph from LDS: the degree exactly, and sampled rows of the width-41 layer against the oracle
+    gpu.mgg_SAG_np_div(out, ones, d_ptr, d_col, zp, zc, 0, V, 16, V, 0, 16, 8, 16, core_rows=24576)
+    gpu.sync()
+    assert "core=24576" in gpu.last_agg_kernel() and "blocks=5" in gpu.last_agg_kernel()
+    assert np.array_equal(out.cpu().numpy()[:, 0], np.diff(ptr).astype(np.float32))
+    out44 = torch.full((V, 44), -1.0, device="cuda")
+    gpu.mgg_SAG_np_div(out44, d_x, d_ptr, d_col, zp, zc, 0, V, 44, V, 0, 16, 4, 16, row_scale_out=to_dev(s), ld_in=44, ld_out=44,
+                       core_rows=24576)
+    gpu.sync()
+    check_sampled_rows(gpu, out44.cpu().numpy()[:, :41], sh, x, x, 41, n_samples=300, rs_out=s)
+    assert np.all(out44.cpu().numpy()[:, 41:] == 0.0)
     acc = torch.ones(V, 16, device="cuda")  # the single-GPU SpMM entry point adds into its output
     gpu.SpMM(acc, ones, d_ptr, d_col, V, 16, 16, 8)
     gpu.sync()
