@@ -872,22 +872,37 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
         rc = core_plan_get(d_ptr_l, d_col_l, ub - lb, lb, k.core_rows, &cp);
         if (rc) return rc;
         if (!cp->unsuitable) {
-            // the core block first: out = (accumulate ? out : 0) + scale * core sums; then what is left of the CSR on top, with
-            // the caller's epilogue (its row scale applies to its own sums, the self term and the ReLU come last)
+            // The core block is bound by the LDS, the rest of the CSR by the caches: they run side by side.  The core's sums
+            // go to partial rows on a second stream; the rest of the CSR runs here with the caller's epilogue except the
+            // ReLU; then the partial rows are added (with the row scale) and the ReLU comes last.
             const long long ld_in = o.ld_in ? o.ld_in : dim, ld_out = o.ld_out ? o.ld_out : dim;
             if (ld_in < dim || ld_out < dim) return fail(MGGX_EINVAL, "aggregation: row stride smaller than dim");
-            rc = run_core(cp, d_out, static_cast<const float *>(d_in_local), dim, ld_in, ld_out, o.d_row_scale_out,
-                          (o.flags & MGGX_AGG_ACCUMULATE) ? 1 : 0);
+            State &st0 = state();
+            hipStream_t side;
+            hipEvent_t fork, join;
+            rc = core_side_stream(&side, &fork, &join);
             if (rc) return rc;
+            MGGX_HIP(hipEventRecord(fork, st0.stream));
+            MGGX_HIP(hipStreamWaitEvent(side, fork, 0));
+            rc = run_core_sums(cp, static_cast<const float *>(d_in_local), dim, ld_in, side);
+            const hipError_t er = hipEventRecord(join, side);
+            int rc2 = MGGX_OK;
             GraphInfo *gr = nullptr;
-            rc = graph_info(cp->d_rem_ptr, nullptr, ub - lb, &gr);
+            if (!rc) rc2 = graph_info(cp->d_rem_ptr, nullptr, ub - lb, &gr);
+            if (!rc && !rc2) {
+                mggx_agg_opts o2 = o;
+                o2.flags &= ~MGGX_AGG_RELU;
+                Knobs k2 = k;
+                k2.core_rows = -1;
+                if (k2.block_rows > 0 && !blocking_eligible(*gr, k2.block_rows)) k2.block_rows = -1;
+                rc2 = run_knobs(*gr, k2, d_out, d_in_local, nullptr, cp->d_rem_ptr, cp->d_rem_col, nullptr, nullptr, lb, ub, dim, o2);
+            }
+            // the caller's stream takes the side stream back in whatever happened, so no work of this call outlives it unordered
+            const hipError_t ew = er == hipSuccess ? hipStreamWaitEvent(st0.stream, join, 0) : er;
             if (rc) return rc;
-            mggx_agg_opts o2 = o;
-            o2.flags |= MGGX_AGG_ACCUMULATE;
-            Knobs k2 = k;
-            k2.core_rows = -1;
-            if (k2.block_rows > 0 && !blocking_eligible(*gr, k2.block_rows)) k2.block_rows = -1;
-            rc = run_knobs(*gr, k2, d_out, d_in_local, nullptr, cp->d_rem_ptr, cp->d_rem_col, nullptr, nullptr, lb, ub, dim, o2);
+            if (rc2) return rc2;
+            if (ew != hipSuccess) return fail(MGGX_EHIP, "aggregation: joining the side stream: %s", hipGetErrorString(ew));
+            rc = run_core_finish(cp, d_out, dim, ld_out, o.d_row_scale_out, (o.flags & MGGX_AGG_RELU) ? 1 : 0, st0.stream);
             if (rc) return rc;
             State &st = state();
             const size_t n = strlen(st.last_kernel);
@@ -962,11 +977,11 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
     int blks[2] = {-1, 0}, n_blk = 1;
     if (o.col_block_rows > 0) blks[0] = o.col_block_rows;
     else if (o.col_block_rows == 0 && mggx::blocking_eligible(*g, mggx::DEFAULT_BLOCK_ROWS)) { blks[1] = mggx::DEFAULT_BLOCK_ROWS; n_blk = 2; }
-    int cores[4] = {-1, 0, 0, 0}, n_core = 1;  // without a dense core and, where it may pay, with one of three sizes
+    int cores[5] = {-1, 0, 0, 0, 0}, n_core = 1;  // without a dense core and, where it may pay, with one of four sizes
     if (o.core_rows > 0) {
         cores[0] = o.core_rows;
     } else if (o.core_rows == 0) {
-        static const int sizes[] = {16 * 1024, 24 * 1024, 32 * 1024};
+        static const int sizes[] = {16 * 1024, 24 * 1024, 32 * 1024, 40 * 1024};
         for (int c : sizes)
             if (mggx::core_eligible(*g, dim, o.in_dtype, c)) cores[n_core++] = c;
     }

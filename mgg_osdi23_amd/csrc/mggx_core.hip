@@ -18,7 +18,8 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned short us4 __attribute__((ext_vector_type(4)));
 
 constexpr int CORE_TC = 256;    // core columns per LDS tile
-constexpr int CORE_WAVES = 8;   // slices (of 64 rows) per workgroup
+constexpr int CORE_WAVES = 4;   // slices (of 64 rows) per workgroup: as small as the aggregation's own workgroups, so the two
+                                // kernels of a call, running side by side, find room on a CU equally easily
 
 // tab[s * core + i] = elements 4 s .. 4 s + 3 of the feature row of the rank-i node (zero past dim)
 __global__ void __launch_bounds__(256) k_core_stage(v4f *__restrict__ tab, const float *__restrict__ in, const int *__restrict__ order,
@@ -85,40 +86,48 @@ __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *_
     for (int s = 0; s < N4; ++s) partial[((size_t)seg * core + r) * N4 + s] = acc[s];
 }
 
-// out[v][d] = (accumulate ? out[v][d] : 0) + scale[v] * sum over segments of the core's partial rows (0 outside the core)
-__global__ void __launch_bounds__(256) k_core_reduce(float *__restrict__ out, const float *__restrict__ partial, const int *__restrict__ rank,
-                                                     const float *__restrict__ rs, int rows, int dim, long long ld_out, int core, int n4,
-                                                     int nseg, int accumulate)
+// Adds the core block's sums to output rows that already hold the rest of the aggregation:
+// out[v][d] = act(out[v][d] + scale[v] * sum over segments of the partial rows of v).  all_rows = 0: one thread per
+// element of the core rows only (idx -> rank -> row); all_rows = 1: every row (needed when act is the ReLU).
+__global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, const float *__restrict__ partial, const int *__restrict__ rank,
+                                                     const int *__restrict__ order, const float *__restrict__ rs, int rows, int dim,
+                                                     long long ld_out, int core, int n4, int nseg, int relu, int all_rows)
 {
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (long long)rows * dim) return;
-    const int v = (int)(idx / dim), d = (int)(idx % dim);
-    const int r = rank[v];
+    if (idx >= (long long)(all_rows ? rows : core) * dim) return;
+    const int i = (int)(idx / dim), d = (int)(idx % dim);
+    const int v = all_rows ? i : order[i];
+    const int r = all_rows ? rank[i] : i;
     float sum = 0.f;
     if (r >= 0) {
         for (int seg = 0; seg < nseg; ++seg) sum += partial[(((size_t)seg * core + r) * n4 + (d >> 2)) * 4 + (d & 3)];
         if (rs) sum *= rs[v];
     }
     float *o = out + (long long)v * ld_out + d;
-    *o = accumulate ? *o + sum : sum;
+    float t = *o + sum;
+    if (relu) t = fmaxf(t, 0.f);
+    *o = t;
 }
 
 // The same, four columns per thread, where the output rows take 16-byte accesses.
-__global__ void __launch_bounds__(256) k_core_reduce4(float *__restrict__ out, const v4f *__restrict__ partial, const int *__restrict__ rank,
-                                                      const float *__restrict__ rs, int rows, int n4, long long ld_out, int core, int nseg,
-                                                      int accumulate)
+__global__ void __launch_bounds__(256) k_core_finish4(float *__restrict__ out, const v4f *__restrict__ partial, const int *__restrict__ rank,
+                                                      const int *__restrict__ order, const float *__restrict__ rs, int rows, int n4,
+                                                      long long ld_out, int core, int nseg, int relu, int all_rows)
 {
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (long long)rows * n4) return;
-    const int v = (int)(idx / n4), q = (int)(idx % n4);
-    const int r = rank[v];
+    if (idx >= (long long)(all_rows ? rows : core) * n4) return;
+    const int i = (int)(idx / n4), q = (int)(idx % n4);
+    const int v = all_rows ? i : order[i];
+    const int r = all_rows ? rank[i] : i;
     v4f sum = {0.f, 0.f, 0.f, 0.f};
     if (r >= 0) {
         for (int seg = 0; seg < nseg; ++seg) sum += partial[((size_t)seg * core + r) * n4 + q];
         if (rs) sum *= rs[v];
     }
     v4f *o = reinterpret_cast<v4f *>(out + (long long)v * ld_out + 4 * q);
-    *o = accumulate ? *o + sum : sum;
+    v4f t = *o + sum;
+    if (relu) { t.x = fmaxf(t.x, 0.f); t.y = fmaxf(t.y, 0.f); t.z = fmaxf(t.z, 0.f); t.w = fmaxf(t.w, 0.f); }
+    *o = t;
 }
 
 template <int N4>
@@ -167,6 +176,20 @@ void core_plan_free(CorePlan *p)
     forget_pointer(p->d_rem_col);
     core_plan_free_arrays(p);
     delete p;
+}
+
+int core_side_stream(hipStream_t *stream, hipEvent_t *fork, hipEvent_t *join)
+{
+    State &s = state();
+    if (!s.side_stream) {
+        MGGX_HIP(hipStreamCreateWithFlags(&s.side_stream, hipStreamNonBlocking));
+        MGGX_HIP(hipEventCreateWithFlags(&s.side_fork, hipEventDisableTiming));
+        MGGX_HIP(hipEventCreateWithFlags(&s.side_join, hipEventDisableTiming));
+    }
+    *stream = s.side_stream;
+    *fork = s.side_fork;
+    *join = s.side_join;
+    return MGGX_OK;
 }
 
 int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, CorePlan **out)
@@ -232,52 +255,68 @@ int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int 
     return MGGX_OK;
 }
 
-// The core's share of the aggregation: out = (accumulate ? out : 0) + scale * (core block sums); every row of out is written.
-int run_core(CorePlan *p, float *d_out, const float *d_in, int dim, long long ld_in, long long ld_out, const float *d_row_scale,
-             int accumulate)
+// Scratch of the dense-core path: the staged core table, then one partial row per core row and segment.
+static int core_scratch(const CorePlan *p, int n4, v4f **tab, v4f **partial)
 {
     State &s = state();
-    const int n4 = (dim + 3) / 4;
-    if (n4 < 1 || n4 > 16) return fail(MGGX_ELIMIT, "core: dim %d outside 1..64", dim);
     const size_t tab_bytes = ((size_t)p->core * n4 * sizeof(v4f) + 255) & ~(size_t)255;
     const size_t part_bytes = (size_t)p->nseg * p->core * n4 * sizeof(v4f);
     if (tab_bytes + part_bytes > s.core_ws_bytes) {
-        MGGX_HIP(hipStreamSynchronize(s.stream));
+        MGGX_HIP(hipDeviceSynchronize());  // both streams may still use the old block
         if (s.core_ws) (void)hipFree(s.core_ws);
         s.core_ws = nullptr;
         s.core_ws_bytes = 0;
         if (hipMalloc(&s.core_ws, tab_bytes + part_bytes) != hipSuccess) return fail(MGGX_ENOMEM, "core: %zu bytes of scratch", tab_bytes + part_bytes);
         s.core_ws_bytes = tab_bytes + part_bytes;
     }
-    v4f *tab = static_cast<v4f *>(s.core_ws);
-    v4f *partial = reinterpret_cast<v4f *>(static_cast<char *>(s.core_ws) + tab_bytes);
+    *tab = static_cast<v4f *>(s.core_ws);
+    *partial = reinterpret_cast<v4f *>(static_cast<char *>(s.core_ws) + tab_bytes);
+    return MGGX_OK;
+}
+
+// The core block's sums into the library's partial rows, on `stream` (reads d_in only).
+int run_core_sums(CorePlan *p, const float *d_in, int dim, long long ld_in, hipStream_t stream)
+{
+    const int n4 = (dim + 3) / 4;
+    if (n4 < 1 || n4 > 16) return fail(MGGX_ELIMIT, "core: dim %d outside 1..64", dim);
+    v4f *tab = nullptr, *partial = nullptr;
+    int rc = core_scratch(p, n4, &tab, &partial);
+    if (rc) return rc;
     {
         const long long n = (long long)p->core * n4;
-        k_core_stage<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s.stream>>>(tab, d_in, p->d_order, p->core, n4, dim, ld_in);
+        k_core_stage<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(tab, d_in, p->d_order, p->core, n4, dim, ld_in);
         MGGX_LAUNCH_CHECK("k_core_stage");
     }
-    int rc;
     switch (n4) {
-#define MGGX_CASE(N) case N: rc = launch_sell<N>(p, tab, partial, s.stream); break;
+#define MGGX_CASE(N) case N: rc = launch_sell<N>(p, tab, partial, stream); break;
         MGGX_CASE(1) MGGX_CASE(2) MGGX_CASE(3) MGGX_CASE(4) MGGX_CASE(5) MGGX_CASE(6) MGGX_CASE(7) MGGX_CASE(8)
         MGGX_CASE(9) MGGX_CASE(10) MGGX_CASE(11) MGGX_CASE(12) MGGX_CASE(13) MGGX_CASE(14) MGGX_CASE(15) MGGX_CASE(16)
 #undef MGGX_CASE
         default: rc = fail(MGGX_ELIMIT, "core: dim %d", dim);
     }
+    return rc;
+}
+
+// out += scale * (partial rows of the core), then the ReLU if asked for, on `stream`.
+int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, hipStream_t stream)
+{
+    const int n4 = (dim + 3) / 4;
+    v4f *tab = nullptr, *partial = nullptr;
+    int rc = core_scratch(p, n4, &tab, &partial);  // sized by run_core_sums already: only hands the pointers out
     if (rc) return rc;
-    {
-        if (dim % 4 == 0 && ld_out % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0) {
-            const long long n = (long long)p->rows * n4;
-            k_core_reduce4<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s.stream>>>(d_out, partial, p->d_rank, d_row_scale, p->rows, n4, ld_out,
-                                                                                           p->core, p->nseg, accumulate);
-        } else {
-            const long long n = (long long)p->rows * dim;
-            k_core_reduce<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s.stream>>>(d_out, reinterpret_cast<const float *>(partial), p->d_rank,
-                                                                                          d_row_scale, p->rows, dim, ld_out, p->core, n4, p->nseg,
-                                                                                          accumulate);
-        }
-        MGGX_LAUNCH_CHECK("k_core_reduce");
+    const int all_rows = relu ? 1 : 0;
+    const long long nrows = all_rows ? p->rows : p->core;
+    if (dim % 4 == 0 && ld_out % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0) {
+        const long long n = nrows * n4;
+        k_core_finish4<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(d_out, partial, p->d_rank, p->d_order, d_row_scale, p->rows, n4,
+                                                                                     ld_out, p->core, p->nseg, relu, all_rows);
+    } else {
+        const long long n = nrows * dim;
+        k_core_finish<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(d_out, reinterpret_cast<const float *>(partial), p->d_rank,
+                                                                                    p->d_order, d_row_scale, p->rows, dim, ld_out, p->core, n4,
+                                                                                    p->nseg, relu, all_rows);
     }
+    MGGX_LAUNCH_CHECK("k_core_finish");
     return MGGX_OK;
 }
 

@@ -102,6 +102,8 @@ struct State {
     std::list<GraphInfo> graphs;  // least recently used first; a list, so records stay where they are while others come and go
     std::vector<CorePlan *> cores;
     void *core_ws = nullptr;      // staged core table and partial rows of the dense-core path (grow-only)
+    hipStream_t side_stream = nullptr;  // the core block runs here, beside the rest of the CSR on `stream`
+    hipEvent_t side_fork = nullptr, side_join = nullptr;
     size_t core_ws_bytes = 0;
     char last_kernel[160] = "";
     int gather_addressing = 0;  // 0 = choose per call, 1 = always 64-bit addresses
@@ -126,8 +128,10 @@ void plan_free(Plan *p);
 int forget_pointer(const void *d_ptr);
 int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, CorePlan **out);
 void core_plan_free(CorePlan *p);
-int run_core(CorePlan *p, float *d_out, const float *d_in, int dim, long long ld_in, long long ld_out, const float *d_row_scale,
-             int accumulate);
+int run_core_sums(CorePlan *p, const float *d_in, int dim, long long ld_in, hipStream_t stream);
+int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, hipStream_t stream);
+// Second stream of the dense-core path (created on first use, default priority) and the two events that fork and join it.
+int core_side_stream(hipStream_t *stream, hipEvent_t *fork, hipEvent_t *join);
 
 }  // namespace mggx
 #endif

@@ -59,10 +59,12 @@ def test_gcn_two_layer_forward(gpu, pad):
     assert np.allclose(P.cpu().numpy().sum(1), 1.0, atol=1e-5)
 
 
-def test_forward_replayed_from_a_hip_graph(gpu):
+@pytest.mark.parametrize("core_rows", [-1, 1024])
+def test_forward_replayed_from_a_hip_graph(gpu, core_rows):
     """After one eager call has built the plan and sized the workspace, a forward issues kernels only (no
     allocation, no memset, no synchronisation), so it can be captured into a HIP graph.  Every replay, with eager work
-    of the library between replays, must reproduce the eager result bit for bit."""
+    of the library between replays, must reproduce the eager result bit for bit.  With a dense core the call forks a
+    second stream and joins it again: the capture takes both in."""
     import torch
     V, in_dim, hidden, out_dim = 5000, 64, 16, 40
     ptr, col = gpu.gen_rmat(13, V, 150_000, seed=9)
@@ -77,9 +79,9 @@ def test_forward_replayed_from_a_hip_graph(gpu):
 
     def forward():
         gpu.dense_forward(Y1, X, W1, V, in_dim, hidden, row_scale=s)
-        gpu.mgg_SAG_np_div(H1, Y1, d_ptr, d_col, zp, zc, 0, V, hidden, V, 0, 16, 4, 2, row_scale_out=s)
+        gpu.mgg_SAG_np_div(H1, Y1, d_ptr, d_col, zp, zc, 0, V, hidden, V, 0, 16, 4, 2, row_scale_out=s, core_rows=core_rows)
         gpu.dense_forward(Y2, H1, W2, V, hidden, out_dim, row_scale=s)
-        gpu.mgg_SAG_np_div(H2, Y2, d_ptr, d_col, zp, zc, 0, V, out_dim, V, 0, 16, 4, 2, row_scale_out=s)
+        gpu.mgg_SAG_np_div(H2, Y2, d_ptr, d_col, zp, zc, 0, V, out_dim, V, 0, 16, 4, 2, row_scale_out=s, core_rows=core_rows)
         gpu.softmax_forward(P, H2, V, out_dim)
 
     side = torch.cuda.Stream()
