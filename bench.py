@@ -107,8 +107,8 @@ MEASURED_TRAFFIC = {
     "gcn2_agg1": (6_481_731_891, (4, 16)),
     "gcn2_agg2_blocked": (7_519_810_150, (4, 16)),   # column blocks of 49152 ids: partial rows and their reduction included
     "gcn2_agg1_blocked": (1_746_502_963, (4, 16)),
-    "gcn2_agg2_core24576_blocked": (6_971_496_140, (4, 16)),   # dense core of 24576 rows from LDS, the rest column-blocked
-    "gcn2_agg1_core24576_blocked": (1_700_438_118, (4, 16)),
+    "gcn2_agg2_core40960_blocked": (5_319_550_054, (4, 8)),   # dense core of 40960 rows from LDS beside the column-blocked rest
+    "gcn2_agg1_core40960_blocked": (1_498_319_462, (4, 8)),
     "share_agg": (1_220_807_373, (8, 1)),
     "gin_agg": (25_550_513_561, (16, 1)),
     "big_agg": (60_511_998_361, (4, 16)),

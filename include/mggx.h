@@ -226,7 +226,8 @@ typedef struct mggx_agg_knobs {
  * of 256 core columns at a time staged with whole-line reads, one lane per core row walking an index list -- and the
  * rest of the CSR runs as usual on top.  Pays on graphs whose high-degree rows hold most edges among themselves; its
  * plan is built on the host (the CSR is copied back once), so by rule it is off and mggx_sag_np_div_tune turns it on
- * where it measures faster.  Same result up to summation order.
+ * where it measures faster.  The core block runs on a second stream of the library's, forked from and joined to the
+ * caller's stream by events inside the call (LDS-bound work beside cache-bound work).  Same result up to summation order.
  * The partition plan of (d_ptr_l, d_ptr_r, d_col_r, rows, ps) -- and d_col_l for the column-blocked order -- is built on first use and
  * cached by pointer identity: the CSR arrays must not be rewritten in place or freed
  * while cached (mggx_forget() drops what hangs on one array, mggx_release_cached() everything). */
