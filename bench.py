@@ -111,6 +111,7 @@ MEASURED_TRAFFIC = {
     "gcn2_agg1_core40960_blocked": (1_498_319_462, (4, 8)),
     "share_agg": (1_220_807_373, (8, 1)),
     "gin_agg": (25_550_513_561, (16, 1)),
+    "gin_agg_core40960": (19_723_389_132, (8, 4)),   # dense core of 40960 rows from LDS beside the rest
     "big_agg": (60_511_998_361, (4, 16)),
 }
 
@@ -380,7 +381,7 @@ def bench_share(args, torch, host):
                                "fp32 dim %d, %s" % (V, R, nnz, len(lc), len(rc), dim, kn)},
         "roofline": {"bound": "hbm", "kernel": "k_agg (dim 16, local+remote)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     **load_traffic("share_agg", args, kn.blk), "algorithmic_bytes": nbytes, "avg_launch_ms": round(ms, 4)},
+                     **load_traffic("share_agg", args, kn.blk, kn.core), "algorithmic_bytes": nbytes, "avg_launch_ms": round(ms, 4)},
         "cpu_baseline": cpu, "detail": detail,
     }
 
@@ -510,8 +511,8 @@ def bench_gin(args, torch, host):
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[2]: 5-layer GIN forward, RMAT V=%d nnz=%d, 100->64->47, 2-layer MLP per layer (%s), eps=0, "
                                "%s" % (V, nnz, "two kernels" if args.unfused_mlp else "one fused kernel", kn)},
-        "roofline": {"bound": "hbm", "kernel": "k_agg (GIN, dim 64)", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("gin_agg", args, kn.blk),
+        "roofline": {"bound": "hbm", "kernel": "%sk_agg (GIN, dim 64)" % ("k_core_sell + " if kn.core > 0 else ""), "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("gin_agg", args, kn.blk, kn.core),
                      "algorithmic_bytes": nbytes, "avg_launch_ms": round(agg_ms, 4)},
         "cpu_baseline": cpu, "parity": parity,
         "detail": {"stage_ms": {k: round(v, 4) for k, v in avg.items()}, "mlp_total_ms": round(mlp_ms, 4)},
@@ -604,7 +605,7 @@ def bench_big(args, torch, host):
                                "bf16 dim %d, fp32 accumulate, then %dx%d bf16 MFMA update; %s"
                                % (k, V, R, nnz, len(lc), len(rc), dim, dim, dim, kn)},
         "roofline": {"bound": "hbm", "kernel": "k_agg (bf16 dim 128, local+remote)", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("big_agg", args, kn.blk),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("big_agg", args, kn.blk, kn.core),
                      "algorithmic_bytes": nbytes, "avg_launch_ms": round(avg["agg"], 4)},
         "cpu_baseline": cpu, "parity": parity,
         "detail": {"stage_ms": {k2: round(v, 4) for k2, v in avg.items()},
