@@ -2,7 +2,7 @@
 // share of the range partition, device upload.  The programs keep the command
 // line and the log lines of the reference's mains (src/mgg_np_div_kernel.cu:47-57,
 // 103,192,195) so the reference's bench/analysis scripts can drive and parse them:
-//   <prog> beg.bin csr.bin weight.bin nGPU partSize warpPerBlock dist dim hidden out [--pe K] [--iters N] [--validate]
+//   <prog> beg.bin csr.bin weight.bin nGPU partSize warpPerBlock dist dim hidden out [--pe K] [--iters N] [--validate] [--tune]
 // nGPU is the number of ranks the graph is partitioned for; the one real GPU
 // runs rank --pe (default 0) with the other ranks' rows staged in its memory.
 #ifndef MGG_HARNESS_COMMON_H
@@ -28,13 +28,14 @@ struct HarnessArgs {
     int num_GPUs, partSize, warpPerBlock, interleaved_dist, dim, hiddenSize, outdim;
     int pe = 0, iters = 100;
     bool validate = false;
+    bool tune = false;  // search warpPerBlock / interleaved_dist / partition order on this input first (mgg_tune_np_div)
 };
 
 inline bool parse_args(int argc, char *argv[], HarnessArgs &a)
 {
     if (argc < 11) {
         printf("Usage: %s beg.bin csr.bin weight.bin num_GPUs partSize warpPerblock interleaved_dist dim hidden out "
-               "[--pe K] [--iters N] [--validate]\n", argv[0]);
+               "[--pe K] [--iters N] [--validate] [--tune]\n", argv[0]);
         return false;
     }
     a.beg_file = argv[1];
@@ -51,6 +52,7 @@ inline bool parse_args(int argc, char *argv[], HarnessArgs &a)
         if (!strcmp(argv[i], "--pe") && i + 1 < argc) a.pe = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--iters") && i + 1 < argc) a.iters = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--validate")) a.validate = true;
+        else if (!strcmp(argv[i], "--tune")) a.tune = true;
     }
     if (a.num_GPUs < 1 || a.pe < 0 || a.pe >= a.num_GPUs || a.iters < 1) {
         printf("bad --pe/--iters/num_GPUs\n");

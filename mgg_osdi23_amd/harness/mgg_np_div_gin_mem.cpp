@@ -54,12 +54,23 @@ int main(int argc, char *argv[])
         mggx_free(d_gptr); mggx_free(d_gcol); mggx_free(d_Xg); mggx_free(d_Hg);
     }
 
+    // --tune: search the knobs on this input once (all five aggregations have the same shape), then leave them to the library
+    int wpb = a.warpPerBlock, dist = a.interleaved_dist;
+    if (a.tune) {
+        dense_beg_new_forward(dp1);
+        mgg_stage_remote(d_stage[0]);
+        const mggx_agg_knobs k = mgg_tune_np_div(dsp_out, den_out, s.d_row_ptr_l, s.d_col_ind_l, s.d_row_ptr_r, s.d_col_ind_r, s.lb, s.ub,
+                                                 hidden, npp, a.partSize);
+        printf("tuned: width %d wpb %d dist %d blocks %d core %d\n", hidden, k.wpb, k.dist, k.col_block_rows, k.core_rows);
+        wpb = dist = 0;
+    }
+
     auto forward = [&](bool with_softmax) {
         dense_beg_new_forward(dp1);
         for (int l = 0; l < layers; ++l) {
             mgg_stage_remote(d_stage[l]);
             mgg_GIN_np_div(dsp_out, den_out, s.d_row_ptr_l, s.d_col_ind_l, s.d_row_ptr_r, s.d_col_ind_r, s.lb, s.ub, hidden, npp,
-                           a.pe, a.partSize, a.warpPerBlock, a.interleaved_dist, eps);
+                           a.pe, a.partSize, wpb, dist, eps);
             dense_hidden_new_forward(dpl[l]);
         }
         if (with_softmax) softmax_new_forward(smx);

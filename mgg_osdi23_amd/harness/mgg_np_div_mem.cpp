@@ -50,15 +50,32 @@ int main(int argc, char *argv[])
         mggx_free(d_gptr); mggx_free(d_gcol); mggx_free(d_Xg); mggx_free(d_H1g);
     }
 
+    // --tune: the design-space search of the reference's bench_MGG_DSE_*.py on this input, once per aggregation width;
+    // the aggregations below then leave warpPerBlock and interleaved_dist to the library, which reuses what it found.
+    int wpb = a.warpPerBlock, dist = a.interleaved_dist;
+    if (a.tune) {
+        dense_beg_new_forward(dp1);
+        mgg_stage_remote(d_Y1g);
+        const mggx_agg_knobs k1 = mgg_tune_np_div(d_buff_2, dp1->d_out, s.d_row_ptr_l, s.d_col_ind_l, s.d_row_ptr_r, s.d_col_ind_r, s.lb,
+                                                  s.ub, hidden, npp, a.partSize);
+        dense_hidden_new_forward(dp2);
+        mgg_stage_remote(d_Y2g);
+        const mggx_agg_knobs k2 = mgg_tune_np_div(d_buff_1, dp2->d_out, s.d_row_ptr_l, s.d_col_ind_l, s.d_row_ptr_r, s.d_col_ind_r, s.lb,
+                                                  s.ub, outdim, npp, a.partSize);
+        printf("tuned: width %d wpb %d dist %d blocks %d core %d; width %d wpb %d dist %d blocks %d core %d\n", hidden, k1.wpb, k1.dist,
+               k1.col_block_rows, k1.core_rows, outdim, k2.wpb, k2.dist, k2.col_block_rows, k2.core_rows);
+        wpb = dist = 0;
+    }
+
     auto forward = [&]() {
         dense_beg_new_forward(dp1);
         mgg_stage_remote(d_Y1g);
         mgg_SAG_np_div(d_buff_2, dp1->d_out, s.d_row_ptr_l, s.d_col_ind_l, s.d_row_ptr_r, s.d_col_ind_r, s.lb, s.ub, hidden,
-                       npp, a.pe, a.partSize, a.warpPerBlock, a.interleaved_dist);
+                       npp, a.pe, a.partSize, wpb, dist);
         dense_hidden_new_forward(dp2);
         mgg_stage_remote(d_Y2g);
         mgg_SAG_np_div(d_buff_1, dp2->d_out, s.d_row_ptr_l, s.d_col_ind_l, s.d_row_ptr_r, s.d_col_ind_r, s.lb, s.ub, outdim,
-                       npp, a.pe, a.partSize, a.warpPerBlock, a.interleaved_dist);
+                       npp, a.pe, a.partSize, wpb, dist);
         if (!a.validate) softmax_new_forward(smx2);
     };
 

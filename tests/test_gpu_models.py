@@ -211,6 +211,18 @@ def test_harness_programs_validate_and_log(gpu, graph_files, prog, dims, ngpu, p
     assert m and float(m.group(1)) > 0
 
 
+@pytest.mark.parametrize("prog,dims", [("mgg_np_div_mem", (6, 8, 4)), ("mgg_np_div_gin_mem", (20, 16, 7))])
+def test_harness_programs_with_the_search(gpu, graph_files, prog, dims):
+    """--tune: the knob search runs on the program's own buffers first; the all-ones validation still passes."""
+    exe = os.path.join(BIN, prog)
+    files, ptr, col = graph_files
+    cmd = [exe] + files + ["1", "16", "4", "2"] + [str(x) for x in dims] + ["--iters", "3", "--validate", "--tune"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert re.search(r"tuned: width \d+ wpb \d+ dist \d+", r.stdout), r.stdout
+    assert re.search(r"Validation on PE-\{0\}, status: True", r.stdout), r.stdout
+
+
 def test_cpp_layer_entry_points(gpu, tmp_path):
     """mgg_api_check calls every function and class of include/mgg/*.h from C++ (loaders, split_CSR, build_part,
     mgg_SAG_np_div, mgg_GIN_np_div, SAG_host, SAG_host_fused_interleaved, sparse_*/dense_*/softmax_* layer objects, the
