@@ -982,7 +982,7 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
     if (o.core_rows > 0) {
         cores[0] = o.core_rows;
     } else if (o.core_rows == 0) {
-        static const int sizes[] = {24 * 1024, 32 * 1024, 40 * 1024, 64 * 1024};
+        static const int sizes[] = {32 * 1024, 40 * 1024, 48 * 1024, 64 * 1024};
         for (int c : sizes)
             if (mggx::core_eligible(*g, dim, o.in_dtype, c)) cores[n_core++] = c;
     }
