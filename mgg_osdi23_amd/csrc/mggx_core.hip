@@ -74,8 +74,17 @@ __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *_
             for (int j = 0; j < 4; ++j) {
                 const int c = cur[j];
                 const v4f *q = tile + (c < TC ? c : TC);
+                // at most eight LDS reads in flight per entry: wide rows otherwise cost a wavefront a hundred registers, and
+                // this kernel shares each SIMD's register file with the aggregation running beside it
+                constexpr int H = N4 > 8 ? (N4 + 1) / 2 : N4;
 #pragma unroll
-                for (int s = 0; s < N4; ++s) acc[s] += q[s * TP];
+                for (int s = 0; s < H; ++s) acc[s] += q[s * TP];
+                if constexpr (H < N4) {
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int s = H; s < N4; ++s) acc[s] += q[s * TP];
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             cur = nxt;
             ++pos;
