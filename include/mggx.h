@@ -19,7 +19,9 @@
  *   - feature tables are row-major [rows x ld] with ld >= dim (the reference
  *     always has ld == dim).
  *   - all device work is issued on the stream set by mggx_set_stream()
- *     (default: the null stream) and is asynchronous unless stated.
+ *     (default: the null stream) and is asynchronous unless stated; the dense-core path of the aggregation also uses a
+ *     second stream of the library's own, forked from and joined to that stream by events inside the call, so every
+ *     call is still ordered on the caller's stream as a whole.
  *   - after a first call of the same shape (which builds the cached plan and grows the library's scratch), the
  *     compute entry points only launch kernels -- no allocation, memset or synchronisation -- and may be captured
  *     into a HIP graph; the scratch block is reallocated when a later call needs more, so warm up the largest call
