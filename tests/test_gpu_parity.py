@@ -292,6 +292,39 @@ def test_dense_core_from_lds(gpu, rmat_graph, dim, core_rows, flags):
     assert np.array_equal(out.cpu().numpy()[:, :dim], np.repeat(np.diff(ptr).astype(np.float32)[:, None], dim, 1))
 
 
+def test_dense_core_on_a_share_with_unsorted_rows_and_parallel_edges(gpu, rmat_graph):
+    """The local half of a share whose rows start at lb > 0, neighbor lists shuffled and some edges listed twice: the
+    core's index lists carry order and multiplicity as they come, so the sums still match the oracle."""
+    import torch
+    V, ptr, col = rmat_graph
+    dim = 24
+    sh = share_of(ptr, col, V, 2, 1)
+    lb, ub = sh["lb"], sh["ub"]
+    R = ub - lb
+    rng = np.random.default_rng(3)
+    lp, lc = sh["ptr_l"], sh["col_l"]
+    new_ptr, new_col = [0], []
+    for v in range(R):
+        nb = lc[lp[v]:lp[v + 1]].copy()
+        if len(nb) and v % 5 == 0:
+            nb = np.concatenate([nb, nb[: 1 + len(nb) // 3]])  # parallel edges
+        rng.shuffle(nb)
+        new_col.append(nb)
+        new_ptr.append(new_ptr[-1] + len(nb))
+    p2 = np.array(new_ptr, np.int32)
+    c2 = np.concatenate(new_col).astype(np.int32)
+    x = gpu.fill_normal((V, dim), seed=197)
+    xl = np.ascontiguousarray(x[lb:ub])
+    sh2 = dict(npp=sh["npp"], lb=lb, ub=ub, ptr_l=p2, col_l=c2, ptr_r=np.zeros(R + 1, np.int32), col_r=np.zeros(0, np.int32))
+    want, mag = oracle_agg(sh2, xl, x, dim)
+    z, zc = torch.zeros(R + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    out = torch.full((R, dim), 7.5, device="cuda")
+    gpu.mgg_SAG_np_div(out, to_dev(xl), to_dev(p2), to_dev(c2), z, zc, lb, ub, dim, sh["npp"], 1, 16, 4, 2, core_rows=1024)
+    gpu.sync()
+    assert "core=1024" in gpu.last_agg_kernel()
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "dense core, lb > 0, shuffled rows, parallel edges")
+
+
 def test_dense_core_falls_back_and_is_searched(gpu, rmat_graph):
     """A core the graph cannot hold (fewer rows than one unit), bf16 tables and remote edges fall back to the ordinary
     path; the search returns a setting with or without a core and later calls reuse it."""
