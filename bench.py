@@ -107,6 +107,8 @@ MEASURED_TRAFFIC = {
     "gcn2_agg1": (6_481_731_891, (4, 16)),
     "gcn2_agg2_blocked": (7_519_810_150, (4, 16)),   # column blocks of 49152 ids: partial rows and their reduction included
     "gcn2_agg1_blocked": (1_746_502_963, (4, 16)),
+    "gcn2_agg2_core32768_blocked": (6_186_012_569, (4, 16)),
+    "gcn2_agg1_core32768_blocked": (1_653_667_737, (4, 16)),
     "gcn2_agg2_core40960_blocked": (5_319_550_054, (4, 8)),   # dense core of 40960 rows from LDS beside the column-blocked rest
     "gcn2_agg1_core40960_blocked": (1_498_319_462, (4, 8)),
     "share_agg": (1_220_807_373, (8, 1)),
