@@ -883,9 +883,11 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
             hipEvent_t fork, join;
             rc = core_side_stream(&side, &fork, &join);
             if (rc) return rc;
+            rc = run_core_stage(cp, static_cast<const float *>(d_in_local), dim, ld_in, st0.stream);
+            if (rc) return rc;
             MGGX_HIP(hipEventRecord(fork, st0.stream));
             MGGX_HIP(hipStreamWaitEvent(side, fork, 0));
-            rc = run_core_sums(cp, static_cast<const float *>(d_in_local), dim, ld_in, side);
+            rc = run_core_sums(cp, dim, side);
             const hipError_t er = hipEventRecord(join, side);
             int rc2 = MGGX_OK;
             GraphInfo *gr = nullptr;

@@ -283,19 +283,29 @@ static int core_scratch(const CorePlan *p, int n4, v4f **tab, v4f **partial)
     return MGGX_OK;
 }
 
-// The core block's sums into the library's partial rows, on `stream` (reads d_in only).
-int run_core_sums(CorePlan *p, const float *d_in, int dim, long long ld_in, hipStream_t stream)
+// The core's feature rows into the slice-major table, on `stream` (a few microseconds on an idle chip, ten times that
+// beside the aggregation: the caller runs it before the two big kernels start).
+int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, hipStream_t stream)
 {
     const int n4 = (dim + 3) / 4;
     if (n4 < 1 || n4 > 16) return fail(MGGX_ELIMIT, "core: dim %d outside 1..64", dim);
     v4f *tab = nullptr, *partial = nullptr;
     int rc = core_scratch(p, n4, &tab, &partial);
     if (rc) return rc;
-    {
-        const long long n = (long long)p->core * n4;
-        k_core_stage<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(tab, d_in, p->d_order, p->core, n4, dim, ld_in);
-        MGGX_LAUNCH_CHECK("k_core_stage");
-    }
+    const long long n = (long long)p->core * n4;
+    k_core_stage<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(tab, d_in, p->d_order, p->core, n4, dim, ld_in);
+    MGGX_LAUNCH_CHECK("k_core_stage");
+    return MGGX_OK;
+}
+
+// The core block's sums from the staged table into the library's partial rows, on `stream`.
+int run_core_sums(CorePlan *p, int dim, hipStream_t stream)
+{
+    const int n4 = (dim + 3) / 4;
+    if (n4 < 1 || n4 > 16) return fail(MGGX_ELIMIT, "core: dim %d outside 1..64", dim);
+    v4f *tab = nullptr, *partial = nullptr;
+    int rc = core_scratch(p, n4, &tab, &partial);
+    if (rc) return rc;
     switch (n4) {
 #define MGGX_CASE(N) case N: rc = launch_sell<N>(p, tab, partial, stream); break;
         MGGX_CASE(1) MGGX_CASE(2) MGGX_CASE(3) MGGX_CASE(4) MGGX_CASE(5) MGGX_CASE(6) MGGX_CASE(7) MGGX_CASE(8)

@@ -128,7 +128,8 @@ void plan_free(Plan *p);
 int forget_pointer(const void *d_ptr);
 int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, CorePlan **out);
 void core_plan_free(CorePlan *p);
-int run_core_sums(CorePlan *p, const float *d_in, int dim, long long ld_in, hipStream_t stream);
+int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, hipStream_t stream);
+int run_core_sums(CorePlan *p, int dim, hipStream_t stream);
 int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, hipStream_t stream);
 // Second stream of the dense-core path (created on first use, default priority) and the two events that fork and join it.
 int core_side_stream(hipStream_t *stream, hipEvent_t *fork, hipEvent_t *join);
