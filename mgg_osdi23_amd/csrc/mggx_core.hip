@@ -4,8 +4,9 @@
 // block does not need one gather per edge from the caches: the feature rows of 256 core columns at a time are staged
 // in LDS with whole-line reads, and every lane owns one core row and adds the LDS rows its index list names
 // (sliced-ELL lists over degree-ranked rows, so the 64 lanes of a wavefront have lists of similar length).  The
-// block's sums go to partial rows per column segment; k_core_reduce adds them to the output, and the rest of the CSR
-// runs through the ordinary aggregation, accumulating on top.
+// block's sums go to partial rows per column segment.  This kernel is bound by the LDS, the ordinary aggregation of
+// the rest of the CSR by the caches, so the caller runs the two side by side on two streams; k_core_finish then adds
+// the partial rows to the output the aggregation wrote.
 #include <algorithm>
 #include <new>
 

@@ -628,6 +628,7 @@ int graph_info(const int *d_ptr_l, const int *d_ptr_r, int rows, GraphInfo **out
 // Drops every cached plan and graph record keyed by this device address (an array about to be freed or rewritten).
 int forget_pointer(const void *d_ptr)
 {
+    if (!d_ptr) return MGGX_OK;  // NULL is what absent arrays are keyed by: nothing hangs on it
     State &s = state();
     bool synced = false;
     for (size_t i = 0; i < s.plans.size();) {
