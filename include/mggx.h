@@ -262,6 +262,20 @@ int mggx_sag_parts(float *d_out, const float *d_in, const int *d_row_ptr, const 
                    const int *d_part_ptr, const int *d_part2node,
                    int lowbound, int num_nodes, int num_parts, int ps, int dim, int wpb, int dist);
 
+/* mggx_sag_parts for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same result bit for bit, but the
+ * call allocates nothing and caches nothing: the partition descriptors, the per-row offsets and the carry buffer of the
+ * call live in a fixed array of MGGX_STATIC_SCRATCH_BYTES that is part of the library's device code (every GPU the
+ * library runs on holds its own copy until the process ends; its address is looked up once per device, in mggx_init or
+ * on the first call there).  A call whose 16 bytes per partition + 4 bytes per row + carry buffer (two partial rows per
+ * workgroup) do not fit returns MGGX_ELIMIT.  The call only launches kernels on the library's stream -- no allocation,
+ * no memset, no copy to the host, no synchronisation.  Every call on a GPU uses that GPU's one array: calls that may
+ * overlap on one GPU (two streams, two host threads) race; issue them on one stream. */
+#define MGGX_STATIC_SCRATCH_BYTES (64u << 20)
+int mggx_sag_parts_static(float *d_out, const float *d_in, const int *d_row_ptr, const int *d_col,
+                          const int *d_part_ptr, const int *d_part2node,
+                          int lowbound, int num_nodes, int num_parts, int ps, int dim, int wpb, int dist);
+
 /* SpMM_cuda_kernel via sparse_beg_forward / sparse_hidden_forward
  * (include/gnn_kernel.cuh:9-71, gnn_layer.cuh:86-161): whole graph on one GPU,
  * out[v,:] += sum_{u in N(v)} in[u,:].  ps = 0 / wpb = 0 let the library choose; the rounds per wavefront and the

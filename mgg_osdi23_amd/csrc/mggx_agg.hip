@@ -23,6 +23,13 @@
 
 #include "mggx_dev.h"
 
+// Device memory of mggx_sag_parts_static, the entry point that allocates nothing: the partition descriptors, the first
+// descriptor of each row and the carry buffer of one call.  Every GPU the library runs on holds its own copy, at its
+// own address, until the process ends; every call on a GPU shares that GPU's copy.  In host code this name is only a
+// handle for hipGetSymbolAddress: static_scratch_ptr() below asks the runtime for the array's device address once per
+// device, and that address is what kernels and host calls get.
+static __device__ __align__(256) unsigned char scratch[MGGX_STATIC_SCRATCH_BYTES];
+
 namespace mggx {
 namespace {
 
@@ -52,6 +59,7 @@ struct AggArgs {
     long long ld_in, ld_out;
     int num_parts;
     int nnz_l, nnz_r;
+    const int *nnz_l_dev;     // when set: the local edge count is read from here (a caller that may not copy it to the host)
     int lb, dim, ps, dist, cpad;
     int parts_per_wg;
     unsigned flags;
@@ -349,7 +357,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
         const long long start = (long long)((unsigned)d.x & 0x7FFFFFFFu);
         const int *col = remote ? a.col_r : a.col_l;
         const int idbase = remote ? 0 : a.lb;
-        const int nnz_side = remote ? a.nnz_r : a.nnz_l;
+        const int nnz_side = remote ? a.nnz_r : (a.nnz_l_dev ? *a.nnz_l_dev : a.nnz_l);
         if constexpr (BUF) g.cbase = (remote ? a.delta_r : a.delta_l) + cofs;
         else g.base = static_cast<const char *>(remote ? a.in_r : a.in_l) + cofs;
 
@@ -649,8 +657,16 @@ int launch_agg(int lpr, dim3 grid, dim3 block, size_t lds_bytes, hipStream_t str
     return MGGX_OK;
 }
 
+// `fixed` != NULL: the carry buffer comes from that block (the static scratch) instead of the library's grow-only
+// workspace, and a call that does not fit is refused; nothing is allocated on that path.
+struct FixedScratch {
+    unsigned char *ptr;
+    size_t bytes;
+    const int *nnz_l_dev;
+};
+
 int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, const int *d_col_l, const int *d_col_r,
-            int lb, int dim, int wpb, int dist, const mggx_agg_opts &o)
+            int lb, int dim, int wpb, int dist, const mggx_agg_opts &o, const FixedScratch *fixed = nullptr)
 {
     State &st = state();
     if (dim < 1 || dim > 256) return fail(MGGX_ELIMIT, "aggregation: dim %d outside 1..256", dim);
@@ -717,6 +733,7 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     a.num_parts = plan->num_parts;
     a.nnz_l = (int)plan->nnz_l;
     a.nnz_r = (int)plan->nnz_r;
+    a.nnz_l_dev = fixed ? fixed->nnz_l_dev : nullptr;
     a.lb = lb;
     a.dim = dim;
     a.ps = plan->ps;
@@ -760,7 +777,15 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         void *ws = nullptr;
         const size_t carry_bytes = (hdr_pad + (size_t)num_wg * 2 * cpad * sizeof(float) + 255) & ~(size_t)255;
         const size_t part_bytes = blocked ? (size_t)plan->rows * ldp * sizeof(float) : 0;
-        int rc = workspace(carry_bytes + part_bytes, &ws);
+        int rc = MGGX_OK;
+        if (fixed) {
+            if (blocked || carry_bytes > fixed->bytes)
+                return fail(MGGX_ELIMIT, "aggregation: %zu bytes of carry buffer for %lld workgroups exceed the static scratch (%zu left)",
+                            carry_bytes, num_wg, fixed->bytes);
+            ws = fixed->ptr;
+        } else {
+            rc = workspace(carry_bytes + part_bytes, &ws);
+        }
         if (rc) return rc;
         a.c_hdr = static_cast<int2 *>(ws);
         a.c_val = reinterpret_cast<float *>(static_cast<char *>(ws) + hdr_pad);
@@ -1040,6 +1065,67 @@ MGGX_EXPORT int mggx_sag_parts(float *d_out, const float *d_in, const int *d_row
     mggx_agg_opts o{};
     o.flags = MGGX_AGG_ACCUMULATE;
     return mggx::run_agg(plan, d_out, d_in, nullptr, d_col, nullptr, lowbound, dim, wpb, dist, o);
+}
+
+namespace mggx {
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+unsigned char *g_scratch_ptr[MAX_DEVICES];  // device address of `scratch` on each device, once asked for
+}  // namespace
+
+// Address of this device's copy of the static scratch array (asked for once per device, with that device current).
+int static_scratch_ptr(unsigned char **out)
+{
+    int dev = -1;
+    MGGX_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return fail(MGGX_ELIMIT, "static scratch: device index %d", dev);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return fail(MGGX_EHIP, "static scratch: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = static_cast<unsigned char *>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return MGGX_OK;
+}
+
+}  // namespace mggx
+
+MGGX_EXPORT int mggx_sag_parts_static(float *d_out, const float *d_in, const int *d_row_ptr, const int *d_col,
+                                      const int *d_part_ptr, const int *d_part2node, int lowbound, int num_nodes,
+                                      int num_parts, int ps, int dim, int wpb, int dist)
+{
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    if (!d_row_ptr || !d_part_ptr || !d_part2node || num_nodes < 0 || num_parts < 0 || ps < 1)
+        return fail(MGGX_EINVAL, "sag_parts_static: bad argument");
+    if (num_nodes == 0 || num_parts == 0) return MGGX_OK;  // out += nothing
+    unsigned char *base = nullptr;
+    rc = mggx::static_scratch_ptr(&base);
+    if (rc) return rc;
+    // layout of the scratch: descriptors | first descriptor of each row | carry buffer (sized by run_agg)
+    const auto pad = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    const size_t desc_bytes = pad(sizeof(int4) * (size_t)num_parts), off_bytes = pad(sizeof(int) * ((size_t)num_nodes + 1));
+    if (desc_bytes + off_bytes >= (size_t)MGGX_STATIC_SCRATCH_BYTES)
+        return fail(MGGX_ELIMIT, "sag_parts_static: %d partitions over %d rows need %zu bytes of descriptors; the static scratch holds %zu",
+                    num_parts, num_nodes, desc_bytes + off_bytes, (size_t)MGGX_STATIC_SCRATCH_BYTES);
+    mggx::Plan plan;  // lives for this call only; its arrays are views into the scratch
+    plan.d_ptr_l = d_row_ptr;
+    plan.d_part_ptr = d_part_ptr;
+    plan.d_part2node = d_part2node;
+    plan.rows = plan.real_rows = num_nodes;
+    plan.ps = ps;
+    plan.num_parts = num_parts;
+    plan.d_desc = reinterpret_cast<int4 *>(base);
+    plan.d_off = reinterpret_cast<int *>(base + desc_bytes);
+    plan.nnz_l = 1;  // "has local edges"; the kernels read the count itself from d_row_ptr[num_nodes]
+    rc = mggx::explicit_desc_fill(d_row_ptr, d_part_ptr, d_part2node, num_nodes, num_parts, ps, plan.d_desc, plan.d_off);
+    if (rc) return rc;
+    const mggx::FixedScratch fx{base + desc_bytes + off_bytes, (size_t)MGGX_STATIC_SCRATCH_BYTES - desc_bytes - off_bytes, d_row_ptr + num_nodes};
+    mggx_agg_opts o{};
+    o.flags = MGGX_AGG_ACCUMULATE;
+    return mggx::run_agg(&plan, d_out, d_in, nullptr, d_col, nullptr, lowbound, dim, wpb, dist, o, &fx);
 }
 
 MGGX_EXPORT int mggx_spmm(float *d_out, const float *d_in, const int *d_row_ptr, const int *d_col, int num_nodes,

@@ -124,6 +124,10 @@ int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, i
 int graph_info(const int *d_ptr_l, const int *d_ptr_r, int rows, GraphInfo **out);
 int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows,
                       int num_parts, int ps, Plan **out);
+int explicit_desc_fill(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows, int num_parts, int ps,
+                       int4 *d_desc, int *d_off);
+// Device address of the static scratch array of mggx_sag_parts_static on the current device.
+int static_scratch_ptr(unsigned char **out);
 void plan_free(Plan *p);
 int forget_pointer(const void *d_ptr);
 int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, CorePlan **out);

@@ -459,6 +459,19 @@ int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int row
     return MGGX_OK;
 }
 
+// Descriptors and row offsets of explicit partition arrays into caller-provided device arrays (two kernels on the
+// library's stream, nothing else).
+int explicit_desc_fill(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows, int num_parts, int ps,
+                       int4 *d_desc, int *d_off)
+{
+    State &s = state();
+    k_off_from_parts<<<(rows + 1 + 255) / 256, 256, 0, s.stream>>>(d_part2node, num_parts, rows, d_off);
+    if (num_parts > 0)
+        k_desc_from_parts<<<(num_parts + 255) / 256, 256, 0, s.stream>>>(d_row_ptr, d_part_ptr, d_part2node, num_parts, ps, d_desc);
+    if (hipGetLastError() != hipSuccess) return fail(MGGX_EHIP, "plan: explicit descriptor kernel launch failed");
+    return MGGX_OK;
+}
+
 int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows, int num_parts,
                       int ps, Plan **out)
 {
@@ -484,14 +497,8 @@ int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_
             rc = fail(MGGX_ENOMEM, "plan: explicit arrays");
             break;
         }
-        k_off_from_parts<<<(rows + 1 + 255) / 256, 256, 0, s.stream>>>(d_part2node, num_parts, rows, p->d_off);
-        if (num_parts > 0)
-            k_desc_from_parts<<<(num_parts + 255) / 256, 256, 0, s.stream>>>(d_row_ptr, d_part_ptr, d_part2node, num_parts,
-                                                                            ps, p->d_desc);
-        if (hipGetLastError() != hipSuccess) {
-            rc = fail(MGGX_EHIP, "plan: explicit descriptor kernel launch failed");
-            break;
-        }
+        rc = explicit_desc_fill(d_row_ptr, d_part_ptr, d_part2node, rows, num_parts, ps, p->d_desc, p->d_off);
+        if (rc) break;
         int end = 0;
         if (rows > 0 && (hipStreamSynchronize(s.stream) != hipSuccess ||
                          hipMemcpy(&end, d_row_ptr + rows, sizeof(int), hipMemcpyDeviceToHost) != hipSuccess)) {

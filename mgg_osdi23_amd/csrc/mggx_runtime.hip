@@ -67,7 +67,8 @@ MGGX_EXPORT int mggx_init(int device)
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(MGGX_EHIP, "init: device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
     state().device = device;
-    return MGGX_OK;
+    unsigned char *scratch_addr = nullptr;  // set-up of the allocation-free entry point: look its array up on this device now
+    return mggx::static_scratch_ptr(&scratch_addr);
 }
 
 MGGX_EXPORT int mggx_device_name(char *buf, size_t len)

@@ -54,7 +54,7 @@ EXPORTS = [
     "mggx_timer_create", "mggx_timer_start", "mggx_timer_stop", "mggx_timer_elapsed_ms", "mggx_timer_destroy",
     "mggx_release_cached", "mggx_forget", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_core_layout_build", "mggx_core_layout_fetch", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
-    "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_compact_remote_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_mlp2_xw", "mggx_spmm",
+    "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_compact_remote_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_sag_parts_static", "mggx_mlp2_xw", "mggx_spmm",
     "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_gather_probe", "mggx_gather_rows", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
 ]
 
@@ -389,6 +389,14 @@ def SAG_host(output, input, row_pointers, column_index, part_pointers, part2Node
     _check(lib().mggx_sag_parts(_dptr(output), _dptr(input), _dptr(row_pointers), _dptr(column_index),
                                 _dptr(part_pointers), _dptr(part2Node), lowbound, num_nodes, num_parts, partSize, dim,
                                 warpPerBlock, interleaved_dist))
+
+
+def SAG_host_static(output, input, row_pointers, column_index, part_pointers, part2Node, lowbound, num_nodes, num_parts,
+                    partSize, dim, dimWorker, warpPerBlock, interleaved_dist=1):
+    """SAG_host through the entry point that allocates nothing (fixed device scratch, nothing cached)."""
+    _check(lib().mggx_sag_parts_static(_dptr(output), _dptr(input), _dptr(row_pointers), _dptr(column_index),
+                                       _dptr(part_pointers), _dptr(part2Node), lowbound, num_nodes, num_parts, partSize, dim,
+                                       warpPerBlock, interleaved_dist))
 
 
 def SpMM(output, input, row_pointers, column_index, num_nodes, dim, partSize, warpPerBlock):

@@ -1,0 +1,54 @@
+"""The aggregation entry point that allocates nothing (mggx_sag_parts_static) against mggx_sag_parts, through the C ABI."""
+import numpy as np
+import pytest
+
+from oracle import orc
+from tests.util import FP32_TOL, assert_close_to_oracle, share_of, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(gpu, V, scale, draws, seed, dim, ps, wpb, dist):
+    ptr, col = gpu.gen_rmat(scale, V, draws, seed=seed)
+    sh = share_of(ptr, col, V, 2, 1)
+    R = sh["ub"] - sh["lb"]
+    x = gpu.fill_normal((V, dim), seed=seed + 1)
+    xl = np.ascontiguousarray(x[sh["lb"]:sh["ub"]])
+    pp, p2n, _ = orc.build_part(sh["ptr_l"], R, ps)
+    base = gpu.fill_normal((R, dim), seed=seed + 2)
+    args = (to_dev(xl), to_dev(sh["ptr_l"]), to_dev(sh["col_l"]), to_dev(pp), to_dev(p2n), sh["lb"], R, len(p2n), ps, dim, 32, wpb, dist)
+    want_dev = to_dev(base)
+    gpu.SAG_host(want_dev, *args)
+    got_dev = to_dev(base)
+    gpu.SAG_host_static(got_dev, *args)
+    gpu.sync()
+    got, want = got_dev.cpu().numpy(), want_dev.cpu().numpy()
+    # same kernels, same order of summation: bit for bit
+    assert np.array_equal(got, want), "static entry point differs from mggx_sag_parts (V=%d dim=%d)" % (V, dim)
+    # and both against the oracle
+    ref = orc.sag_parts(xl, sh["col_l"], pp, p2n, sh["lb"], dim, base.copy())
+    only_local = dict(sh, ptr_r=np.zeros(R + 1, np.int32), col_r=np.zeros(0, np.int32))
+    rows = np.arange(R, dtype=np.int32)
+    mag = orc.sag_np_div_rows(rows, xl, x, only_local["ptr_l"], only_local["col_l"], only_local["ptr_r"], only_local["col_r"],
+                              sh["lb"], sh["ub"], dim, sh["npp"], abs_sum=True)
+    assert_close_to_oracle(got, ref, mag + np.abs(base), FP32_TOL, "static explicit parts")
+
+
+def test_static_entry_point_matches_sag_parts_twice(gpu):
+    """Two calls in a row through the one static array, the second smaller (what the first left behind must not leak in)."""
+    _case(gpu, 40_000, 16, 1_200_000, 3, 16, 16, 4, 2)
+    _case(gpu, 3_000, 12, 40_000, 5, 16, 16, 4, 2)
+    # other row widths and knobs, again larger then smaller
+    _case(gpu, 20_000, 15, 600_000, 7, 41, 8, 8, 1)
+    _case(gpu, 500, 9, 3_000, 9, 64, 3, 2, 3)
+
+
+def test_static_entry_point_rejects_what_does_not_fit(gpu):
+    import torch
+    z = torch.zeros(4, dtype=torch.int32, device="cuda")
+    f = torch.zeros(16, device="cuda")
+    with pytest.raises(gpu.MggxError, match="static scratch"):
+        gpu.SAG_host_static(f, f, z, z, z, z, 0, 1 << 20, 1 << 23, 16, 16, 32, 4, 1)  # 128 MiB of descriptors
+    # nothing to do: fine
+    gpu.SAG_host_static(f, f, z, z, z, z, 0, 0, 0, 16, 16, 32, 4, 1)
+    gpu.sync()
