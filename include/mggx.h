@@ -24,8 +24,10 @@
  *     call is still ordered on the caller's stream as a whole.
  *   - after a first call of the same shape (which builds the cached plan and grows the library's scratch), the
  *     compute entry points only launch kernels -- no allocation, memset or synchronisation -- and may be captured
- *     into a HIP graph; the scratch block is reallocated when a later call needs more, so warm up the largest call
- *     before capturing.  mggx_sag_np_div_tune, the *_device preparation calls and first calls synchronise.
+ *     into a HIP graph.  What a capture uses (plans, scratch blocks) is never freed or evicted before
+ *     mggx_release_cached(); a call that would have to build a plan or grow the scratch while the stream is capturing
+ *     returns MGGX_EINVAL instead (run it once outside the capture first).  mggx_sag_np_div_tune, the *_device
+ *     preparation calls and first calls synchronise.
  *   - one host thread per device at a time; the library keeps per-process
  *     state (stream, workspace, plan cache) without locks, as MGG runs one
  *     host thread per GPU.
@@ -79,12 +81,31 @@ int mggx_timer_start(void *timer);
 int mggx_timer_stop(void *timer);
 int mggx_timer_elapsed_ms(void *timer, float *ms); /* synchronises on the stop event */
 int mggx_timer_destroy(void *timer);
-/* Frees the workspace and every cached plan. */
+/* Frees the workspace and every cached plan (also what captured graphs may still point at: destroy those first). */
 int mggx_release_cached(void);
 /* Drops what the library remembers about the CSR array at this device address (cached partition plans, search
  * results): call it before freeing or rewriting an index array that aggregation calls have seen, when the memory is
- * not released through mggx_free (which does this itself) -- an allocator may hand the same address out again. */
+ * not released through mggx_free (which does this itself) -- an allocator may hand the same address out again.
+ * A caller that forgets to is still safe: cached records are found by address, but before every use a small kernel on
+ * the call's stream compares a fingerprint of the arrays (their last entries -- the edge counts -- and up to 2048
+ * entries of each at a fixed stride) with the one taken when the record was made.  On a mismatch every kernel of that
+ * call returns at once (the output is left as it was, nothing is read through stale indices), and the next library
+ * call on this thread, mggx_sync() included, drops the record and returns MGGX_EINVAL; calling again then works on the
+ * arrays as they are.  The check is a sample: an edit that keeps every row count and misses every sampled entry is not
+ * seen -- mggx_forget() stays the rule for in-place edits.  mggx_set_plan_check(0) turns the checks off. */
 int mggx_forget(const void *d_ptr);
+int mggx_set_plan_check(int on);
+
+/* What the library holds and what its set-up has cost so far (host clock, milliseconds, since the process started). */
+typedef struct mggx_cache_stats_t {
+    int64_t plans, plan_bytes;             /* cached partition plans (descriptors, row offsets) and their device bytes */
+    int64_t core_plans, core_plan_bytes;   /* dense-core plans (ranking, index lists, remaining CSR) */
+    int64_t workspace_bytes;               /* carry buffer and per-block partial rows */
+    int64_t core_scratch_bytes;            /* staged core table and per-segment partial rows */
+    int64_t retired_bytes;                 /* outgrown blocks kept because a captured graph may point at them */
+    double plan_build_ms, core_plan_build_ms, search_ms;  /* search_ms excludes the plan builds inside the search */
+} mggx_cache_stats_t;
+int mggx_cache_stats(mggx_cache_stats_t *out);
 
 /* ---- host-side graph preparation (CPU; replaces the host code of the path) ---- */
 

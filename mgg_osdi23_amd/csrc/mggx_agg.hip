@@ -18,6 +18,7 @@
 //   workgroups a row that crosses workgroups leaves two partial rows in a
 //              carry buffer; a small second kernel sums them in a fixed order
 // No atomics anywhere; the summation order depends only on (ps, wpb, dist, dim).
+#include <chrono>
 #include <cstring>
 #include <type_traits>
 
@@ -54,6 +55,7 @@ struct AggArgs {
     const int4 *desc;
     const int *off;
     const float *rs_out;
+    const int *ok;  // when set: *ok == 0 means the plan is stale (the CSR arrays changed) and every kernel returns at once
     int2 *c_hdr;   // [2 * workgroups]: head, tail
     float *c_val;  // [2 * workgroups][cpad]
     long long ld_in, ld_out;
@@ -280,6 +282,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     // (-5 % at width 16).  With fewer slots adjacent wavefronts share those lines and the hint costs 1-3 %.
     constexpr bool STREAM = S >= 16;
     extern __shared__ float lds[];
+    if (a.ok && *a.ok == 0) return;
 
     const int lane = lane_id();
     const int wave = (int)(threadIdx.x >> 6);
@@ -553,6 +556,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
 // wavefront and several components per lane.
 __global__ void __launch_bounds__(256) k_agg_fixup(const AggArgs a, int num_wg, int comp_lanes)
 {
+    if (a.ok && *a.ok == 0) return;
     const int lane = lane_id();
     const int group = 64 / comp_lanes;
     const long long b = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * group + lane / comp_lanes;
@@ -582,6 +586,7 @@ __global__ void __launch_bounds__(256) k_agg_fixup(const AggArgs a, int num_wg, 
 // Rows with no neighbor at all: the sum is zero.
 __global__ void __launch_bounds__(256) k_agg_empty_rows(const AggArgs a, const int *__restrict__ rows, int n_rows)
 {
+    if (a.ok && *a.ok == 0) return;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (long long)n_rows * a.dim) return;
     const int r = rows[idx / a.dim];
@@ -592,6 +597,7 @@ __global__ void __launch_bounds__(256) k_agg_empty_rows(const AggArgs a, const i
 // Column-blocked plans: out[v] = epilogue(sum over blocks c of P[c * rows + v]), blocks summed in order.
 __global__ void __launch_bounds__(256) k_agg_block_reduce(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp)
 {
+    if (a.ok && *a.ok == 0) return;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (long long)rows * a.dim) return;
     const int v = (int)(idx / a.dim), d = (int)(idx % a.dim);
@@ -604,6 +610,7 @@ __global__ void __launch_bounds__(256) k_agg_block_reduce(const AggArgs a, const
 // other tables (row scale, accumulation and ReLU only).
 __global__ void __launch_bounds__(256) k_agg_block_reduce4(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp)
 {
+    if (a.ok && *a.ok == 0) return;
     const int q = a.dim >> 2;  // float4 per row
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (long long)rows * q) return;
@@ -666,7 +673,7 @@ struct FixedScratch {
 };
 
 int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, const int *d_col_l, const int *d_col_r,
-            int lb, int dim, int wpb, int dist, const mggx_agg_opts &o, const FixedScratch *fixed = nullptr)
+            int lb, int dim, int wpb, int dist, const mggx_agg_opts &o, const int *ok, const FixedScratch *fixed = nullptr)
 {
     State &st = state();
     if (dim < 1 || dim > 256) return fail(MGGX_ELIMIT, "aggregation: dim %d outside 1..256", dim);
@@ -728,6 +735,7 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     a.desc = plan->d_desc;
     a.off = plan->d_off;
     a.rs_out = blocked ? nullptr : o.d_row_scale_out;
+    a.ok = ok;
     a.ld_in = ld_in;
     a.ld_out = blocked ? ldp : ld_out;
     a.num_parts = plan->num_parts;
@@ -887,8 +895,9 @@ Knobs resolve_knobs(const GraphInfo &g, int dim, int dtype, int ps, int wpb, int
     return k;
 }
 
+// `ok`: the verdict word of the call's content check (NULL = no gate); every kernel launched below is gated on it.
 int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in_local, const void *d_in_remote, const int *d_ptr_l,
-              const int *d_col_l, const int *d_ptr_r, const int *d_col_r, int lb, int ub, int dim, const mggx_agg_opts &o)
+              const int *d_col_l, const int *d_ptr_r, const int *d_col_r, int lb, int ub, int dim, const mggx_agg_opts &o, const int *ok)
 {
     Plan *plan = nullptr;
     int rc;
@@ -908,29 +917,29 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
             hipEvent_t fork, join;
             rc = core_side_stream(&side, &fork, &join);
             if (rc) return rc;
-            rc = run_core_stage(cp, static_cast<const float *>(d_in_local), dim, ld_in, st0.stream);
+            rc = run_core_stage(cp, static_cast<const float *>(d_in_local), dim, ld_in, ok, st0.stream);
             if (rc) return rc;
             MGGX_HIP(hipEventRecord(fork, st0.stream));
             MGGX_HIP(hipStreamWaitEvent(side, fork, 0));
-            rc = run_core_sums(cp, dim, side);
+            rc = run_core_sums(cp, dim, ok, side);
             const hipError_t er = hipEventRecord(join, side);
             int rc2 = MGGX_OK;
             GraphInfo *gr = nullptr;
-            if (!rc) rc2 = graph_info(cp->d_rem_ptr, nullptr, ub - lb, &gr);
+            if (!rc) rc2 = graph_info(cp->d_rem_ptr, nullptr, cp->d_rem_col, nullptr, ub - lb, true, &gr);
             if (!rc && !rc2) {
                 mggx_agg_opts o2 = o;
                 o2.flags &= ~MGGX_AGG_RELU;
                 Knobs k2 = k;
                 k2.core_rows = -1;
                 if (k2.block_rows > 0 && !blocking_eligible(*gr, k2.block_rows)) k2.block_rows = -1;
-                rc2 = run_knobs(*gr, k2, d_out, d_in_local, nullptr, cp->d_rem_ptr, cp->d_rem_col, nullptr, nullptr, lb, ub, dim, o2);
+                rc2 = run_knobs(*gr, k2, d_out, d_in_local, nullptr, cp->d_rem_ptr, cp->d_rem_col, nullptr, nullptr, lb, ub, dim, o2, ok);
             }
             // the caller's stream takes the side stream back in whatever happened, so no work of this call outlives it unordered
             const hipError_t ew = er == hipSuccess ? hipStreamWaitEvent(st0.stream, join, 0) : er;
             if (rc) return rc;
             if (rc2) return rc2;
             if (ew != hipSuccess) return fail(MGGX_EHIP, "aggregation: joining the side stream: %s", hipGetErrorString(ew));
-            rc = run_core_finish(cp, d_out, dim, ld_out, o.d_row_scale_out, (o.flags & MGGX_AGG_RELU) ? 1 : 0, st0.stream);
+            rc = run_core_finish(cp, d_out, dim, ld_out, o.d_row_scale_out, (o.flags & MGGX_AGG_RELU) ? 1 : 0, ok, st0.stream);
             if (rc) return rc;
             State &st = state();
             const size_t n = strlen(st.last_kernel);
@@ -947,7 +956,7 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
         rc = plan_get(d_ptr_l, d_ptr_r, d_col_r, ub - lb, k.ps, &plan);
         if (rc) return rc;
     }
-    return run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, k.wpb, k.dist, o);
+    return run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, k.wpb, k.dist, o, ok);
 }
 
 int check_np_div_args(const char *who, const int *d_ptr_l, int lb, int ub, int nodes_per_pe, int &ps, int block_rows, int core_rows)
@@ -974,11 +983,16 @@ MGGX_EXPORT int mggx_sag_np_div(float *d_out, const void *d_in_local, const void
     if (opts) o = *opts;
     rc = mggx::check_np_div_args("sag_np_div", d_ptr_l, lb, ub, nodes_per_pe, ps, o.col_block_rows, o.core_rows);
     if (rc) return rc;
+    rc = mggx::stale_poll();
+    if (rc) return rc;
     mggx::GraphInfo *g = nullptr;
-    rc = mggx::graph_info(d_ptr_l, d_ptr_r, ub - lb, &g);
+    rc = mggx::graph_info(d_ptr_l, d_ptr_r, d_col_l, d_col_r, ub - lb, false, &g);
+    if (rc) return rc;
+    const int *ok = nullptr;
+    rc = mggx::guard_check(g->guard, &ok);
     if (rc) return rc;
     const mggx::Knobs k = mggx::resolve_knobs(*g, dim, o.in_dtype, ps, wpb, dist, o.col_block_rows, o.core_rows);
-    return mggx::run_knobs(*g, k, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o);
+    return mggx::run_knobs(*g, k, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o, ok);
 }
 
 MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const void *d_in_remote, const int *d_ptr_l,
@@ -992,10 +1006,18 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
     rc = mggx::check_np_div_args("sag_np_div_tune", d_ptr_l, lb, ub, nodes_per_pe, ps, o.col_block_rows, o.core_rows);
     if (rc) return rc;
     if (o.flags & MGGX_AGG_ACCUMULATE) return fail(MGGX_EINVAL, "sag_np_div_tune: repeated runs would accumulate; clear MGGX_AGG_ACCUMULATE");
+    rc = mggx::stale_poll();
+    if (rc) return rc;
+    if (mggx::capturing()) return fail(MGGX_EINVAL, "sag_np_div_tune: not inside a stream capture");
     mggx::GraphInfo *g = nullptr;
-    rc = mggx::graph_info(d_ptr_l, d_ptr_r, ub - lb, &g);
+    rc = mggx::graph_info(d_ptr_l, d_ptr_r, d_col_l, d_col_r, ub - lb, false, &g);
+    if (rc) return rc;
+    const int *ok = nullptr;
+    rc = mggx::guard_check(g->guard, &ok);  // one check for the whole search
     if (rc) return rc;
     mggx::State &st = mggx::state();
+    const auto search_t0 = std::chrono::steady_clock::now();
+    const double build_ms0 = st.plan_build_ms + st.core_plan_build_ms;
     hipEvent_t e0, e1;
     MGGX_HIP(hipEventCreate(&e0));
     MGGX_HIP(hipEventCreate(&e1));
@@ -1016,7 +1038,7 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
     static const int wpbs[] = {8, 4, 16}, dists[] = {1, 2, 4, 8, 16};
     float best = -1.f;
     mggx::Knobs bk{pss[0], 8, 1, blks[0], cores[0]};
-    rc = mggx::run_knobs(*g, bk, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o);  // warm-up
+    rc = mggx::run_knobs(*g, bk, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o, ok);  // warm-up
     for (int ci = 0; ci < n_core && !rc; ++ci)
     for (int pi = 0; pi < n_ps && !rc; ++pi)
         for (int bi = 0; bi < n_blk && !rc; ++bi)
@@ -1026,7 +1048,7 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
                     float ms_min = -1.f;
                     for (int rep = 0; rep < 3 && !rc; ++rep) {
                         hipError_t e = hipEventRecord(e0, st.stream);
-                        rc = mggx::run_knobs(*g, k, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o);
+                        rc = mggx::run_knobs(*g, k, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o, ok);
                         if (e == hipSuccess) e = hipEventRecord(e1, st.stream);
                         if (e == hipSuccess) e = hipEventSynchronize(e1);
                         float ms = 0.f;
@@ -1040,8 +1062,12 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
     (void)hipEventDestroy(e1);
     if (rc) return rc;
     // leave the winner's result in d_out and remember it
-    rc = mggx::run_knobs(*g, bk, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o);
+    rc = mggx::run_knobs(*g, bk, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o, ok);
     if (rc) return rc;
+    MGGX_HIP(hipStreamSynchronize(st.stream));
+    // the search's own time: what the plan builds inside it took is accounted for separately
+    st.search_ms += std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - search_t0).count() -
+                    (st.plan_build_ms + st.core_plan_build_ms - build_ms0);
     bool found = false;
     for (mggx::GraphInfo::Tuned &t : g->tuned)
         if (t.dim == dim && t.dtype == o.in_dtype) { t.ps = bk.ps; t.wpb = bk.wpb; t.dist = bk.dist; t.block_rows = bk.block_rows; t.core_rows = bk.core_rows; found = true; }
@@ -1060,11 +1086,16 @@ MGGX_EXPORT int mggx_sag_parts(float *d_out, const float *d_in, const int *d_row
     if (!d_row_ptr || !d_part_ptr || !d_part2node || num_nodes < 0 || num_parts < 0 || ps < 1)
         return fail(MGGX_EINVAL, "sag_parts: bad argument");
     mggx::Plan *plan = nullptr;
+    rc = mggx::stale_poll();
+    if (rc) return rc;
     rc = mggx::plan_get_explicit(d_row_ptr, d_part_ptr, d_part2node, num_nodes, num_parts, ps, &plan);
+    if (rc) return rc;
+    const int *ok = nullptr;
+    rc = mggx::guard_check(plan->guard, &ok);
     if (rc) return rc;
     mggx_agg_opts o{};
     o.flags = MGGX_AGG_ACCUMULATE;
-    return mggx::run_agg(plan, d_out, d_in, nullptr, d_col, nullptr, lowbound, dim, wpb, dist, o);
+    return mggx::run_agg(plan, d_out, d_in, nullptr, d_col, nullptr, lowbound, dim, wpb, dist, o, ok);
 }
 
 namespace mggx {
@@ -1125,7 +1156,7 @@ MGGX_EXPORT int mggx_sag_parts_static(float *d_out, const float *d_in, const int
     const mggx::FixedScratch fx{base + desc_bytes + off_bytes, (size_t)MGGX_STATIC_SCRATCH_BYTES - desc_bytes - off_bytes, d_row_ptr + num_nodes};
     mggx_agg_opts o{};
     o.flags = MGGX_AGG_ACCUMULATE;
-    return mggx::run_agg(&plan, d_out, d_in, nullptr, d_col, nullptr, lowbound, dim, wpb, dist, o, &fx);
+    return mggx::run_agg(&plan, d_out, d_in, nullptr, d_col, nullptr, lowbound, dim, wpb, dist, o, nullptr, &fx);
 }
 
 MGGX_EXPORT int mggx_spmm(float *d_out, const float *d_in, const int *d_row_ptr, const int *d_col, int num_nodes,
@@ -1136,10 +1167,15 @@ MGGX_EXPORT int mggx_spmm(float *d_out, const float *d_in, const int *d_row_ptr,
     if (!d_row_ptr || num_nodes < 0 || ps < 0) return fail(MGGX_EINVAL, "spmm: bad argument");
     mggx_agg_opts o{};
     o.flags = MGGX_AGG_ACCUMULATE;
+    rc = mggx::stale_poll();
+    if (rc) return rc;
     mggx::GraphInfo *g = nullptr;
-    rc = mggx::graph_info(d_row_ptr, nullptr, num_nodes, &g);
+    rc = mggx::graph_info(d_row_ptr, nullptr, d_col, nullptr, num_nodes, false, &g);
+    if (rc) return rc;
+    const int *ok = nullptr;
+    rc = mggx::guard_check(g->guard, &ok);
     if (rc) return rc;
     // the whole graph on one GPU: the same knob rules (and column-blocked order for long rows) as mggx_sag_np_div
     mggx::Knobs k = mggx::resolve_knobs(*g, dim, MGGX_F32, ps, wpb, 0, 0, 0);
-    return mggx::run_knobs(*g, k, d_out, d_in, nullptr, d_row_ptr, d_col, nullptr, nullptr, 0, num_nodes, dim, o);
+    return mggx::run_knobs(*g, k, d_out, d_in, nullptr, d_row_ptr, d_col, nullptr, nullptr, 0, num_nodes, dim, o, ok);
 }

@@ -38,6 +38,23 @@ static constexpr unsigned DESC_FIRST = 0x40000000u;  // first partition of its r
 static constexpr unsigned DESC_LAST = 0x80000000u;   // last partition of its row
 static constexpr unsigned DESC_LEN_MASK = 0x3FFFFFFFu;
 
+// Content check of the caller's CSR arrays behind a cached record.  The records are found by device address, and an
+// address says nothing about what is stored there now (arrays rewritten in place, memory freed through another allocator
+// and handed out again).  When a record is made, a small kernel stores a fingerprint of the arrays (their last entries --
+// the edge counts -- and up to 2048 entries of each at a fixed stride); before every later use the same kernel takes the
+// fingerprint again on the call's stream and writes the verdict to *d_ok.  Every kernel of the call reads that word
+// first and returns at once when it is 0, so a stale plan never produces sums or touches memory through stale indices;
+// the mismatch is also written to a host-visible flag, which the next library call reports as MGGX_EINVAL after
+// dropping the record.
+struct Guard {
+    const int *arr[4] = {nullptr, nullptr, nullptr, nullptr};
+    long long len[4] = {0, 0, 0, 0};
+    unsigned long long *d_fp = nullptr;  // device: [0] fingerprint, [1] verdict word (as int) -- one 16-byte allocation
+    int id = 0;                          // reported through the host flag on a mismatch
+    bool armed = false;
+    const int *ok() const { return reinterpret_cast<const int *>(d_fp + 1); }
+};
+
 struct Plan {
     // cache key
     const int *d_ptr_l = nullptr;
@@ -64,6 +81,9 @@ struct Plan {
     int block_lb = 0;          // id of the first row of block 0 (part of the cache key)
     int blocks = 1;
     bool unsuitable = false;   // blocked plan asked for, but the rows are not sorted by neighbor id
+    bool pinned = false;       // used inside a stream capture: a captured graph holds its device addresses, never evicted
+    size_t bytes = 0;          // device memory held
+    Guard guard;               // explicit-partition plans only (the others are guarded through their GraphInfo)
 };
 
 // Dense-core plan of a local-only CSR (layout: CoreLayout in mggx_internal.h), built on the host and kept on the device.
@@ -80,13 +100,20 @@ struct CorePlan {
     unsigned short *d_idx = nullptr;
     int *d_rem_ptr = nullptr, *d_rem_col = nullptr;
     bool unsuitable = false;  // no core of whole units fits, or the ids do not allow it
+    bool pinned = false;      // used inside a stream capture: never evicted
+    size_t bytes = 0;         // device memory held
 };
 
 // What is known about a CSR the aggregation has been called with (keyed by pointer identity).
 struct GraphInfo {
     const int *d_ptr_l = nullptr;
     const int *d_ptr_r = nullptr;
+    const int *d_col_l = nullptr;
+    const int *d_col_r = nullptr;
     int rows = 0;
+    bool internal = false;  // arrays owned by the library (the remainder CSR of a dense-core plan): no content check
+    bool pinned = false;    // used inside a stream capture: never evicted
+    Guard guard;
     int64_t nnz_l = 0, nnz_r = 0;
     // knobs measured best by mggx_sag_np_div_tune for a row width and element type; used where a call passes 0
     struct Tuned { int dim, dtype, ps, wpb, dist, block_rows, core_rows; };
@@ -105,8 +132,18 @@ struct State {
     hipStream_t side_stream = nullptr;  // the core block runs here, beside the rest of the CSR on `stream`
     hipEvent_t side_fork = nullptr, side_join = nullptr;
     size_t core_ws_bytes = 0;
-    char last_kernel[160] = "";
+    char last_kernel[224] = "";
     int gather_addressing = 0;  // 0 = choose per call, 1 = always 64-bit addresses
+    // content checks of cached records (Guard)
+    int plan_check = 1;            // 0: checks off (the caller vouches for its arrays)
+    volatile int *h_stale = nullptr;  // pinned host word the check kernel writes a record id to on a mismatch
+    int next_guard_id = 1;
+    // blocks a captured graph may still point at: kept until mggx_release_cached instead of being freed on growth
+    bool ws_captured = false, core_ws_captured = false;
+    std::vector<void *> retired;
+    size_t retired_bytes = 0;
+    // host-clock time spent on set-up so far (mggx_cache_stats)
+    double plan_build_ms = 0.0, core_plan_build_ms = 0.0, search_ms = 0.0;
 };
 
 State &state();
@@ -118,10 +155,19 @@ int workspace(size_t bytes, void **p);
 // total is also copied to *total_host when non-NULL (synchronises).
 int exclusive_scan_i32(const int *d_in, int *d_out, int n, long long *total_host);
 
+// True while the library's stream is being captured into a HIP graph.
+bool capturing();
+// Content checks (see Guard).  guard_arm stores the fingerprint of a new record; guard_check takes it again on the stream
+// and returns the device word the call's kernels are gated on (NULL when checks are off); stale_poll reports a mismatch
+// an earlier check found (MGGX_EINVAL, after dropping the record) -- called on entry of every compute call and by mggx_sync.
+int guard_arm(Guard &g);
+int guard_check(Guard &g, const int **d_ok);
+void guard_free(Guard &g);
+int stale_poll();
 int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int rows, int ps, Plan **out);
 // Column-blocked plan of a local-only CSR; (*out)->unsuitable is set when the rows are not sorted by neighbor id.
 int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int ps, int block_rows, Plan **out);
-int graph_info(const int *d_ptr_l, const int *d_ptr_r, int rows, GraphInfo **out);
+int graph_info(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_l, const int *d_col_r, int rows, bool internal, GraphInfo **out);
 int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows,
                       int num_parts, int ps, Plan **out);
 int explicit_desc_fill(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows, int num_parts, int ps,
@@ -132,9 +178,10 @@ void plan_free(Plan *p);
 int forget_pointer(const void *d_ptr);
 int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, CorePlan **out);
 void core_plan_free(CorePlan *p);
-int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, hipStream_t stream);
-int run_core_sums(CorePlan *p, int dim, hipStream_t stream);
-int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, hipStream_t stream);
+// `ok`: the word the call's kernels are gated on (NULL = no gate), see Guard.
+int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, const int *ok, hipStream_t stream);
+int run_core_sums(CorePlan *p, int dim, const int *ok, hipStream_t stream);
+int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, const int *ok, hipStream_t stream);
 // Second stream of the dense-core path (created on first use, default priority) and the two events that fork and join it.
 int core_side_stream(hipStream_t *stream, hipEvent_t *fork, hipEvent_t *join);
 

@@ -339,11 +339,15 @@ MGGX_EXPORT int mggx_mtx_read(const char *path, int *num_rows, int *num_entries,
 // 1-based "row col [value]" lines) or a 0-based "src dst" list.  Output: <prefix>_beg_pos.bin / _csr.bin /
 // _weight.bin in the layout mggx_graph_read expects; edges are grouped by source with a stable counting sort (file
 // order is kept inside a row), weights are 1.
-MGGX_EXPORT int mggx_edgelist_to_bin(const char *path, int is_mtx, const char *out_prefix, int *num_nodes, int64_t *num_edges)
+static int edgelist_to_bin_impl(const char *path, int is_mtx, const char *out_prefix, int *num_nodes, int64_t *num_edges)
 {
     if (!path || !out_prefix) return fail(MGGX_EINVAL, "edgelist_to_bin: NULL argument");
     FILE *f = fopen(path, "r");
     if (!f) return fail(MGGX_EIO, "edgelist_to_bin: cannot open %s", path);
+    struct Closer {  // closes the file on every way out, a thrown bad_alloc included
+        FILE *f;
+        ~Closer() { fclose(f); }
+    } closer{f};
     std::vector<int> src, dst;
     long long declared_rows = 0;
     char line[512];
@@ -353,31 +357,31 @@ MGGX_EXPORT int mggx_edgelist_to_bin(const char *path, int is_mtx, const char *o
         if (size_line_pending) {
             long long m = 0, n = 0, l = 0;
             if (sscanf(line, "%lld %lld %lld", &m, &n, &l) < 2) {
-                fclose(f);
                 return fail(MGGX_EFORMAT, "edgelist_to_bin: bad size line in %s", path);
             }
             declared_rows = std::max(m, n);
+            if (declared_rows < 0 || declared_rows > std::numeric_limits<int>::max() - 1) {  // node ids are int32
+                return fail(MGGX_ELIMIT, "edgelist_to_bin: %lld nodes declared in %s exceed int32 ids", declared_rows, path);
+            }
             size_line_pending = false;
             continue;
         }
         long long a = 0, b = 0;
         if (sscanf(line, "%lld %lld", &a, &b) != 2) {
-            fclose(f);
             return fail(MGGX_EFORMAT, "edgelist_to_bin: malformed line in %s: %.40s", path, line);
         }
         if (is_mtx) { --a; --b; }
         if (a < 0 || b < 0 || a > std::numeric_limits<int>::max() - 1 || b > std::numeric_limits<int>::max() - 1) {
-            fclose(f);
             return fail(MGGX_EFORMAT, "edgelist_to_bin: node id out of range in %s", path);
         }
         src.push_back((int)a);
         dst.push_back((int)b);
     }
-    fclose(f);
     if (src.empty()) return fail(MGGX_EFORMAT, "edgelist_to_bin: no edges in %s", path);
     if (src.size() > (size_t)std::numeric_limits<int>::max()) return fail(MGGX_ELIMIT, "edgelist_to_bin: too many edges");
     long long V = declared_rows;
     for (size_t i = 0; i < src.size(); ++i) V = std::max<long long>(V, std::max(src[i], dst[i]) + 1LL);
+    if (V > std::numeric_limits<int>::max() - 1) return fail(MGGX_ELIMIT, "edgelist_to_bin: %lld nodes exceed int32 ids", V);
     std::vector<int> beg((size_t)V + 1, 0), csr(src.size());
     for (int s : src) beg[(size_t)s + 1]++;
     for (long long v = 0; v < V; ++v) beg[(size_t)v + 1] += beg[(size_t)v];
@@ -391,6 +395,18 @@ MGGX_EXPORT int mggx_edgelist_to_bin(const char *path, int is_mtx, const char *o
     if (num_edges) *num_edges = (int64_t)src.size();
     return MGGX_OK;
 }
+
+// Allocation failures (a size line that declares billions of nodes, an edge list beyond host memory) come back as an
+// error code: no exception crosses the C boundary.
+MGGX_EXPORT int mggx_edgelist_to_bin(const char *path, int is_mtx, const char *out_prefix, int *num_nodes, int64_t *num_edges)
+{
+    try {
+        return edgelist_to_bin_impl(path, is_mtx, out_prefix, num_nodes, num_edges);
+    } catch (const std::bad_alloc &) {
+        return fail(MGGX_ENOMEM, "edgelist_to_bin: out of host memory reading %s", path ? path : "(null)");
+    }
+}
+
 
 // ---------------------------------------------------------------------------
 // Synthetic graphs.

@@ -2,6 +2,7 @@
 // reference's layout, and the merged partition-descriptor list the aggregation
 // kernels consume.
 #include <algorithm>
+#include <chrono>
 
 #include "mggx_dev.h"
 
@@ -302,12 +303,146 @@ __global__ void __launch_bounds__(256) k_split_fill(const int *__restrict__ ptr,
     }
 }
 
+struct GuardArgs {
+    const int *arr[4];
+    long long len[4];
+};
+
+__device__ __forceinline__ unsigned long long guard_mix(unsigned long long x)
+{
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+
+// Fingerprint of up to four index arrays: the last entry of each and up to GUARD_SAMPLES entries at a fixed stride,
+// each mixed with its position.  arm != 0 stores it; otherwise it is compared with the stored one, the verdict goes to
+// fp[1] (read as int: 1 = unchanged) and, on a mismatch, `tag` to the host-visible flag.
+constexpr int GUARD_SAMPLES = 2048;
+__global__ void __launch_bounds__(256) k_guard(const GuardArgs g, unsigned long long *__restrict__ fp, volatile int *host_flag, int tag, int arm)
+{
+    __shared__ unsigned long long red[256];
+    unsigned long long h = 0;
+    for (int a = 0; a < 4; ++a) {
+        const long long n = g.len[a];
+        if (!g.arr[a] || n <= 0) continue;
+        const long long samples = n < GUARD_SAMPLES ? n : GUARD_SAMPLES;
+        const long long stride = n / samples;
+        for (long long i = threadIdx.x; i < samples; i += 256) {
+            const long long idx = i * stride;
+            h += guard_mix(((unsigned long long)(a + 1) << 56) ^ ((unsigned long long)idx << 24) ^ (unsigned)g.arr[a][idx]);
+        }
+        if (threadIdx.x == 0) h += guard_mix(((unsigned long long)(a + 5) << 56) ^ ((unsigned long long)n << 24) ^ (unsigned)g.arr[a][n - 1]);
+    }
+    red[threadIdx.x] = h;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if ((int)threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        int *ok = reinterpret_cast<int *>(fp + 1);
+        if (arm) {
+            fp[0] = red[0];
+            *ok = 1;
+        } else {
+            const int same = fp[0] == red[0];
+            *ok = same;
+            if (!same) *host_flag = tag;
+        }
+    }
+}
+
 __global__ void k_set_tail(int *node2part, int num_nodes)
 {
     node2part[num_nodes + 1] = node2part[num_nodes];
 }
 
 }  // namespace
+
+bool capturing()
+{
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(state().stream, &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return st == hipStreamCaptureStatusActive;
+}
+
+static int guard_launch(Guard &g, int arm)
+{
+    State &s = state();
+    if (!s.h_stale) {
+        void *p = nullptr;
+        if (hipHostMalloc(&p, 64, hipHostMallocMapped) != hipSuccess) return fail(MGGX_ENOMEM, "content check: pinned flag");
+        s.h_stale = static_cast<volatile int *>(p);
+        *s.h_stale = 0;
+    }
+    GuardArgs a;
+    for (int i = 0; i < 4; ++i) {
+        a.arr[i] = g.arr[i];
+        a.len[i] = g.len[i];
+    }
+    k_guard<<<1, 256, 0, s.stream>>>(a, g.d_fp, s.h_stale, g.id, arm);
+    MGGX_LAUNCH_CHECK("k_guard");
+    return MGGX_OK;
+}
+
+int guard_arm(Guard &g)
+{
+    State &s = state();
+    if (!g.d_fp) {
+        if (capturing()) return fail(MGGX_EINVAL, "first use of these CSR arrays inside a stream capture: call once outside the capture first");
+        if (hipMalloc((void **)&g.d_fp, 16) != hipSuccess) return fail(MGGX_ENOMEM, "content check: fingerprint");
+    }
+    g.id = s.next_guard_id++;
+    if (s.next_guard_id > 0x3fffffff) s.next_guard_id = 1;
+    const int rc = guard_launch(g, 1);
+    g.armed = rc == MGGX_OK;
+    return rc;
+}
+
+int guard_check(Guard &g, const int **d_ok)
+{
+    *d_ok = nullptr;
+    if (!state().plan_check || !g.armed) return MGGX_OK;
+    const int rc = guard_launch(g, 0);
+    if (rc) return rc;
+    *d_ok = g.ok();
+    return MGGX_OK;
+}
+
+void guard_free(Guard &g)
+{
+    if (g.d_fp) (void)hipFree(g.d_fp);
+    g.d_fp = nullptr;
+    g.armed = false;
+}
+
+// A check that ran on the stream since the last call found arrays that no longer match their record: everything cached
+// for those addresses is dropped (the next call builds it anew from what is there now) and the caller gets an error.
+int stale_poll()
+{
+    State &s = state();
+    if (!s.h_stale || !*s.h_stale) return MGGX_OK;
+    const int id = *s.h_stale;
+    if (capturing()) return fail(MGGX_EINVAL, "CSR arrays changed under a cached plan (found while capturing; end the capture and call mggx_forget)");
+    (void)hipStreamSynchronize(s.stream);
+    *s.h_stale = 0;
+    const int *arrs[4] = {nullptr, nullptr, nullptr, nullptr};
+    for (const GraphInfo &g : s.graphs)
+        if (g.guard.id == id)
+            for (int i = 0; i < 4; ++i) arrs[i] = g.guard.arr[i];
+    for (const Plan *p : s.plans)
+        if (p->guard.id == id)
+            for (int i = 0; i < 4; ++i) arrs[i] = p->guard.arr[i];
+    for (int i = 0; i < 4; ++i)
+        if (arrs[i]) (void)forget_pointer(arrs[i]);
+    return fail(MGGX_EINVAL, "the CSR arrays at %p changed after the library cached a plan for them: that call's kernels did nothing and the "
+                             "plan was dropped; call again (and mggx_forget() before rewriting or freeing cached arrays)", (const void *)arrs[0]);
+}
 
 int exclusive_scan_i32(const int *d_in, int *d_out, int n, long long *total_host)
 {
@@ -340,6 +475,7 @@ void plan_free(Plan *p)
     if (p->d_desc) (void)hipFree(p->d_desc);
     if (p->d_off) (void)hipFree(p->d_off);
     if (p->d_empty_rows) (void)hipFree(p->d_empty_rows);
+    guard_free(p->guard);
     delete p;
 }
 
@@ -361,27 +497,57 @@ static int plan_finish(Plan *p)
     return MGGX_OK;
 }
 
+// The cache keeps the 16 most recently used plans (front = least recently used); plans a captured graph may point at
+// are never evicted.
 static void cache_insert(Plan *p)
 {
     State &s = state();
     const size_t max_plans = 16;
+    p->bytes = sizeof(int4) * (size_t)std::max(p->num_parts, 1) + sizeof(int) * ((size_t)p->rows + 1) + sizeof(int) * (size_t)std::max(p->rows, 1);
     if (s.plans.size() >= max_plans) {
-        (void)hipStreamSynchronize(s.stream);
-        plan_free(s.plans.front());
-        s.plans.erase(s.plans.begin());
+        for (size_t i = 0; i < s.plans.size(); ++i)
+            if (!s.plans[i]->pinned) {
+                (void)hipStreamSynchronize(s.stream);
+                plan_free(s.plans[i]);
+                s.plans.erase(s.plans.begin() + (long)i);
+                break;
+            }
     }
     s.plans.push_back(p);
 }
 
+// A cache hit: most recently used last; a plan used while capturing stays for good.
+static Plan *cache_hit(size_t i)
+{
+    State &s = state();
+    Plan *p = s.plans[i];
+    if (i + 1 != s.plans.size()) {
+        s.plans.erase(s.plans.begin() + (long)i);
+        s.plans.push_back(p);
+    }
+    if (!p->pinned && capturing()) p->pinned = true;
+    return p;
+}
+
+struct BuildClock {  // adds the host-clock time of a plan build to the library's set-up account
+    std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
+    ~BuildClock() { state().plan_build_ms += std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count(); }
+};
+static const char *const CAPTURE_MSG = "plan: first use of this CSR and partition size inside a stream capture; call once outside the capture first";
+
 int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int rows, int ps, Plan **out)
 {
     State &s = state();
-    for (Plan *p : s.plans)
+    for (size_t i = 0; i < s.plans.size(); ++i) {
+        const Plan *p = s.plans[i];
         if (p->d_ptr_l == d_ptr_l && p->d_ptr_r == d_ptr_r && p->d_col_r == d_col_r && p->rows == rows && p->ps == ps &&
             !p->d_part_ptr && p->blocks == 1 && !p->unsuitable) {
-            *out = p;
+            *out = cache_hit(i);
             return MGGX_OK;
         }
+    }
+    if (capturing()) return fail(MGGX_EINVAL, "%s", CAPTURE_MSG);
+    BuildClock clock;
     Plan *p = new Plan;
     p->d_ptr_l = d_ptr_l;
     p->d_ptr_r = d_ptr_r;
@@ -476,12 +642,16 @@ int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_
                       int ps, Plan **out)
 {
     State &s = state();
-    for (Plan *p : s.plans)
+    for (size_t i = 0; i < s.plans.size(); ++i) {
+        const Plan *p = s.plans[i];
         if (p->d_ptr_l == d_row_ptr && p->d_part_ptr == d_part_ptr && p->d_part2node == d_part2node && p->rows == rows &&
             p->ps == ps && p->num_parts == num_parts) {
-            *out = p;
+            *out = cache_hit(i);
             return MGGX_OK;
         }
+    }
+    if (capturing()) return fail(MGGX_EINVAL, "%s", CAPTURE_MSG);
+    BuildClock clock;
     Plan *p = new Plan;
     p->d_ptr_l = d_row_ptr;
     p->d_part_ptr = d_part_ptr;
@@ -507,6 +677,15 @@ int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_
         }
         p->nnz_l = end;
         rc = plan_finish(p);
+        if (rc) break;
+        // the descriptors depend on these three arrays (the column array is only read while aggregating)
+        p->guard.arr[0] = d_row_ptr;
+        p->guard.len[0] = (long long)rows + 1;
+        p->guard.arr[1] = d_part_ptr;
+        p->guard.len[1] = num_parts;
+        p->guard.arr[2] = d_part2node;
+        p->guard.len[2] = num_parts;
+        rc = guard_arm(p->guard);
     } while (0);
     if (rc) {
         plan_free(p);
@@ -520,12 +699,16 @@ int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_
 int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int ps, int block_rows, Plan **out)
 {
     State &s = state();
-    for (Plan *p : s.plans)
+    for (size_t i = 0; i < s.plans.size(); ++i) {
+        const Plan *p = s.plans[i];
         if (p->d_ptr_l == d_ptr_l && p->d_col_l == d_col_l && p->real_rows == rows && p->ps == ps && p->block_rows == block_rows && p->block_lb == lb &&
             (p->blocks > 1 || p->unsuitable)) {
-            *out = p;
+            *out = cache_hit(i);
             return MGGX_OK;
         }
+    }
+    if (capturing()) return fail(MGGX_EINVAL, "%s", CAPTURE_MSG);
+    BuildClock clock;
     if (block_rows < 1 || rows < 1) return fail(MGGX_EINVAL, "plan: column blocks of %d rows over %d rows", block_rows, rows);
     const long long blocks = ((long long)rows + block_rows - 1) / block_rows;
     const long long vrows = blocks * rows;
@@ -605,19 +788,24 @@ int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, i
     return MGGX_OK;
 }
 
-int graph_info(const int *d_ptr_l, const int *d_ptr_r, int rows, GraphInfo **out)
+int graph_info(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_l, const int *d_col_r, int rows, bool internal, GraphInfo **out)
 {
     State &s = state();
     for (auto it = s.graphs.begin(); it != s.graphs.end(); ++it)
-        if (it->d_ptr_l == d_ptr_l && it->d_ptr_r == d_ptr_r && it->rows == rows) {
+        if (it->d_ptr_l == d_ptr_l && it->d_ptr_r == d_ptr_r && it->d_col_l == d_col_l && it->d_col_r == d_col_r && it->rows == rows) {
             s.graphs.splice(s.graphs.end(), s.graphs, it);  // most recently used last; the record itself does not move
+            if (!it->pinned && capturing()) it->pinned = true;
             *out = &*it;
             return MGGX_OK;
         }
+    if (capturing()) return fail(MGGX_EINVAL, "first use of these CSR arrays inside a stream capture: call once outside the capture first");
     GraphInfo g;
     g.d_ptr_l = d_ptr_l;
     g.d_ptr_r = d_ptr_r;
+    g.d_col_l = d_col_l;
+    g.d_col_r = d_col_r;
     g.rows = rows;
+    g.internal = internal;
     int ends[2] = {0, 0};
     if (rows > 0) {
         MGGX_HIP(hipStreamSynchronize(s.stream));
@@ -626,9 +814,33 @@ int graph_info(const int *d_ptr_l, const int *d_ptr_r, int rows, GraphInfo **out
     }
     g.nnz_l = ends[0];
     g.nnz_r = ends[1];
-    if (s.graphs.size() >= 32) s.graphs.erase(s.graphs.begin());
+    if (s.graphs.size() >= 32)
+        for (auto it = s.graphs.begin(); it != s.graphs.end(); ++it)
+            if (!it->pinned) {
+                (void)hipStreamSynchronize(s.stream);  // a check kernel in flight may still write the record's verdict word
+                guard_free(it->guard);
+                s.graphs.erase(it);
+                break;
+            }
     s.graphs.push_back(g);
-    *out = &s.graphs.back();
+    GraphInfo &r = s.graphs.back();
+    if (!internal && rows > 0) {
+        r.guard.arr[0] = d_ptr_l;
+        r.guard.len[0] = (long long)rows + 1;
+        r.guard.arr[1] = d_ptr_r;
+        r.guard.len[1] = d_ptr_r ? (long long)rows + 1 : 0;
+        r.guard.arr[2] = g.nnz_l > 0 ? d_col_l : nullptr;
+        r.guard.len[2] = g.nnz_l;
+        r.guard.arr[3] = g.nnz_r > 0 ? d_col_r : nullptr;
+        r.guard.len[3] = g.nnz_r;
+        const int rc = guard_arm(r.guard);
+        if (rc) {
+            guard_free(r.guard);
+            s.graphs.pop_back();
+            return rc;
+        }
+    }
+    *out = &r;
     return MGGX_OK;
 }
 
@@ -652,7 +864,18 @@ int forget_pointer(const void *d_ptr)
             ++i;
         }
     }
-    s.graphs.remove_if([d_ptr](const GraphInfo &g) { return g.d_ptr_l == d_ptr || g.d_ptr_r == d_ptr; });
+    for (auto it = s.graphs.begin(); it != s.graphs.end();) {
+        if (it->d_ptr_l == d_ptr || it->d_ptr_r == d_ptr || it->d_col_l == d_ptr || it->d_col_r == d_ptr) {
+            if (!synced && s.device >= 0) {  // a check kernel in flight may still write the record's verdict word
+                MGGX_HIP(hipStreamSynchronize(s.stream));
+                synced = true;
+            }
+            guard_free(it->guard);
+            it = s.graphs.erase(it);
+        } else {
+            ++it;
+        }
+    }
     // dense-core plans keyed by the array (freeing one forgets its own remainder arrays in turn: take them out first)
     std::vector<CorePlan *> gone;
     for (size_t i = 0; i < s.cores.size();) {

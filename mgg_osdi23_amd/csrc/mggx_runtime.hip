@@ -31,9 +31,16 @@ int workspace(size_t bytes, void **p)
 {
     State &s = state();
     if (bytes > s.ws_bytes) {
+        if (capturing()) return fail(MGGX_EINVAL, "the workspace would have to grow inside a stream capture; run the largest call once outside it first");
         if (s.ws) {
             MGGX_HIP(hipStreamSynchronize(s.stream));
-            MGGX_HIP(hipFree(s.ws));
+            if (s.ws_captured) {  // a captured graph may still point at it: kept until mggx_release_cached
+                s.retired.push_back(s.ws);
+                s.retired_bytes += s.ws_bytes;
+                s.ws_captured = false;
+            } else {
+                MGGX_HIP(hipFree(s.ws));
+            }
             s.ws = nullptr;
             s.ws_bytes = 0;
         }
@@ -45,6 +52,7 @@ int workspace(size_t bytes, void **p)
         }
         s.ws_bytes = want;
     }
+    if (!s.ws_captured && capturing()) s.ws_captured = true;
     *p = s.ws;
     return MGGX_OK;
 }
@@ -91,7 +99,7 @@ MGGX_EXPORT int mggx_set_stream(void *hip_stream)
 MGGX_EXPORT int mggx_sync(void)
 {
     MGGX_HIP(hipStreamSynchronize(state().stream));
-    return MGGX_OK;
+    return mggx::stale_poll();  // a content check that ran on the stream may have found changed CSR arrays
 }
 
 MGGX_EXPORT int mggx_malloc(void **d_ptr, size_t bytes)
@@ -217,12 +225,47 @@ MGGX_EXPORT int mggx_release_cached(void)
     }
     for (mggx::Plan *p : s.plans) mggx::plan_free(p);
     s.plans.clear();
+    for (mggx::GraphInfo &g : s.graphs) mggx::guard_free(g.guard);
     s.graphs.clear();
     if (s.ws) {
         MGGX_HIP(hipFree(s.ws));
         s.ws = nullptr;
         s.ws_bytes = 0;
     }
+    for (void *p : s.retired) (void)hipFree(p);
+    s.retired.clear();
+    s.retired_bytes = 0;
+    s.ws_captured = s.core_ws_captured = false;
+    if (s.h_stale) *s.h_stale = 0;
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_set_plan_check(int on)
+{
+    if (on != 0 && on != 1) return fail(MGGX_EINVAL, "set_plan_check: %d", on);
+    state().plan_check = on;
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_cache_stats(mggx_cache_stats_t *out)
+{
+    if (!out) return fail(MGGX_EINVAL, "cache_stats: NULL");
+    mggx::State &s = state();
+    *out = mggx_cache_stats_t{};
+    for (const mggx::Plan *p : s.plans) {
+        out->plans += 1;
+        out->plan_bytes += (int64_t)p->bytes;
+    }
+    for (const mggx::CorePlan *c : s.cores) {
+        out->core_plans += 1;
+        out->core_plan_bytes += (int64_t)c->bytes;
+    }
+    out->workspace_bytes = (int64_t)s.ws_bytes;
+    out->core_scratch_bytes = (int64_t)s.core_ws_bytes;
+    out->retired_bytes = (int64_t)s.retired_bytes;
+    out->plan_build_ms = s.plan_build_ms;
+    out->core_plan_build_ms = s.core_plan_build_ms;
+    out->search_ms = s.search_ms;
     return MGGX_OK;
 }
 

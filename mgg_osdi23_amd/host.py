@@ -36,6 +36,12 @@ class _AggKnobs(C.Structure):
     _fields_ = [("ps", C.c_int), ("wpb", C.c_int), ("dist", C.c_int), ("col_block_rows", C.c_int), ("core_rows", C.c_int)]
 
 
+class _CacheStats(C.Structure):
+    _fields_ = [("plans", C.c_int64), ("plan_bytes", C.c_int64), ("core_plans", C.c_int64), ("core_plan_bytes", C.c_int64),
+                ("workspace_bytes", C.c_int64), ("core_scratch_bytes", C.c_int64), ("retired_bytes", C.c_int64),
+                ("plan_build_ms", C.c_double), ("core_plan_build_ms", C.c_double), ("search_ms", C.c_double)]
+
+
 class _DenseOpts(C.Structure):
     _fields_ = [("ld_x", C.c_int64), ("ld_out", C.c_int64), ("d_row_scale", C.c_void_p), ("relu", C.c_uint32)]
 
@@ -52,7 +58,7 @@ EXPORTS = [
     "mggx_last_error", "mggx_version", "mggx_init", "mggx_device_name", "mggx_set_stream", "mggx_sync",
     "mggx_malloc", "mggx_free", "mggx_memset", "mggx_memcpy_h2d", "mggx_memcpy_d2h", "mggx_memcpy_d2d",
     "mggx_timer_create", "mggx_timer_start", "mggx_timer_stop", "mggx_timer_elapsed_ms", "mggx_timer_destroy",
-    "mggx_release_cached", "mggx_forget", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_core_layout_build", "mggx_core_layout_fetch", "mggx_graph_read",
+    "mggx_release_cached", "mggx_forget", "mggx_set_plan_check", "mggx_cache_stats", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_core_layout_build", "mggx_core_layout_fetch", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
     "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_compact_remote_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_sag_parts_static", "mggx_mlp2_xw", "mggx_spmm",
     "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_gather_probe", "mggx_gather_rows", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
@@ -265,14 +271,19 @@ def sync() -> None:
 
 
 _pinned = {}  # CSR tensors of cached plans, by address: keeps the addresses from being reused while cached
+_PIN_MAX_SETS, _PIN_MAX_BYTES = 64, 8 << 30
 
 
 def _pin(*tensors) -> None:
+    """Holds a reference to the CSR tensors of a call so that torch's allocator does not hand their addresses to other
+    data while the library has plans cached for them; bounded by count and bytes, oldest first, and the library forgets
+    a set before it is let go."""
     key = tuple(t.data_ptr() if t is not None else 0 for t in tensors)
     if key in _pinned:
         return
     _pinned[key] = tensors
-    while len(_pinned) > 256:  # before the oldest set may be freed, the library forgets what it cached for it
+    size = lambda ts: sum(t.numel() * t.element_size() for t in ts if t is not None)
+    while len(_pinned) > _PIN_MAX_SETS or (len(_pinned) > 1 and sum(size(ts) for ts in _pinned.values()) > _PIN_MAX_BYTES):
         old = _pinned.pop(next(iter(_pinned)))
         for t in old:
             if t is not None:
@@ -289,6 +300,18 @@ def forget(tensor) -> None:
 def release_cached() -> None:
     _check(lib().mggx_release_cached())
     _pinned.clear()
+
+
+def set_plan_check(on: bool) -> None:
+    """Content checks of cached plans against the caller's CSR arrays (on by default)."""
+    _check(lib().mggx_set_plan_check(int(on)))
+
+
+def cache_stats() -> dict:
+    """What the library holds (plans, scratch) and what its set-up has cost so far (ms, host clock)."""
+    st = _CacheStats()
+    _check(lib().mggx_cache_stats(C.byref(st)))
+    return {k: getattr(st, k) for k, _ in _CacheStats._fields_}
 
 
 def device_name() -> str:

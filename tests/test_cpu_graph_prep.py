@@ -228,6 +228,11 @@ def test_edgelist_to_bin_converter(tmp_path):
     assert b.tolist() == want_ptr and c.tolist() == want_col
     with pytest.raises(host.MggxError):
         host.edgelist_to_bin(str(tmp_path / "missing.txt"), str(tmp_path / "x"))
+    # a size line beyond int32 node ids is an error code, not a crash or a truncated count
+    huge = tmp_path / "huge.mtx"
+    huge.write_text("%%MatrixMarket matrix coordinate pattern general\n4000000000 4000000000 1\n1 2\n")
+    with pytest.raises(host.MggxError, match="int32"):
+        host.edgelist_to_bin(str(huge), str(tmp_path / "y"), is_mtx=True)
 
 
 # --------------------------------------------------------------------------- generators

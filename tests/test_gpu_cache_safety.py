@@ -1,0 +1,149 @@
+"""Cached plans against the caller's memory: arrays rewritten in place without mggx_forget, captured graphs that outlive
+a growing workspace, first uses inside a capture."""
+import numpy as np
+import pytest
+
+from oracle import orc
+from tests.util import FP32_TOL, assert_close_to_oracle, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _agg(gpu, out, x, d_ptr, d_col, V, dim, ps=16, wpb=4, dist=2, **kw):
+    import torch
+    zp = torch.zeros(V + 1, dtype=torch.int32, device="cuda")
+    zc = torch.zeros(1, dtype=torch.int32, device="cuda")
+    _agg.keep = (zp, zc)
+    gpu.mgg_SAG_np_div(out, x, d_ptr, d_col, zp, zc, 0, V, dim, V, 0, ps, wpb, dist, **kw)
+
+
+def _want(x, ptr, col, V, dim):
+    want = orc.sag_np_div(x, x, ptr, col, None, None, 0, V, dim, V)
+    mag = orc.sag_np_div_rows(np.arange(V, dtype=np.int32), x, x, ptr, col, None, None, 0, V, dim, V, abs_sum=True)
+    return want, mag
+
+
+@pytest.mark.parametrize("core_rows", [-1, 1024])
+def test_csr_rewritten_in_place_without_forget(gpu, core_rows):
+    """A different graph written into the same device arrays, and no mggx_forget: the cached plan (and dense-core plan)
+    no longer fits.  The call must give an error or the right answer, never a sum through the stale plan."""
+    import torch
+    V, dim = 6000, 16
+    ptr_a, col_a = gpu.gen_rmat(13, V, 200_000, seed=1)
+    ptr_b, col_b = gpu.gen_rmat(13, V, 120_000, seed=2)
+    assert len(col_b) < len(col_a)
+    x = gpu.fill_normal((V, dim), seed=3)
+    d_x = to_dev(x)
+    d_ptr, d_col = to_dev(ptr_a), to_dev(col_a)
+    zp = torch.zeros(V + 1, dtype=torch.int32, device="cuda")
+    zc = torch.zeros(1, dtype=torch.int32, device="cuda")
+    call = lambda out: gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, zp, zc, 0, V, dim, V, 0, 16, 4, 2, core_rows=core_rows)
+    out = torch.empty(V, dim, device="cuda")
+    call(out)
+    gpu.sync()
+    want, mag = _want(x, ptr_a, col_a, V, dim)
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "graph A")
+    # graph B into the same arrays, behind the library's back
+    d_ptr.copy_(torch.from_numpy(ptr_b))
+    d_col[: len(col_b)].copy_(torch.from_numpy(col_b))
+    torch.cuda.synchronize()
+    want, mag = _want(x, ptr_b, col_b, V, dim)
+    out.fill_(-7.0)
+    errors = 0
+    for attempt in range(3):
+        try:
+            call(out)
+            gpu.sync()
+        except gpu.MggxError as e:
+            assert "changed" in str(e)
+            errors += 1
+            # the stale plan's kernels did nothing
+            assert bool((out == -7.0).all()), "kernels of a stale plan wrote to the output"
+            continue
+        break
+    else:
+        raise AssertionError("no call succeeded after the rewrite")
+    assert errors == 1
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "graph B after the rewrite")
+    gpu.forget(d_ptr)
+
+
+def test_explicit_partition_arrays_rewritten_in_place(gpu):
+    import torch
+    V, dim, ps = 4000, 16, 8
+    ptr_a, col_a = gpu.gen_rmat(12, V, 60_000, seed=4)
+    ptr_b, col_b = gpu.gen_rmat(12, V, 30_000, seed=5)
+    x = gpu.fill_normal((V, dim), seed=6)
+    pa, p2na, _ = orc.build_part(ptr_a, V, ps)
+    pb, p2nb, _ = orc.build_part(ptr_b, V, ps)
+    assert len(p2nb) < len(p2na) and len(col_b) < len(col_a)
+    d_ptr, d_col, d_pp, d_p2n, d_x = to_dev(ptr_a), to_dev(col_a), to_dev(pa), to_dev(p2na), to_dev(x)
+    out = torch.zeros(V, dim, device="cuda")
+    gpu.SAG_host(out, d_x, d_ptr, d_col, d_pp, d_p2n, 0, V, len(p2na), ps, dim, 32, 4, 1)
+    gpu.sync()
+    assert np.allclose(out.cpu().numpy(), orc.sag_ref(x, ptr_a, col_a), rtol=1e-4, atol=1e-4)
+    # same arrays, same partition count passed, other contents
+    d_ptr.copy_(torch.from_numpy(ptr_b))
+    d_col[: len(col_b)].copy_(torch.from_numpy(col_b))
+    d_pp.zero_()
+    d_pp[: len(pb)].copy_(torch.from_numpy(pb))
+    d_p2n[: len(p2nb)].copy_(torch.from_numpy(p2nb))
+    torch.cuda.synchronize()
+    out.fill_(-7.0)
+    with pytest.raises(gpu.MggxError, match="changed"):
+        gpu.SAG_host(out, d_x, d_ptr, d_col, d_pp, d_p2n, 0, V, len(p2na), ps, dim, 32, 4, 1)
+        gpu.sync()
+    assert bool((out == -7.0).all())
+    gpu.forget(d_ptr)
+
+
+def test_captured_graph_survives_workspace_growth_and_cache_pressure(gpu):
+    """A captured forward keeps pointing at the plan and the scratch block of its capture.  Later eager calls that need a
+    larger block, and enough other plans to fill the cache, must not free what the graph uses."""
+    import torch
+    V, dim = 5000, 16
+    ptr, col = gpu.gen_rmat(13, V, 150_000, seed=9)
+    x = gpu.fill_normal((V, dim), seed=1)
+    d_ptr, d_col, d_x = to_dev(ptr), to_dev(col), to_dev(x)
+    zp, zc = torch.zeros(V + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    out = torch.empty(V, dim, device="cuda")
+    big_V = 60_000
+    bptr, bcol = gpu.gen_rmat(16, big_V, 1_500_000, seed=10)
+    d_bptr, d_bcol = to_dev(bptr), to_dev(bcol)
+    bzp = torch.zeros(big_V + 1, dtype=torch.int32, device="cuda")
+    d_bx, bout = to_dev(gpu.fill_normal((big_V, 64), seed=2)), torch.empty(big_V, 64, device="cuda")
+    call = lambda: gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, zp, zc, 0, V, dim, V, 0, 16, 4, 2)
+    gpu.release_cached()  # start from an empty workspace, so the capture below pins a small one
+    side = torch.cuda.Stream()
+    try:
+        with torch.cuda.stream(side):
+            gpu.use_torch_stream()
+            call()
+            side.synchronize()
+            want = out.clone()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                gpu.use_torch_stream()
+                call()
+                # a first use inside the capture is refused before anything is launched or allocated
+                with pytest.raises(gpu.MggxError, match="capture"):
+                    gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, zp, zc, 0, V, dim, V, 0, 7, 4, 2)
+            before = gpu.cache_stats()
+            # eager: a much larger call (the workspace must grow) and 20 other plans (the cache holds 16)
+            gpu.use_torch_stream()
+            gpu.mgg_SAG_np_div(bout, d_bx, d_bptr, d_bcol, bzp, zc, 0, big_V, 64, big_V, 0, 16, 1, 1)
+            for ps in range(20, 40):
+                gpu.mgg_SAG_np_div(bout, d_bx, d_bptr, d_bcol, bzp, zc, 0, big_V, 64, big_V, 0, ps, 8, 1)
+            side.synchronize()
+            after = gpu.cache_stats()
+            assert after["workspace_bytes"] > before["workspace_bytes"]
+            assert after["retired_bytes"] >= before["workspace_bytes"] > 0
+            for i in range(2):
+                out.fill_(-1.0)
+                graph.replay()
+                side.synchronize()
+                assert torch.equal(out, want), "replay %d after the workspace grew differs" % i
+    finally:
+        torch.cuda.synchronize()
+        gpu.use_torch_stream()
+        gpu.release_cached()
