@@ -86,15 +86,18 @@ int mggx_release_cached(void);
 /* Drops what the library remembers about the CSR array at this device address (cached partition plans, search
  * results): call it before freeing or rewriting an index array that aggregation calls have seen, when the memory is
  * not released through mggx_free (which does this itself) -- an allocator may hand the same address out again.
- * A caller that forgets to is still safe: cached records are found by address, but before every use a small kernel on
- * the call's stream compares a fingerprint of the arrays (their last entries -- the edge counts -- and up to 2048
- * entries of each at a fixed stride) with the one taken when the record was made.  On a mismatch every kernel of that
- * call returns at once (the output is left as it was, nothing is read through stale indices), and the next library
- * call on this thread, mggx_sync() included, drops the record and returns MGGX_EINVAL; calling again then works on the
- * arrays as they are.  The check is a sample: an edit that keeps every row count and misses every sampled entry is not
- * seen -- mggx_forget() stays the rule for in-place edits.  mggx_set_plan_check(0) turns the checks off. */
+ * A caller that forgets to is still covered: cached records are found by address, but every kernel of a call first
+ * compares the live edge counts of the arrays (ptr_l[rows], ptr_r[rows]) with the counts its records were built for
+ * (level 1, the default: two scalar loads per kernel), and at level 2 a one-workgroup kernel on the call's stream also
+ * compares a fingerprint of the arrays (their last entries and up to 512 entries of each at a fixed stride) with the
+ * one taken when the record was made (about 8 microseconds per call).  On a mismatch every kernel of that call returns
+ * at once (the output is left as it was, nothing is read through stale indices), and the next library call on this
+ * thread, mggx_sync() included, drops the records and returns MGGX_EINVAL; calling again then works on the arrays as
+ * they are.  Neither check sees an edit that keeps the edge counts and misses every sampled entry -- mggx_forget()
+ * stays the rule for in-place edits.  mggx_set_plan_check(level): 0 = off, 1 = edge counts, 2 = edge counts and
+ * fingerprint. */
 int mggx_forget(const void *d_ptr);
-int mggx_set_plan_check(int on);
+int mggx_set_plan_check(int level);
 
 /* What the library holds and what its set-up has cost so far (host clock, milliseconds, since the process started). */
 typedef struct mggx_cache_stats_t {
@@ -364,6 +367,12 @@ int mggx_copy_bytes(void *d_dst, const void *d_src, size_t n);
  * a given size is the ceiling the aggregation kernels are measured against where their table is cache resident. */
 int mggx_gather_probe(float *d_sink, const void *d_table, int64_t rows, size_t ld_bytes, size_t row_bytes,
                       int64_t n_gathers, unsigned seed, int64_t *n_done);
+
+/* Yardstick for the dense-core kernel (no counterpart in the reference): at least n_reads row reads of row_bytes bytes
+ * (16..256, in 16-byte pieces) from an LDS tile of 256 columns laid out like that kernel's, at pseudo-random columns,
+ * one row per lane and step, summed in registers; no memory traffic inside the loop.  d_sink as for mggx_gather_probe.
+ * What this sustains is the ceiling of the core x core block's sums. */
+int mggx_lds_probe(float *d_sink, size_t row_bytes, int64_t n_reads, unsigned seed, int64_t *n_done);
 
 /* How the aggregation kernels address feature rows: 0 (default) picks per call -- 32-bit buffer offsets when both
  * tables lie inside one window of < 2 GiB and < 2^24 rows, 64-bit addresses otherwise; 1 always uses 64-bit

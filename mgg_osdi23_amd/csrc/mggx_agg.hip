@@ -55,7 +55,7 @@ struct AggArgs {
     const int4 *desc;
     const int *off;
     const float *rs_out;
-    const int *ok;  // when set: *ok == 0 means the plan is stale (the CSR arrays changed) and every kernel returns at once
+    Gate gate;      // closed = the plan is stale (the caller's CSR arrays changed): every kernel returns at once
     int2 *c_hdr;   // [2 * workgroups]: head, tail
     float *c_val;  // [2 * workgroups][cpad]
     long long ld_in, ld_out;
@@ -282,7 +282,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     // (-5 % at width 16).  With fewer slots adjacent wavefronts share those lines and the hint costs 1-3 %.
     constexpr bool STREAM = S >= 16;
     extern __shared__ float lds[];
-    if (a.ok && *a.ok == 0) return;
+    if (gate_closed(a.gate)) return;
 
     const int lane = lane_id();
     const int wave = (int)(threadIdx.x >> 6);
@@ -556,7 +556,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
 // wavefront and several components per lane.
 __global__ void __launch_bounds__(256) k_agg_fixup(const AggArgs a, int num_wg, int comp_lanes)
 {
-    if (a.ok && *a.ok == 0) return;
+    if (gate_closed(a.gate)) return;
     const int lane = lane_id();
     const int group = 64 / comp_lanes;
     const long long b = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * group + lane / comp_lanes;
@@ -586,7 +586,7 @@ __global__ void __launch_bounds__(256) k_agg_fixup(const AggArgs a, int num_wg, 
 // Rows with no neighbor at all: the sum is zero.
 __global__ void __launch_bounds__(256) k_agg_empty_rows(const AggArgs a, const int *__restrict__ rows, int n_rows)
 {
-    if (a.ok && *a.ok == 0) return;
+    if (gate_closed(a.gate)) return;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (long long)n_rows * a.dim) return;
     const int r = rows[idx / a.dim];
@@ -597,7 +597,7 @@ __global__ void __launch_bounds__(256) k_agg_empty_rows(const AggArgs a, const i
 // Column-blocked plans: out[v] = epilogue(sum over blocks c of P[c * rows + v]), blocks summed in order.
 __global__ void __launch_bounds__(256) k_agg_block_reduce(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp)
 {
-    if (a.ok && *a.ok == 0) return;
+    if (gate_closed(a.gate)) return;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (long long)rows * a.dim) return;
     const int v = (int)(idx / a.dim), d = (int)(idx % a.dim);
@@ -610,7 +610,7 @@ __global__ void __launch_bounds__(256) k_agg_block_reduce(const AggArgs a, const
 // other tables (row scale, accumulation and ReLU only).
 __global__ void __launch_bounds__(256) k_agg_block_reduce4(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp)
 {
-    if (a.ok && *a.ok == 0) return;
+    if (gate_closed(a.gate)) return;
     const int q = a.dim >> 2;  // float4 per row
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (long long)rows * q) return;
@@ -673,7 +673,7 @@ struct FixedScratch {
 };
 
 int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, const int *d_col_l, const int *d_col_r,
-            int lb, int dim, int wpb, int dist, const mggx_agg_opts &o, const int *ok, const FixedScratch *fixed = nullptr)
+            int lb, int dim, int wpb, int dist, const mggx_agg_opts &o, const Gate &gate, const FixedScratch *fixed = nullptr)
 {
     State &st = state();
     if (dim < 1 || dim > 256) return fail(MGGX_ELIMIT, "aggregation: dim %d outside 1..256", dim);
@@ -735,7 +735,7 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     a.desc = plan->d_desc;
     a.off = plan->d_off;
     a.rs_out = blocked ? nullptr : o.d_row_scale_out;
-    a.ok = ok;
+    a.gate = gate;
     a.ld_in = ld_in;
     a.ld_out = blocked ? ldp : ld_out;
     a.num_parts = plan->num_parts;
@@ -895,9 +895,9 @@ Knobs resolve_knobs(const GraphInfo &g, int dim, int dtype, int ps, int wpb, int
     return k;
 }
 
-// `ok`: the verdict word of the call's content check (NULL = no gate); every kernel launched below is gated on it.
+// `gate`: the call's content check of the caller's CSR arrays; every kernel launched below looks at it first.
 int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in_local, const void *d_in_remote, const int *d_ptr_l,
-              const int *d_col_l, const int *d_ptr_r, const int *d_col_r, int lb, int ub, int dim, const mggx_agg_opts &o, const int *ok)
+              const int *d_col_l, const int *d_ptr_r, const int *d_col_r, int lb, int ub, int dim, const mggx_agg_opts &o, const Gate &gate)
 {
     Plan *plan = nullptr;
     int rc;
@@ -917,11 +917,11 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
             hipEvent_t fork, join;
             rc = core_side_stream(&side, &fork, &join);
             if (rc) return rc;
-            rc = run_core_stage(cp, static_cast<const float *>(d_in_local), dim, ld_in, ok, st0.stream);
+            rc = run_core_stage(cp, static_cast<const float *>(d_in_local), dim, ld_in, gate, st0.stream);
             if (rc) return rc;
             MGGX_HIP(hipEventRecord(fork, st0.stream));
             MGGX_HIP(hipStreamWaitEvent(side, fork, 0));
-            rc = run_core_sums(cp, dim, ok, side);
+            rc = run_core_sums(cp, dim, gate, side);
             const hipError_t er = hipEventRecord(join, side);
             int rc2 = MGGX_OK;
             GraphInfo *gr = nullptr;
@@ -932,18 +932,19 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
                 Knobs k2 = k;
                 k2.core_rows = -1;
                 if (k2.block_rows > 0 && !blocking_eligible(*gr, k2.block_rows)) k2.block_rows = -1;
-                rc2 = run_knobs(*gr, k2, d_out, d_in_local, nullptr, cp->d_rem_ptr, cp->d_rem_col, nullptr, nullptr, lb, ub, dim, o2, ok);
+                rc2 = run_knobs(*gr, k2, d_out, d_in_local, nullptr, cp->d_rem_ptr, cp->d_rem_col, nullptr, nullptr, lb, ub, dim, o2, gate);
             }
             // the caller's stream takes the side stream back in whatever happened, so no work of this call outlives it unordered
             const hipError_t ew = er == hipSuccess ? hipStreamWaitEvent(st0.stream, join, 0) : er;
             if (rc) return rc;
             if (rc2) return rc2;
             if (ew != hipSuccess) return fail(MGGX_EHIP, "aggregation: joining the side stream: %s", hipGetErrorString(ew));
-            rc = run_core_finish(cp, d_out, dim, ld_out, o.d_row_scale_out, (o.flags & MGGX_AGG_RELU) ? 1 : 0, ok, st0.stream);
+            rc = run_core_finish(cp, d_out, dim, ld_out, o.d_row_scale_out, (o.flags & MGGX_AGG_RELU) ? 1 : 0, gate, st0.stream);
             if (rc) return rc;
             State &st = state();
             const size_t n = strlen(st.last_kernel);
-            snprintf(st.last_kernel + n, sizeof(st.last_kernel) - n, " core=%d", cp->core);
+            snprintf(st.last_kernel + n, sizeof(st.last_kernel) - n, " core=%d core_nnz=%lld rem_nnz=%lld", cp->core, (long long)cp->core_nnz,
+                     (long long)cp->rem_nnz);
             return MGGX_OK;
         }
     }
@@ -956,7 +957,7 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
         rc = plan_get(d_ptr_l, d_ptr_r, d_col_r, ub - lb, k.ps, &plan);
         if (rc) return rc;
     }
-    return run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, k.wpb, k.dist, o, ok);
+    return run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, k.wpb, k.dist, o, gate);
 }
 
 int check_np_div_args(const char *who, const int *d_ptr_l, int lb, int ub, int nodes_per_pe, int &ps, int block_rows, int core_rows)
@@ -988,11 +989,11 @@ MGGX_EXPORT int mggx_sag_np_div(float *d_out, const void *d_in_local, const void
     mggx::GraphInfo *g = nullptr;
     rc = mggx::graph_info(d_ptr_l, d_ptr_r, d_col_l, d_col_r, ub - lb, false, &g);
     if (rc) return rc;
-    const int *ok = nullptr;
-    rc = mggx::guard_check(g->guard, &ok);
+    mggx::Gate gate;
+    rc = mggx::guard_check(g->guard, &gate);
     if (rc) return rc;
     const mggx::Knobs k = mggx::resolve_knobs(*g, dim, o.in_dtype, ps, wpb, dist, o.col_block_rows, o.core_rows);
-    return mggx::run_knobs(*g, k, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o, ok);
+    return mggx::run_knobs(*g, k, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o, gate);
 }
 
 MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const void *d_in_remote, const int *d_ptr_l,
@@ -1012,8 +1013,8 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
     mggx::GraphInfo *g = nullptr;
     rc = mggx::graph_info(d_ptr_l, d_ptr_r, d_col_l, d_col_r, ub - lb, false, &g);
     if (rc) return rc;
-    const int *ok = nullptr;
-    rc = mggx::guard_check(g->guard, &ok);  // one check for the whole search
+    mggx::Gate gate;
+    rc = mggx::guard_check(g->guard, &gate);  // one fingerprint check for the whole search
     if (rc) return rc;
     mggx::State &st = mggx::state();
     const auto search_t0 = std::chrono::steady_clock::now();
@@ -1038,7 +1039,7 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
     static const int wpbs[] = {8, 4, 16}, dists[] = {1, 2, 4, 8, 16};
     float best = -1.f;
     mggx::Knobs bk{pss[0], 8, 1, blks[0], cores[0]};
-    rc = mggx::run_knobs(*g, bk, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o, ok);  // warm-up
+    rc = mggx::run_knobs(*g, bk, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o, gate);  // warm-up
     for (int ci = 0; ci < n_core && !rc; ++ci)
     for (int pi = 0; pi < n_ps && !rc; ++pi)
         for (int bi = 0; bi < n_blk && !rc; ++bi)
@@ -1048,7 +1049,7 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
                     float ms_min = -1.f;
                     for (int rep = 0; rep < 3 && !rc; ++rep) {
                         hipError_t e = hipEventRecord(e0, st.stream);
-                        rc = mggx::run_knobs(*g, k, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o, ok);
+                        rc = mggx::run_knobs(*g, k, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o, gate);
                         if (e == hipSuccess) e = hipEventRecord(e1, st.stream);
                         if (e == hipSuccess) e = hipEventSynchronize(e1);
                         float ms = 0.f;
@@ -1062,7 +1063,7 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
     (void)hipEventDestroy(e1);
     if (rc) return rc;
     // leave the winner's result in d_out and remember it
-    rc = mggx::run_knobs(*g, bk, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o, ok);
+    rc = mggx::run_knobs(*g, bk, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o, gate);
     if (rc) return rc;
     MGGX_HIP(hipStreamSynchronize(st.stream));
     // the search's own time: what the plan builds inside it took is accounted for separately
@@ -1090,12 +1091,12 @@ MGGX_EXPORT int mggx_sag_parts(float *d_out, const float *d_in, const int *d_row
     if (rc) return rc;
     rc = mggx::plan_get_explicit(d_row_ptr, d_part_ptr, d_part2node, num_nodes, num_parts, ps, &plan);
     if (rc) return rc;
-    const int *ok = nullptr;
-    rc = mggx::guard_check(plan->guard, &ok);
+    mggx::Gate gate;
+    rc = mggx::guard_check(plan->guard, &gate);
     if (rc) return rc;
     mggx_agg_opts o{};
     o.flags = MGGX_AGG_ACCUMULATE;
-    return mggx::run_agg(plan, d_out, d_in, nullptr, d_col, nullptr, lowbound, dim, wpb, dist, o, ok);
+    return mggx::run_agg(plan, d_out, d_in, nullptr, d_col, nullptr, lowbound, dim, wpb, dist, o, gate);
 }
 
 namespace mggx {
@@ -1156,7 +1157,7 @@ MGGX_EXPORT int mggx_sag_parts_static(float *d_out, const float *d_in, const int
     const mggx::FixedScratch fx{base + desc_bytes + off_bytes, (size_t)MGGX_STATIC_SCRATCH_BYTES - desc_bytes - off_bytes, d_row_ptr + num_nodes};
     mggx_agg_opts o{};
     o.flags = MGGX_AGG_ACCUMULATE;
-    return mggx::run_agg(&plan, d_out, d_in, nullptr, d_col, nullptr, lowbound, dim, wpb, dist, o, nullptr, &fx);
+    return mggx::run_agg(&plan, d_out, d_in, nullptr, d_col, nullptr, lowbound, dim, wpb, dist, o, mggx::Gate{}, &fx);
 }
 
 MGGX_EXPORT int mggx_spmm(float *d_out, const float *d_in, const int *d_row_ptr, const int *d_col, int num_nodes,
@@ -1172,10 +1173,10 @@ MGGX_EXPORT int mggx_spmm(float *d_out, const float *d_in, const int *d_row_ptr,
     mggx::GraphInfo *g = nullptr;
     rc = mggx::graph_info(d_row_ptr, nullptr, d_col, nullptr, num_nodes, false, &g);
     if (rc) return rc;
-    const int *ok = nullptr;
-    rc = mggx::guard_check(g->guard, &ok);
+    mggx::Gate gate;
+    rc = mggx::guard_check(g->guard, &gate);
     if (rc) return rc;
     // the whole graph on one GPU: the same knob rules (and column-blocked order for long rows) as mggx_sag_np_div
     mggx::Knobs k = mggx::resolve_knobs(*g, dim, MGGX_F32, ps, wpb, 0, 0, 0);
-    return mggx::run_knobs(*g, k, d_out, d_in, nullptr, d_row_ptr, d_col, nullptr, nullptr, 0, num_nodes, dim, o, ok);
+    return mggx::run_knobs(*g, k, d_out, d_in, nullptr, d_row_ptr, d_col, nullptr, nullptr, 0, num_nodes, dim, o, gate);
 }

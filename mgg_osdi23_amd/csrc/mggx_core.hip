@@ -25,9 +25,9 @@ constexpr int CORE_WAVES = 4;   // slices (of 64 rows) per workgroup: as small a
 
 // tab[s * core + i] = elements 4 s .. 4 s + 3 of the feature row of the rank-i node (zero past dim)
 __global__ void __launch_bounds__(256) k_core_stage(v4f *__restrict__ tab, const float *__restrict__ in, const int *__restrict__ order,
-                                                    int core, int n4, int dim, long long ld_in, const int *__restrict__ ok)
+                                                    int core, int n4, int dim, long long ld_in, const Gate gate)
 {
-    if (ok && *ok == 0) return;
+    if (gate_closed(gate)) return;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (long long)core * n4) return;
     const int s = (int)(idx / core), i = (int)(idx % core);
@@ -45,11 +45,11 @@ __global__ void __launch_bounds__(256) k_core_stage(v4f *__restrict__ tab, const
 template <int N4>
 __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *__restrict__ blk_off, const unsigned short *__restrict__ idx,
                                                                const v4f *__restrict__ tab, v4f *__restrict__ partial, int core, int ntiles,
-                                                               int tiles_per_seg, const int *__restrict__ ok)
+                                                               int tiles_per_seg, const Gate gate)
 {
     constexpr int TC = CORE_TC, TP = TC + 1;  // column TC of every slice row is zero: what padding entries read
     extern __shared__ v4f tile[];             // [N4][TP]
-    if (ok && *ok == 0) return;
+    if (gate_closed(gate)) return;
     const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
     const int g = (int)blockIdx.x * CORE_WAVES + wave;
     const int seg = (int)blockIdx.y;
@@ -104,9 +104,9 @@ __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *_
 // element of the core rows only (idx -> rank -> row); all_rows = 1: every row (needed when act is the ReLU).
 __global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, const float *__restrict__ partial, const int *__restrict__ rank,
                                                      const int *__restrict__ order, const float *__restrict__ rs, int rows, int dim,
-                                                     long long ld_out, int core, int n4, int nseg, int relu, int all_rows, const int *__restrict__ ok)
+                                                     long long ld_out, int core, int n4, int nseg, int relu, int all_rows, const Gate gate)
 {
-    if (ok && *ok == 0) return;
+    if (gate_closed(gate)) return;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (long long)(all_rows ? rows : core) * dim) return;
     const int i = (int)(idx / dim), d = (int)(idx % dim);
@@ -126,9 +126,9 @@ __global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, co
 // The same, four columns per thread, where the output rows take 16-byte accesses.
 __global__ void __launch_bounds__(256) k_core_finish4(float *__restrict__ out, const v4f *__restrict__ partial, const int *__restrict__ rank,
                                                       const int *__restrict__ order, const float *__restrict__ rs, int rows, int n4,
-                                                      long long ld_out, int core, int nseg, int relu, int all_rows, const int *__restrict__ ok)
+                                                      long long ld_out, int core, int nseg, int relu, int all_rows, const Gate gate)
 {
-    if (ok && *ok == 0) return;
+    if (gate_closed(gate)) return;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (long long)(all_rows ? rows : core) * n4) return;
     const int i = (int)(idx / n4), q = (int)(idx % n4);
@@ -146,7 +146,7 @@ __global__ void __launch_bounds__(256) k_core_finish4(float *__restrict__ out, c
 }
 
 template <int N4>
-int launch_sell(const CorePlan *p, const v4f *tab, v4f *partial, const int *ok, hipStream_t stream)
+int launch_sell(const CorePlan *p, const v4f *tab, v4f *partial, const Gate &gate, hipStream_t stream)
 {
     const size_t lds = (size_t)N4 * (CORE_TC + 1) * sizeof(v4f);
     static bool raised = false;  // per instantiation
@@ -157,7 +157,7 @@ int launch_sell(const CorePlan *p, const v4f *tab, v4f *partial, const int *ok, 
     // row groups vary fastest in the grid: workgroups that run side by side then read the same tiles, and a CU holds dense
     // and sparse row groups at once (the reverse order measured 25 % slower)
     const dim3 grid((unsigned)(p->core / (CORE_WAVES * 64)), (unsigned)p->nseg);
-    k_core_sell<N4><<<grid, dim3(CORE_WAVES * 64), lds, stream>>>(p->d_blk_off, p->d_idx, tab, partial, p->core, p->ntiles, p->ntiles / p->nseg, ok);
+    k_core_sell<N4><<<grid, dim3(CORE_WAVES * 64), lds, stream>>>(p->d_blk_off, p->d_idx, tab, partial, p->core, p->ntiles, p->ntiles / p->nseg, gate);
     MGGX_LAUNCH_CHECK("k_core_sell");
     return MGGX_OK;
 }
@@ -317,7 +317,7 @@ static int core_scratch(const CorePlan *p, int n4, v4f **tab, v4f **partial)
 
 // The core's feature rows into the slice-major table, on `stream` (a few microseconds on an idle chip, ten times that
 // beside the aggregation: the caller runs it before the two big kernels start).
-int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, const int *ok, hipStream_t stream)
+int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, const Gate &gate, hipStream_t stream)
 {
     const int n4 = (dim + 3) / 4;
     if (n4 < 1 || n4 > 16) return fail(MGGX_ELIMIT, "core: dim %d outside 1..64", dim);
@@ -325,13 +325,13 @@ int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, con
     int rc = core_scratch(p, n4, &tab, &partial);
     if (rc) return rc;
     const long long n = (long long)p->core * n4;
-    k_core_stage<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(tab, d_in, p->d_order, p->core, n4, dim, ld_in, ok);
+    k_core_stage<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(tab, d_in, p->d_order, p->core, n4, dim, ld_in, gate);
     MGGX_LAUNCH_CHECK("k_core_stage");
     return MGGX_OK;
 }
 
 // The core block's sums from the staged table into the library's partial rows, on `stream`.
-int run_core_sums(CorePlan *p, int dim, const int *ok, hipStream_t stream)
+int run_core_sums(CorePlan *p, int dim, const Gate &gate, hipStream_t stream)
 {
     const int n4 = (dim + 3) / 4;
     if (n4 < 1 || n4 > 16) return fail(MGGX_ELIMIT, "core: dim %d outside 1..64", dim);
@@ -339,7 +339,7 @@ int run_core_sums(CorePlan *p, int dim, const int *ok, hipStream_t stream)
     int rc = core_scratch(p, n4, &tab, &partial);
     if (rc) return rc;
     switch (n4) {
-#define MGGX_CASE(N) case N: rc = launch_sell<N>(p, tab, partial, ok, stream); break;
+#define MGGX_CASE(N) case N: rc = launch_sell<N>(p, tab, partial, gate, stream); break;
         MGGX_CASE(1) MGGX_CASE(2) MGGX_CASE(3) MGGX_CASE(4) MGGX_CASE(5) MGGX_CASE(6) MGGX_CASE(7) MGGX_CASE(8)
         MGGX_CASE(9) MGGX_CASE(10) MGGX_CASE(11) MGGX_CASE(12) MGGX_CASE(13) MGGX_CASE(14) MGGX_CASE(15) MGGX_CASE(16)
 #undef MGGX_CASE
@@ -349,7 +349,7 @@ int run_core_sums(CorePlan *p, int dim, const int *ok, hipStream_t stream)
 }
 
 // out += scale * (partial rows of the core), then the ReLU if asked for, on `stream`.
-int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, const int *ok, hipStream_t stream)
+int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, const Gate &gate, hipStream_t stream)
 {
     const int n4 = (dim + 3) / 4;
     v4f *tab = nullptr, *partial = nullptr;
@@ -360,12 +360,12 @@ int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const 
     if (dim % 4 == 0 && ld_out % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0) {
         const long long n = nrows * n4;
         k_core_finish4<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(d_out, partial, p->d_rank, p->d_order, d_row_scale, p->rows, n4,
-                                                                                     ld_out, p->core, p->nseg, relu, all_rows, ok);
+                                                                                     ld_out, p->core, p->nseg, relu, all_rows, gate);
     } else {
         const long long n = nrows * dim;
         k_core_finish<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(d_out, reinterpret_cast<const float *>(partial), p->d_rank,
                                                                                     p->d_order, d_row_scale, p->rows, dim, ld_out, p->core, n4,
-                                                                                    p->nseg, relu, all_rows, ok);
+                                                                                    p->nseg, relu, all_rows, gate);
     }
     MGGX_LAUNCH_CHECK("k_core_finish");
     return MGGX_OK;

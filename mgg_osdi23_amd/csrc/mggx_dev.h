@@ -38,17 +38,45 @@ static constexpr unsigned DESC_FIRST = 0x40000000u;  // first partition of its r
 static constexpr unsigned DESC_LAST = 0x80000000u;   // last partition of its row
 static constexpr unsigned DESC_LEN_MASK = 0x3FFFFFFFu;
 
-// Content check of the caller's CSR arrays behind a cached record.  The records are found by device address, and an
+// Content checks of the caller's CSR arrays behind a cached record.  The records are found by device address, and an
 // address says nothing about what is stored there now (arrays rewritten in place, memory freed through another allocator
-// and handed out again).  When a record is made, a small kernel stores a fingerprint of the arrays (their last entries --
-// the edge counts -- and up to 2048 entries of each at a fixed stride); before every later use the same kernel takes the
-// fingerprint again on the call's stream and writes the verdict to *d_ok.  Every kernel of the call reads that word
-// first and returns at once when it is 0, so a stale plan never produces sums or touches memory through stale indices;
-// the mismatch is also written to a host-visible flag, which the next library call reports as MGGX_EINVAL after
-// dropping the record.
+// and handed out again).  Two checks, both on the device, so that a call stays asynchronous:
+//   edge counts (level 1, default)  every kernel of a call first compares the arrays' live edge counts -- ptr_l[rows],
+//                                   ptr_r[rows], two scalar loads -- with the counts its records were built for;
+//   fingerprint (level 2)           before the call's kernels, a one-workgroup kernel takes a fingerprint of the arrays
+//                                   (their last entries and up to 512 entries of each at a fixed stride), compares it
+//                                   with the one stored when the record was made and writes the verdict to a word
+//                                   every kernel of the call reads first (about 8 us per call).
+// A kernel that finds its gate closed returns at once: a stale plan never produces sums or reads through stale indices.
+// The mismatch also goes to a host-visible word; the next library call reports it as MGGX_EINVAL after dropping the
+// records of those arrays.
+struct Gate {
+    const int *ok = nullptr;     // level 2: verdict word of the fingerprint kernel (0 = stale)
+    const int *cnt_l = nullptr;  // level 1: &ptr_l[rows] of the caller's CSR ...
+    const int *cnt_r = nullptr;  //          ... and &ptr_r[rows] (NULL: no remote side)
+    int want_l = 0, want_r = 0;  //          the edge counts the records were built for
+    volatile int *flag = nullptr;
+    int tag = 0;
+};
+
+__device__ __forceinline__ bool gate_closed(const Gate &g)
+{
+    if (g.ok && *g.ok == 0) return true;
+    if (g.cnt_l) {
+        const bool bad = *g.cnt_l != g.want_l || (g.cnt_r && *g.cnt_r != g.want_r);
+        if (bad) {
+            *g.flag = g.tag;
+            return true;
+        }
+    }
+    return false;
+}
+
 struct Guard {
-    const int *arr[4] = {nullptr, nullptr, nullptr, nullptr};
-    long long len[4] = {0, 0, 0, 0};
+    const int *arr[4] = {nullptr, nullptr, nullptr, nullptr};  // fingerprinted arrays ...
+    long long len[4] = {0, 0, 0, 0};                           // ... and their lengths
+    const int *cnt_l = nullptr, *cnt_r = nullptr;              // where the live edge counts are
+    int want_l = 0, want_r = 0;
     unsigned long long *d_fp = nullptr;  // device: [0] fingerprint, [1] verdict word (as int) -- one 16-byte allocation
     int id = 0;                          // reported through the host flag on a mismatch
     bool armed = false;
@@ -135,7 +163,7 @@ struct State {
     char last_kernel[224] = "";
     int gather_addressing = 0;  // 0 = choose per call, 1 = always 64-bit addresses
     // content checks of cached records (Guard)
-    int plan_check = 1;            // 0: checks off (the caller vouches for its arrays)
+    int plan_check = 1;            // 0: checks off (the caller vouches for its arrays), 1: live edge counts, 2: + fingerprint kernel
     volatile int *h_stale = nullptr;  // pinned host word the check kernel writes a record id to on a mismatch
     int next_guard_id = 1;
     // blocks a captured graph may still point at: kept until mggx_release_cached instead of being freed on growth
@@ -157,11 +185,11 @@ int exclusive_scan_i32(const int *d_in, int *d_out, int n, long long *total_host
 
 // True while the library's stream is being captured into a HIP graph.
 bool capturing();
-// Content checks (see Guard).  guard_arm stores the fingerprint of a new record; guard_check takes it again on the stream
-// and returns the device word the call's kernels are gated on (NULL when checks are off); stale_poll reports a mismatch
-// an earlier check found (MGGX_EINVAL, after dropping the record) -- called on entry of every compute call and by mggx_sync.
+// Content checks (see Gate).  guard_arm stores the fingerprint of a new record; guard_check builds the gate of a call from
+// the record (and, at level 2, takes the fingerprint again on the stream); stale_poll reports a mismatch an earlier call
+// found (MGGX_EINVAL, after dropping the records) -- called on entry of every compute call and by mggx_sync.
 int guard_arm(Guard &g);
-int guard_check(Guard &g, const int **d_ok);
+int guard_check(Guard &g, Gate *gate);
 void guard_free(Guard &g);
 int stale_poll();
 int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int rows, int ps, Plan **out);
@@ -178,10 +206,9 @@ void plan_free(Plan *p);
 int forget_pointer(const void *d_ptr);
 int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, CorePlan **out);
 void core_plan_free(CorePlan *p);
-// `ok`: the word the call's kernels are gated on (NULL = no gate), see Guard.
-int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, const int *ok, hipStream_t stream);
-int run_core_sums(CorePlan *p, int dim, const int *ok, hipStream_t stream);
-int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, const int *ok, hipStream_t stream);
+int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, const Gate &gate, hipStream_t stream);
+int run_core_sums(CorePlan *p, int dim, const Gate &gate, hipStream_t stream);
+int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, const Gate &gate, hipStream_t stream);
 // Second stream of the dense-core path (created on first use, default priority) and the two events that fork and join it.
 int core_side_stream(hipStream_t *stream, hipEvent_t *fork, hipEvent_t *join);
 

@@ -318,36 +318,48 @@ __device__ __forceinline__ unsigned long long guard_mix(unsigned long long x)
 
 // Fingerprint of up to four index arrays: the last entry of each and up to GUARD_SAMPLES entries at a fixed stride,
 // each mixed with its position.  arm != 0 stores it; otherwise it is compared with the stored one, the verdict goes to
-// fp[1] (read as int: 1 = unchanged) and, on a mismatch, `tag` to the host-visible flag.
-constexpr int GUARD_SAMPLES = 2048;
+// fp[1] (read as int: 1 = unchanged) and, on a mismatch, `tag` to the host-visible flag.  One workgroup; every thread
+// issues all of its loads before it uses the first, so the kernel costs one trip to memory.
+constexpr int GUARD_SAMPLES = 512;
 __global__ void __launch_bounds__(256) k_guard(const GuardArgs g, unsigned long long *__restrict__ fp, volatile int *host_flag, int tag, int arm)
 {
-    __shared__ unsigned long long red[256];
-    unsigned long long h = 0;
+    __shared__ unsigned long long red[4];
+    constexpr int PER = GUARD_SAMPLES / 256;
+    int v[4][PER + 1];
+    long long at[4][PER + 1];
+#pragma unroll
     for (int a = 0; a < 4; ++a) {
-        const long long n = g.len[a];
-        if (!g.arr[a] || n <= 0) continue;
+        const long long n = g.arr[a] ? g.len[a] : 0;
         const long long samples = n < GUARD_SAMPLES ? n : GUARD_SAMPLES;
-        const long long stride = n / samples;
-        for (long long i = threadIdx.x; i < samples; i += 256) {
-            const long long idx = i * stride;
-            h += guard_mix(((unsigned long long)(a + 1) << 56) ^ ((unsigned long long)idx << 24) ^ (unsigned)g.arr[a][idx]);
+        const long long stride = samples > 0 ? n / samples : 1;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const long long i = (long long)threadIdx.x + 256 * j;
+            at[a][j] = i < samples ? i * stride : -1;
         }
-        if (threadIdx.x == 0) h += guard_mix(((unsigned long long)(a + 5) << 56) ^ ((unsigned long long)n << 24) ^ (unsigned)g.arr[a][n - 1]);
+        at[a][PER] = (threadIdx.x == 0 && n > 0) ? n - 1 : -1;
+#pragma unroll
+        for (int j = 0; j <= PER; ++j) v[a][j] = at[a][j] >= 0 ? __builtin_nontemporal_load(g.arr[a] + at[a][j]) : 0;
     }
-    red[threadIdx.x] = h;
+    unsigned long long h = 0;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+#pragma unroll
+        for (int j = 0; j <= PER; ++j)
+            if (at[a][j] >= 0)
+                h += guard_mix(((unsigned long long)(a + 1 + (j == PER ? 4 : 0)) << 56) ^ ((unsigned long long)at[a][j] << 24) ^ (unsigned)v[a][j]);
+    }
+    for (int o = 32; o > 0; o >>= 1) h += __shfl_xor(h, o, 64);
+    if ((threadIdx.x & 63u) == 0) red[threadIdx.x >> 6] = h;
     __syncthreads();
-    for (int o = 128; o > 0; o >>= 1) {
-        if ((int)threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
-        __syncthreads();
-    }
     if (threadIdx.x == 0) {
+        const unsigned long long total = red[0] + red[1] + red[2] + red[3];
         int *ok = reinterpret_cast<int *>(fp + 1);
         if (arm) {
-            fp[0] = red[0];
+            fp[0] = total;
             *ok = 1;
         } else {
-            const int same = fp[0] == red[0];
+            const int same = fp[0] == total;
             *ok = same;
             if (!same) *host_flag = tag;
         }
@@ -371,7 +383,7 @@ bool capturing()
     return st == hipStreamCaptureStatusActive;
 }
 
-static int guard_launch(Guard &g, int arm)
+static int host_flag_init()
 {
     State &s = state();
     if (!s.h_stale) {
@@ -380,6 +392,12 @@ static int guard_launch(Guard &g, int arm)
         s.h_stale = static_cast<volatile int *>(p);
         *s.h_stale = 0;
     }
+    return MGGX_OK;
+}
+
+static int guard_launch(Guard &g, int arm)
+{
+    State &s = state();
     GuardArgs a;
     for (int i = 0; i < 4; ++i) {
         a.arr[i] = g.arr[i];
@@ -393,24 +411,35 @@ static int guard_launch(Guard &g, int arm)
 int guard_arm(Guard &g)
 {
     State &s = state();
+    int rc = host_flag_init();
+    if (rc) return rc;
     if (!g.d_fp) {
         if (capturing()) return fail(MGGX_EINVAL, "first use of these CSR arrays inside a stream capture: call once outside the capture first");
         if (hipMalloc((void **)&g.d_fp, 16) != hipSuccess) return fail(MGGX_ENOMEM, "content check: fingerprint");
     }
     g.id = s.next_guard_id++;
     if (s.next_guard_id > 0x3fffffff) s.next_guard_id = 1;
-    const int rc = guard_launch(g, 1);
+    rc = guard_launch(g, 1);
     g.armed = rc == MGGX_OK;
     return rc;
 }
 
-int guard_check(Guard &g, const int **d_ok)
+int guard_check(Guard &g, Gate *gate)
 {
-    *d_ok = nullptr;
-    if (!state().plan_check || !g.armed) return MGGX_OK;
-    const int rc = guard_launch(g, 0);
-    if (rc) return rc;
-    *d_ok = g.ok();
+    State &s = state();
+    *gate = Gate{};
+    if (!s.plan_check || !g.armed) return MGGX_OK;
+    gate->cnt_l = g.cnt_l;
+    gate->cnt_r = g.cnt_r;
+    gate->want_l = g.want_l;
+    gate->want_r = g.want_r;
+    gate->flag = s.h_stale;
+    gate->tag = g.id;
+    if (s.plan_check >= 2) {
+        const int rc = guard_launch(g, 0);
+        if (rc) return rc;
+        gate->ok = g.ok();
+    }
     return MGGX_OK;
 }
 
@@ -685,6 +714,8 @@ int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_
         p->guard.len[1] = num_parts;
         p->guard.arr[2] = d_part2node;
         p->guard.len[2] = num_parts;
+        p->guard.cnt_l = d_row_ptr + rows;
+        p->guard.want_l = end;
         rc = guard_arm(p->guard);
     } while (0);
     if (rc) {
@@ -833,6 +864,10 @@ int graph_info(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_l, const
         r.guard.len[2] = g.nnz_l;
         r.guard.arr[3] = g.nnz_r > 0 ? d_col_r : nullptr;
         r.guard.len[3] = g.nnz_r;
+        r.guard.cnt_l = d_ptr_l + rows;
+        r.guard.want_l = ends[0];
+        r.guard.cnt_r = d_ptr_r ? d_ptr_r + rows : nullptr;
+        r.guard.want_r = ends[1];
         const int rc = guard_arm(r.guard);
         if (rc) {
             guard_free(r.guard);

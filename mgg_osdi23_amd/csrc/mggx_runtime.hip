@@ -242,7 +242,7 @@ MGGX_EXPORT int mggx_release_cached(void)
 
 MGGX_EXPORT int mggx_set_plan_check(int on)
 {
-    if (on != 0 && on != 1) return fail(MGGX_EINVAL, "set_plan_check: %d", on);
+    if (on < 0 || on > 2) return fail(MGGX_EINVAL, "set_plan_check: level %d (0, 1 or 2)", on);
     state().plan_check = on;
     return MGGX_OK;
 }
@@ -346,7 +346,73 @@ __global__ void __launch_bounds__(256) k_gather_probe(float *__restrict__ sink, 
 
 constexpr int PROBE_BLOCKS = 1024;
 
+// Yardstick for the dense-core kernel's LDS reads: every lane adds N4 16-byte pieces of an LDS tile row at a
+// pseudo-random column per step (tile [N4][257] like the core kernel's, 4 wavefronts per workgroup), four steps per
+// index draw; no global memory traffic inside the loop.
+typedef float probe_v4f __attribute__((ext_vector_type(4)));
+
+template <int N4>
+__global__ void __launch_bounds__(256) k_lds_probe(float *__restrict__ sink, int iters, unsigned seed)
+{
+    constexpr int TC = 256, TP = TC + 1;
+    extern __shared__ probe_v4f probe_tile[];
+    for (int i = (int)threadIdx.x; i < N4 * TP; i += 256) probe_tile[i] = (probe_v4f){1.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+    unsigned x = ((unsigned)blockIdx.x * 256u + threadIdx.x + 1u) * 2654435761u ^ seed;
+    probe_v4f acc[N4];
+#pragma unroll
+    for (int s = 0; s < N4; ++s) acc[s] = (probe_v4f){0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < iters; ++it) {
+        x = x * 1664525u + 1013904223u;
+        const unsigned r = x ^ (x >> 13);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const probe_v4f *q = probe_tile + ((r >> (8 * j)) & 255u);
+#pragma unroll
+            for (int s = 0; s < N4; ++s) acc[s] += q[s * TP];
+        }
+    }
+    probe_v4f t = acc[0];
+#pragma unroll
+    for (int s = 1; s < N4; ++s) t += acc[s];
+    sink[(size_t)blockIdx.x * 256 + threadIdx.x] = t.x + t.y + t.z + t.w;
+}
+
+template <int N4>
+int launch_lds_probe(float *sink, int iters, unsigned seed, hipStream_t stream)
+{
+    const size_t lds = (size_t)N4 * 257 * sizeof(probe_v4f);
+    static bool raised = false;
+    if (lds > 48 * 1024 && !raised) {
+        MGGX_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_lds_probe<N4>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        raised = true;
+    }
+    k_lds_probe<N4><<<dim3(PROBE_BLOCKS), dim3(256), lds, stream>>>(sink, iters, seed);
+    MGGX_LAUNCH_CHECK("k_lds_probe");
+    return MGGX_OK;
+}
+
 }  // namespace
+
+MGGX_EXPORT int mggx_lds_probe(float *d_sink, size_t row_bytes, int64_t n_reads, unsigned seed, int64_t *n_done)
+{
+    if (!d_sink || row_bytes < 16 || row_bytes > 256 || (row_bytes % 16) || n_reads < 1)
+        return fail(MGGX_EINVAL, "lds_probe: NULL sink, or rows not 16..256 bytes in 16-byte pieces");
+    const long long per_iter = (long long)PROBE_BLOCKS * 256 * 4;
+    const long long iters = (n_reads + per_iter - 1) / per_iter;
+    if (iters > 0x7fffffffLL) return fail(MGGX_ELIMIT, "lds_probe: too many reads");
+    int rc;
+    switch ((int)(row_bytes / 16)) {
+#define MGGX_CASE(N) case N: rc = launch_lds_probe<N>(d_sink, (int)iters, seed, state().stream); break;
+        MGGX_CASE(1) MGGX_CASE(2) MGGX_CASE(3) MGGX_CASE(4) MGGX_CASE(5) MGGX_CASE(6) MGGX_CASE(7) MGGX_CASE(8)
+        MGGX_CASE(9) MGGX_CASE(10) MGGX_CASE(11) MGGX_CASE(12) MGGX_CASE(13) MGGX_CASE(14) MGGX_CASE(15) MGGX_CASE(16)
+#undef MGGX_CASE
+        default: rc = fail(MGGX_EINVAL, "lds_probe: row of %zu bytes", row_bytes);
+    }
+    if (rc) return rc;
+    if (n_done) *n_done = iters * per_iter;
+    return MGGX_OK;
+}
 
 MGGX_EXPORT int mggx_gather_probe(float *d_sink, const void *d_table, int64_t rows, size_t ld_bytes, size_t row_bytes,
                                   int64_t n_gathers, unsigned seed, int64_t *n_done)

@@ -61,7 +61,7 @@ EXPORTS = [
     "mggx_release_cached", "mggx_forget", "mggx_set_plan_check", "mggx_cache_stats", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_core_layout_build", "mggx_core_layout_fetch", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
     "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_compact_remote_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_sag_parts_static", "mggx_mlp2_xw", "mggx_spmm",
-    "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_gather_probe", "mggx_gather_rows", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
+    "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_gather_probe", "mggx_lds_probe", "mggx_gather_rows", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
 ]
 
 
@@ -302,9 +302,10 @@ def release_cached() -> None:
     _pinned.clear()
 
 
-def set_plan_check(on: bool) -> None:
-    """Content checks of cached plans against the caller's CSR arrays (on by default)."""
-    _check(lib().mggx_set_plan_check(int(on)))
+def set_plan_check(level: int) -> None:
+    """Content checks of cached plans against the caller's CSR arrays: 0 = off, 1 = live edge counts inside every kernel
+    (default), 2 = also a fingerprint kernel before every call."""
+    _check(lib().mggx_set_plan_check(int(level)))
 
 
 def cache_stats() -> dict:
@@ -480,6 +481,13 @@ def gather_probe(sink, table, rows: int, ld_bytes: int, row_bytes: int, n_gather
     done = C.c_int64(0)
     _check(lib().mggx_gather_probe(_dptr(sink), _dptr(table), C.c_int64(rows), C.c_size_t(ld_bytes), C.c_size_t(row_bytes),
                                    C.c_int64(n_gathers), C.c_uint(seed), C.byref(done)))
+    return int(done.value)
+
+
+def lds_probe(sink, row_bytes: int, n_reads: int, seed: int = 1) -> int:
+    """Random row reads from an LDS tile laid out like the dense-core kernel's; returns the number issued."""
+    done = C.c_int64(0)
+    _check(lib().mggx_lds_probe(_dptr(sink), C.c_size_t(row_bytes), C.c_int64(n_reads), C.c_uint(seed), C.byref(done)))
     return int(done.value)
 
 

@@ -23,8 +23,16 @@ def _want(x, ptr, col, V, dim):
     return want, mag
 
 
+@pytest.fixture(params=[1, 2])
+def check_level(gpu, request):
+    """Both levels of the content check: live edge counts inside the kernels; the fingerprint kernel on top."""
+    gpu.set_plan_check(request.param)
+    yield request.param
+    gpu.set_plan_check(1)
+
+
 @pytest.mark.parametrize("core_rows", [-1, 1024])
-def test_csr_rewritten_in_place_without_forget(gpu, core_rows):
+def test_csr_rewritten_in_place_without_forget(gpu, core_rows, check_level):
     """A different graph written into the same device arrays, and no mggx_forget: the cached plan (and dense-core plan)
     no longer fits.  The call must give an error or the right answer, never a sum through the stale plan."""
     import torch
@@ -68,7 +76,42 @@ def test_csr_rewritten_in_place_without_forget(gpu, core_rows):
     gpu.forget(d_ptr)
 
 
-def test_explicit_partition_arrays_rewritten_in_place(gpu):
+def test_same_edge_count_other_graph_needs_the_fingerprint(gpu):
+    """Level 2 also catches a rewrite that keeps the edge count (here: the rows of the graph rotated by one)."""
+    import torch
+    V, dim = 3000, 16
+    ptr, col = gpu.gen_rmat(12, V, 50_000, seed=11)
+    deg = np.diff(ptr)
+    deg_b = np.roll(deg, 1)
+    ptr_b = np.zeros(V + 1, np.int32)
+    ptr_b[1:] = np.cumsum(deg_b)
+    assert ptr_b[-1] == ptr[-1] and not np.array_equal(ptr_b, ptr)
+    x = gpu.fill_normal((V, dim), seed=3)
+    d_x, d_ptr, d_col = to_dev(x), to_dev(ptr), to_dev(col)
+    zp, zc = torch.zeros(V + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    out = torch.empty(V, dim, device="cuda")
+    call = lambda: gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, zp, zc, 0, V, dim, V, 0, 16, 4, 2)
+    gpu.set_plan_check(2)
+    try:
+        call()
+        gpu.sync()
+        d_ptr.copy_(torch.from_numpy(ptr_b))
+        torch.cuda.synchronize()
+        out.fill_(-7.0)
+        with pytest.raises(gpu.MggxError, match="changed"):
+            call()
+            gpu.sync()
+        assert bool((out == -7.0).all())
+        call()
+        gpu.sync()
+        want, mag = _want(x, ptr_b, col, V, dim)
+        assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "rows rotated")
+    finally:
+        gpu.set_plan_check(1)
+        gpu.forget(d_ptr)
+
+
+def test_explicit_partition_arrays_rewritten_in_place(gpu, check_level):
     import torch
     V, dim, ps = 4000, 16, 8
     ptr_a, col_a = gpu.gen_rmat(12, V, 60_000, seed=4)
