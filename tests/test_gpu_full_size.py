@@ -1,0 +1,186 @@
+"""Parity at the full sizes of the benchmark configurations that the smaller tests do not reach: the 2.45 M-node GIN
+graph at width 64 with the fused two-layer update (configs[2]), the 13.9 M-row bf16 width-128 share with its 28 GB
+remote table (configs[4]: element offsets beyond 2^31, ids beyond 2^24, so the 64-bit address path), and the whole
+2-layer GCN forward at 233 K nodes (configs[1]).  Inputs are the benchmark's own seeded graphs.  The oracle checks
+sampled rows (the heaviest and a random set) in double precision; closed forms and bit-identity cover every row."""
+import numpy as np
+import pytest
+
+from oracle import orc
+from tests.util import BF16_TOL, FP32_TOL, assert_close_to_oracle, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def zeros_i32(n=1):
+    import torch
+    return torch.zeros(n, dtype=torch.int32, device="cuda")
+
+
+def sample_rows(deg, n_random, seed=0):
+    rng = np.random.default_rng(seed)
+    R = len(deg)
+    return np.unique(np.concatenate([np.argsort(deg)[-40:], rng.integers(0, R, n_random), [0, R - 1]])).astype(np.int32)
+
+
+def test_full_size_gin_graph_layer(gpu):
+    """configs[2]: V = 2.45 M, ~123 M nnz, width 64, eps 0.  ones -> deg + 1 exactly on every row; sampled rows of the
+    aggregation and of one whole layer (aggregate, then the fused 64->64->64 update with ReLU between) against the
+    double-precision oracle; with the dense core from LDS and without it."""
+    import torch
+    V, dim, eps = 2_450_000, 64, 0.0
+    ptr, col = gpu.gen_rmat(22, V, 64_000_000, seed=3)
+    assert 118_000_000 < len(col) < 128_000_000
+    deg = np.diff(ptr)
+    x = gpu.fill_normal((V, dim), seed=1)
+    wa, wb = gpu.glorot(dim, dim, seed=10) * 0.2, gpu.glorot(dim, dim, seed=30) * 0.2
+    d_ptr, d_col, zp, zc = to_dev(ptr), to_dev(col), zeros_i32(V + 1), zeros_i32()
+    d_x, d_wa, d_wb = to_dev(x), to_dev(wa), to_dev(wb)
+    rows = sample_rows(deg, 400)
+    args = (rows, x, x, ptr, col, None, None, 0, V, dim, V)
+    want = orc.sag_np_div_rows(*args, flags=orc.GIN, eps=eps)
+    mag = orc.sag_np_div_rows(*args, flags=orc.GIN, eps=eps, abs_sum=True)
+    # the layer on the sampled rows, in double precision, from the oracle's aggregation
+    t = np.maximum(want.astype(np.float64) @ wa.astype(np.float64), 0.0)
+    y_want = t @ wb.astype(np.float64)
+    y_mag = (mag.astype(np.float64) @ np.abs(wa).astype(np.float64)) @ np.abs(wb).astype(np.float64)
+    ones = torch.ones(V, dim, device="cuda")
+    H = torch.empty(V, dim, device="cuda")
+    Y = torch.empty(V, dim, device="cuda")
+    idx = torch.from_numpy(rows.astype(np.int64)).cuda()
+    for core_rows, wpb, dist in ((-1, 16, 2), (40960, 8, 4)):
+        H.fill_(-5.0)
+        gpu.mgg_GIN_np_div(H, ones, d_ptr, d_col, zp, zc, 0, V, dim, V, 0, 16, wpb, dist, eps, core_rows=core_rows)
+        gpu.sync()
+        assert ("core=40960" in gpu.last_agg_kernel()) == (core_rows > 0)
+        h = H.cpu().numpy()
+        assert np.array_equal(h[:, 0], (deg + 1).astype(np.float32)) and np.array_equal(h[:, 63], h[:, 0])
+        gpu.mgg_GIN_np_div(H, d_x, d_ptr, d_col, zp, zc, 0, V, dim, V, 0, 16, wpb, dist, eps, core_rows=core_rows)
+        gpu.mlp2_forward(Y, H, d_wa, d_wb, V, dim, dim, dim, relu_mid=True)
+        gpu.sync()
+        assert_close_to_oracle(H[idx].cpu().numpy(), want, mag, FP32_TOL, "GIN aggregation, core_rows=%d" % core_rows)
+        # three chained fp32 stages (sum, two products): 3 x the single-stage bound on the magnitudes flowing through
+        assert_close_to_oracle(Y[idx].cpu().numpy(), y_want, y_mag, 3 * FP32_TOL, "GIN layer, core_rows=%d" % core_rows)
+    gpu.forget(d_ptr)
+
+
+def test_full_size_large_share_bf16(gpu):
+    """configs[4]: rank 0's 1/8 share of a 111 M-node scrambled RMAT graph: 13.9 M rows, ~209 M neighbors, bf16 width-128
+    tables -- 3.6 GB local, 28 GB remote indexed by global id (byte offsets far beyond 2^31, ids beyond 2^24: the 64-bit
+    address path) -- fp32 accumulation, then the 128x128 update on the bf16 matrix cores."""
+    import torch
+    V, dim, n = 111_000_000, 128, 8
+    npp, lb, ub = gpu.range_partition(V, n, 0)
+    ptr, col = gpu.gen_rmat(27, V, 790_000_000, seed=5, scramble=True, row_lo=lb, row_hi=ub)
+    lp, rp, lc, rc = gpu.split_CSR(ptr, col, lb, ub)
+    del ptr, col
+    R = ub - lb
+    assert R > 13_000_000 and len(lc) + len(rc) > 190_000_000 and int(rc.max()) >= (1 << 24)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    d_xr = torch.randn(n * npp, dim, device="cuda", dtype=torch.bfloat16, generator=gen)
+    assert d_xr.numel() * 2 > (1 << 34)
+    d_xl = d_xr[lb:ub].clone()
+    d = [to_dev(a) for a in (lp, lc, rp, rc)]
+    out = torch.full((R, dim), -2.0, device="cuda")
+    gpu.mgg_SAG_np_div(out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, 16, 4, 16, input_remote=d_xr)
+    gpu.sync()
+    assert ",2,0>" in gpu.last_agg_kernel()  # bf16 rows, 64-bit addresses
+
+    # the sampled rows as a small problem of their own: the feature rows they touch, ids renumbered
+    deg = np.diff(lp) + np.diff(rp)
+    rows = sample_rows(deg, 1500)
+    nbrs = [np.concatenate([lc[lp[r]:lp[r + 1]], rc[rp[r]:rp[r + 1]]]) for r in rows]
+    need = np.unique(np.concatenate(nbrs))
+    x_small = d_xr[torch.from_numpy(need.astype(np.int64)).cuda()].float().cpu().numpy()  # bf16 values, exact in fp32
+    sp = np.zeros(len(rows) + 1, np.int32)
+    sp[1:] = np.cumsum([len(v) for v in nbrs])
+    cc = np.searchsorted(need, np.concatenate(nbrs)).astype(np.int32)
+    m = len(rows)
+    zl, zc_ = np.zeros(m + 1, np.int32), np.zeros(0, np.int32)
+    dummy = np.zeros((m, dim), np.float32)
+    sub = (np.arange(m, dtype=np.int32), dummy, x_small, zl, zc_, sp, cc, 0, m, dim, m)
+    want = orc.sag_np_div_rows(*sub)
+    mag = orc.sag_np_div_rows(*sub, abs_sum=True)
+    idx = torch.from_numpy(rows.astype(np.int64)).cuda()
+    got = out[idx].cpu().numpy()
+    # fp32 accumulation of exactly representable inputs: the fp32 bound, far inside the 2e-2 the configuration allows
+    assert_close_to_oracle(got, want, mag, FP32_TOL, "bf16 share, sampled rows")
+    assert_close_to_oracle(got, want, mag, BF16_TOL, "bf16 share, sampled rows (configuration tolerance)")
+
+    # compact staging of the remote rows: same sums bit for bit (same order of summation, other addresses)
+    d_rcc, d_ids = gpu.compact_remote_device(d[3], len(rc))
+    assert 10_000_000 < len(d_ids) < 30_000_000
+    assert torch.equal(d_ids[d_rcc.long()], d[3])  # the round trip fetch_ids[compact] == remote_col
+    d_xc = torch.empty(len(d_ids), dim, device="cuda", dtype=torch.bfloat16)
+    gpu.gather_rows(d_xc, d_xr, d_ids, len(d_ids), dim * 2)
+    out2 = torch.full((R, dim), -3.0, device="cuda")
+    gpu.mgg_SAG_np_div(out2, d_xl, d[0], d[1], d[2], d_rcc, lb, ub, dim, npp, 0, 16, 4, 16, input_remote=d_xc)
+    gpu.sync()
+    assert torch.equal(out, out2), "compact staging differs from the table indexed by global id"
+    del out2, d_xc
+
+    # size-independent: all-ones tables -> the degree, exactly, on every row (the remote table is reused in place)
+    del d_xl
+    d_xr.fill_(1.0)
+    ones_l = torch.ones(R, dim, device="cuda", dtype=torch.bfloat16)
+    chk = torch.empty(R, dim, device="cuda")
+    gpu.mgg_SAG_np_div(chk, ones_l, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, 16, 8, 4, input_remote=d_xr)
+    gpu.sync()
+    c = chk.cpu().numpy()
+    assert np.array_equal(c[:, 0], deg.astype(np.float32)) and np.array_equal(c[:, dim - 1], c[:, 0])
+    del chk, ones_l
+
+    # the update that follows: out (fp32, rounded to bf16 in the kernel) x W (bf16), fp32 accumulation, bf16 result
+    W = gpu.glorot(dim, dim, seed=6)
+    d_W = to_dev(W).to(torch.bfloat16)
+    nxt = torch.empty(R, dim, device="cuda", dtype=torch.bfloat16)
+    gpu.dense_forward_bf16(nxt, out, d_W, R, dim, dim)
+    gpu.sync()
+    xb = out[idx].to(torch.bfloat16).double().cpu().numpy()  # round to nearest even, as the kernel does
+    wb = d_W.double().cpu().numpy()
+    y_want = xb @ wb
+    y_mag = np.abs(xb) @ np.abs(wb)
+    # fp32 accumulation of exact products, then one rounding to bf16 (2^-9 relative)
+    assert_close_to_oracle(nxt[idx].float().cpu().numpy(), y_want, y_mag + np.abs(y_want) * 400, FP32_TOL, "128x128 bf16 update")
+    for t in d:
+        gpu.forget(t)
+
+
+@pytest.mark.parametrize("core_rows", [-1, 40960])
+def test_full_size_gcn_forward_end_to_end(gpu, core_rows):
+    """configs[1] end to end: 233 K nodes, ~228 M nnz, 602 -> 16 -> 41 through the softmax, in the benchmark's device
+    layout (41-wide layer at width 44, row pitch 48), against the oracle's whole forward in double precision."""
+    import torch
+    V, in_dim, hidden, out_dim = 233_000, 602, 16, 41
+    ptr, col = gpu.gen_rmat(18, V, 216_000_000, seed=42)
+    X = gpu.fill_normal((V, in_dim), seed=1)
+    W1, W2 = gpu.glorot(in_dim, hidden, seed=2), gpu.glorot(hidden, out_dim, seed=3)
+    s = (1.0 / np.sqrt(np.maximum(np.diff(ptr), 1))).astype(np.float32)
+    ldo, pitch = 44, 48
+    W2p = np.zeros((hidden, ldo), np.float32)
+    W2p[:, :out_dim] = W2
+    d_ptr, d_col, zp, zc = to_dev(ptr), to_dev(col), zeros_i32(V + 1), zeros_i32()
+    d_s = to_dev(s)
+    Y1, H1 = torch.empty(V, hidden, device="cuda"), torch.empty(V, hidden, device="cuda")
+    Y2, H2 = torch.zeros(V, pitch, device="cuda"), torch.zeros(V, pitch, device="cuda")
+    P = torch.empty(V, out_dim, device="cuda")
+    gpu.dense_forward(Y1, to_dev(X), to_dev(W1), V, in_dim, hidden, row_scale=d_s)
+    gpu.mgg_SAG_np_div(H1, Y1, d_ptr, d_col, zp, zc, 0, V, hidden, V, 0, 16, 4, 4, row_scale_out=d_s, core_rows=core_rows)
+    gpu.dense_forward(Y2, H1, to_dev(W2p), V, hidden, ldo, row_scale=d_s, ld_out=pitch)
+    gpu.mgg_SAG_np_div(H2, Y2, d_ptr, d_col, zp, zc, 0, V, ldo, V, 0, 16, 4, 16, row_scale_out=d_s, core_rows=core_rows, ld_in=pitch,
+                       ld_out=pitch)
+    gpu.softmax_forward(P, H2, V, out_dim, ld_in=pitch)
+    gpu.sync()
+    assert ("core=40960" in gpu.last_agg_kernel()) == (core_rows > 0)
+    P_ref, H2_ref, H1_ref = orc.gcn2_forward(X, W1, W2, ptr, col, None, None, 0, V, V, rs=s, f64=True)
+
+    def rel(a, b):  # per row, against the largest magnitude flowing through that row
+        return float(np.max(np.abs(a - b).max(1) / (np.abs(b).max(1) + 1e-30)))
+    assert rel(H1.cpu().numpy(), H1_ref) < 2e-5
+    assert rel(H2.cpu().numpy()[:, :out_dim], H2_ref) < 5e-5
+    p = P.cpu().numpy()
+    assert np.abs(p - P_ref).max() < 1e-5
+    assert np.allclose(p.sum(1), 1.0, atol=1e-5)
+    assert np.all(H2.cpu().numpy()[:, out_dim:ldo] == 0.0)
+    gpu.forget(d_ptr)
