@@ -20,7 +20,8 @@ import sys
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
 from oracle import orc  # noqa: E402
 
 
@@ -97,6 +98,24 @@ def main():
             rec["parts"].append({"ps": ps, "local": [digest(x) for x in pl], "remote": [digest(x) for x in pr]})
         big["split"].append(rec)
     out["large"].append(big)
+
+    # the graph of the first benchmark configuration itself: Erdos-Renyi, 4096 nodes, average degree 16, self loops,
+    # seed 0, from the library's generator (its digests pin the generator too); nGPU = 1 and rank 0 of 8, ps = 16
+    from mgg_osdi23_amd import host
+    ptr, col = host.gen_er(4096, 16.0, seed=0)
+    cfg = {"name": "config1_er_4096", "generator": "gen_er", "num_nodes": 4096, "avg_deg": 16.0, "seed": 0, "ptr": digest(ptr),
+           "col": digest(col), "split": [], "parts": []}
+    for num_gpus, pe in ((1, 0), (8, 0)):
+        npp = (4096 + num_gpus - 1) // num_gpus
+        lb, ub = npp * pe, min(npp * pe + npp, 4096)
+        lp, rp, lc, rc = orc.ref_split_csr(ptr, col, lb, ub)
+        rec = {"lb": lb, "ub": ub, "local_ptr": digest(lp), "remote_ptr": digest(rp), "local_col": digest(lc),
+               "remote_col": digest(rc), "parts": []}
+        pl = orc.ref_build_part(lp, ub - lb, 16)
+        pr = orc.ref_build_part(rp, ub - lb, 16)
+        rec["parts"].append({"ps": 16, "local": [digest(x) for x in pl], "remote": [digest(x) for x in pr]})
+        cfg["split"].append(rec)
+    out["large"].append(cfg)
 
     # SAG_ref (utils.cuh:71-86) on a small seeded case, floats stored exactly as hex
     rng = np.random.default_rng(7)

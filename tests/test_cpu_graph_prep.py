@@ -69,10 +69,16 @@ def test_build_part_matches_reference_golden(golden):
                     assert same(g, w), (case["name"], rec["ps"], name, impl.__module__)
 
 
-def test_large_case_digests(golden):
-    big = golden["large"][0]
-    rng = np.random.default_rng(big["seed"])
-    ptr, col = random_csr(rng, 4096, big["avg_deg"])
+@pytest.mark.parametrize("which", [0, 1])
+def test_large_case_digests(golden, which):
+    """4096-node cases as SHA-256 digests of every array the reference's split_CSR / build_part produced: a numpy-generated
+    graph, and the first benchmark configuration's own graph (Erdos-Renyi, average degree 16, seed 0, nGPU = 1 and 8)."""
+    big = golden["large"][which]
+    if big.get("generator") == "gen_er":
+        ptr, col = host.gen_er(big["num_nodes"], big["avg_deg"], seed=big["seed"])
+    else:
+        rng = np.random.default_rng(big["seed"])
+        ptr, col = random_csr(rng, 4096, big["avg_deg"])
     assert sha(ptr) == big["ptr"]["sha256"] and sha(col) == big["col"]["sha256"], "fixture input regenerated differently"
     for rec in big["split"]:
         for impl in (orc.split_csr, host.split_CSR):
