@@ -146,6 +146,14 @@ int mggx_core_layout_build(const int *ptr, const int *col, int rows, int lb, int
 int mggx_core_layout_fetch(void *handle, int *order, int *rank, unsigned *blk_off, unsigned short *idx, int *rem_ptr,
                            int *rem_col);
 
+/* The same layout as the aggregation itself builds it: on the GPU, from the device copy of the CSR (a stable radix sort
+ * by degree, a counting pass, two prefix sums, a fill pass; only scalars travel to the host), bit-identical to
+ * mggx_core_layout_build.  Builds (or finds) the cached dense-core plan of (d_ptr, d_col, rows, lb, core_rows), returns
+ * sizes[5] as above and copies the arrays that are not NULL to host memory: call once with NULL arrays for the sizes.
+ * Synchronises. */
+int mggx_core_layout_device(const int *d_ptr, const int *d_col, int rows, int lb, int core_rows, int64_t *sizes, int *order,
+                            int *rank, unsigned *blk_off, unsigned short *idx, int *rem_ptr, int *rem_col);
+
 /* build_part<int> (include/neighbor_utils.cuh:411-460).  part_ptr has
  * num_parts+1 entries, part2node num_parts, node2part num_nodes+2 (the
  * reference's layout).  compat != 0 reproduces the reference's terminal entry
@@ -251,8 +259,7 @@ typedef struct mggx_agg_knobs {
  * multiple of 512) are ranked by degree; the edges among them leave the CSR and are summed from LDS -- the feature rows
  * of 256 core columns at a time staged with whole-line reads, one lane per core row walking an index list -- and the
  * rest of the CSR runs as usual on top.  Pays on graphs whose high-degree rows hold most edges among themselves; its
- * plan is built on the host (the CSR is copied back once), so by rule it is off and mggx_sag_np_div_tune turns it on
- * where it measures faster.  The core block runs on a second stream of the library's, forked from and joined to the
+ * plan is built on the GPU on first use (milliseconds).  The core block runs on a second stream of the library's, forked from and joined to the
  * caller's stream by events inside the call (LDS-bound work beside cache-bound work).  Same result up to summation order.
  * The partition plan of (d_ptr_l, d_ptr_r, d_col_r, rows, ps) -- and d_col_l for the column-blocked order -- is built on first use and
  * cached by pointer identity: the CSR arrays must not be rewritten in place or freed
@@ -359,6 +366,9 @@ int mggx_cast_f32_to_bf16(void *d_dst, const float *d_src, int64_t n);
 /* Plain device copy kernel of n bytes (n % 16 == 0): the known-size yardstick the
  * profiler's HBM byte counters are scaled against. */
 int mggx_copy_bytes(void *d_dst, const void *d_src, size_t n);
+/* The same copy as one workgroup per 16 KiB with non-temporal loads and stores, four loads in flight per thread: a
+ * second copy kernel, so the copy ceiling quoted beside the bandwidth-bound kernels does not rest on one variant. */
+int mggx_copy_bytes_nt(void *d_dst, const void *d_src, size_t n);
 
 /* Yardstick for row gathers (no counterpart in the reference): at least n_gathers loads of row_bytes bytes (16..256, in
  * 16-byte pieces) from rows at pseudo-random indices of a table of `rows` rows with a stride of ld_bytes, eight loads in

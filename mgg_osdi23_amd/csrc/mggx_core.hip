@@ -11,6 +11,8 @@
 #include <chrono>
 #include <new>
 
+#include <rocprim/device/device_radix_sort.hpp>
+
 #include "mggx_dev.h"
 
 namespace mggx {
@@ -145,6 +147,139 @@ __global__ void __launch_bounds__(256) k_core_finish4(float *__restrict__ out, c
     *o = t;
 }
 
+// ---- the plan, built on the GPU (same arrays, bit for bit, as core_layout_build makes on the host) ----
+
+__global__ void __launch_bounds__(256) k_core_deg(const int *__restrict__ ptr, int rows, int *__restrict__ deg, int *__restrict__ ids)
+{
+    const int v = blockIdx.x * 256 + threadIdx.x;
+    if (v >= rows) return;
+    deg[v] = ptr[v + 1] - ptr[v];
+    ids[v] = v;
+}
+
+// sorted = row ids by falling degree, ties by rising id: the first `core` are the core, in rank order
+__global__ void __launch_bounds__(256) k_core_rank(const int *__restrict__ sorted, int rows, int core, int *__restrict__ order, int *__restrict__ rank)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows) return;
+    const int v = sorted[i];
+    if (i < core) {
+        order[i] = v;
+        rank[v] = i;
+    } else {
+        rank[v] = -1;
+    }
+}
+
+constexpr int BUILD_WAVES = 4;  // rows per workgroup of the two passes below (one wavefront each)
+
+// Pass 1, one wavefront per row: how many neighbors of a core row fall into each tile of core columns (cnt, one
+// 16-bit count per core row and tile), and how many neighbors every row keeps in the remaining CSR.  flag |= 1 on a
+// neighbor id outside [lb, lb + rows) or a list longer than 65534.
+__global__ void __launch_bounds__(BUILD_WAVES * 64) k_core_count(const int *__restrict__ ptr, const int *__restrict__ col,
+                                                                 const int *__restrict__ rank, int rows, int lb, int ntiles, int tc,
+                                                                 unsigned short *__restrict__ cnt, int *__restrict__ keep, int *__restrict__ flag)
+{
+    extern __shared__ int hist_all[];  // [BUILD_WAVES][ntiles]
+    const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
+    int *hist = hist_all + (size_t)wave * ntiles;
+    for (long long v = (long long)blockIdx.x * BUILD_WAVES + wave; v < rows; v += (long long)gridDim.x * BUILD_WAVES) {
+        const int i = rank[v];
+        const int beg = ptr[v], end = ptr[v + 1];
+        if (i >= 0)
+            for (int t = lane; t < ntiles; t += 64) hist[t] = 0;
+        int kept = 0, bad = 0;
+        for (int e = beg + lane; e < end; e += 64) {
+            const int u = col[e] - lb;
+            if (u < 0 || u >= rows) {
+                bad = 1;
+                ++kept;
+                continue;
+            }
+            const int j = rank[u];
+            if (i >= 0 && j >= 0) atomicAdd(&hist[j / tc], 1);
+            else ++kept;
+        }
+        for (int o = 32; o > 0; o >>= 1) kept += __shfl_xor(kept, o, 64);
+        if (i >= 0) {
+            for (int t = lane; t < ntiles; t += 64) {
+                const int c = hist[t];
+                if (c > 0xFFFE) bad = 1;
+                cnt[(size_t)i * ntiles + t] = (unsigned short)(c > 0xFFFE ? 0xFFFE : c);
+            }
+        }
+        if (lane == 0) keep[v] = kept;
+        if (bad) *flag = 1;
+    }
+}
+
+// chunks[g * ntiles + t] = list positions of block (slice g, tile t) in units of 4: the longest of the slice's 64 lists, rounded up
+__global__ void __launch_bounds__(256) k_core_widths(const unsigned short *__restrict__ cnt, int nslices, int ntiles, int *__restrict__ chunks)
+{
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long long)nslices * ntiles) return;
+    const int g = (int)(idx / ntiles), t = (int)(idx % ntiles);
+    int w = 0;
+    for (int l = 0; l < 64; ++l) w = max(w, (int)cnt[(size_t)(g * 64 + l) * ntiles + t]);
+    chunks[idx] = (w + 3) / 4;
+}
+
+// Pass 2, one wavefront per row, 64 neighbors at a time in edge order: neighbors that stay go to the remaining CSR (order
+// kept); a core row's core neighbors go to the list of their tile, the k-th of a tile (in edge order) to list position k.
+// Inside a group of 64 every lane counts the lanes before it with the same tile (64 lane reads, no memory); the counts so
+// far per tile and the row's block offsets sit in LDS, so the loop over a long row never waits for global memory.
+__global__ void __launch_bounds__(BUILD_WAVES * 64) k_core_fill(const int *__restrict__ ptr, const int *__restrict__ col,
+                                                                const int *__restrict__ rank, int rows, int lb, int ntiles, int tc,
+                                                                const int *__restrict__ blk_off, const int *__restrict__ rem_ptr,
+                                                                unsigned short *__restrict__ idx, int *__restrict__ rem_col)
+{
+    extern __shared__ int fill_lds[];  // [BUILD_WAVES][2][ntiles]: entries already in each tile's list; the row's block offsets
+    const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
+    volatile int *cur = fill_lds + (size_t)wave * 2 * ntiles;
+    volatile int *blk = cur + ntiles;
+    const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    for (long long v = (long long)blockIdx.x * BUILD_WAVES + wave; v < rows; v += (long long)gridDim.x * BUILD_WAVES) {
+        const int i = rank[v];
+        const int beg = ptr[v], end = ptr[v + 1];
+        int w = rem_ptr[v];
+        if (i < 0) {  // every neighbor stays
+            for (int e = beg + lane; e < end; e += 64) rem_col[w + (e - beg)] = col[e];
+            continue;
+        }
+        const size_t row_blocks = (size_t)(i / 64) * ntiles;
+        for (int t = lane; t < ntiles; t += 64) {
+            cur[t] = 0;
+            blk[t] = blk_off[row_blocks + t];
+        }
+        const size_t lane_base = (size_t)(i % 64) * 4;
+        for (int e0 = beg; e0 < end; e0 += 64) {
+            const int e = e0 + lane;
+            const bool valid = e < end;
+            const int c = valid ? col[e] : 0;
+            const int j = valid ? rank[c - lb] : -1;
+            const bool in_core = valid && j >= 0;
+            const unsigned long long stay = __ballot(valid && !in_core);
+            if (valid && !in_core) rem_col[w + __popcll(stay & below)] = c;
+            w += __popcll(stay);
+            if (!__any(in_core)) continue;
+            const int t = in_core ? j / tc : -1 - lane;  // lanes without a core neighbor match nobody
+            int before = 0, after = 0;
+#pragma unroll
+            for (int l = 0; l < 64; ++l) {
+                const int tl = __builtin_amdgcn_readlane(t, l);
+                before += (tl == t && l < lane) ? 1 : 0;
+                after += (tl == t && l > lane) ? 1 : 0;
+            }
+            if (in_core) {
+                const int k = cur[t] + before;
+                const size_t chunk = (size_t)blk[t] + (size_t)(k / 4);
+                idx[chunk * 256 + lane_base + (size_t)(k % 4)] = (unsigned short)(j % tc);
+                if (after == 0) cur[t] = k + 1;  // the last lane of its tile in this group
+            }
+        }
+    }
+}
+
 template <int N4>
 int launch_sell(const CorePlan *p, const v4f *tab, v4f *partial, const Gate &gate, hipStream_t stream)
 {
@@ -172,16 +307,6 @@ void core_plan_free_arrays(CorePlan *p)
     if (p->d_rem_col) (void)hipFree(p->d_rem_col);
 }
 
-template <typename T>
-int upload(T **d, const std::vector<T> &h, size_t min_elems = 1)
-{
-    const size_t n = std::max(h.size(), min_elems);
-    if (hipMalloc((void **)d, n * sizeof(T)) != hipSuccess) return fail(MGGX_ENOMEM, "core plan: %zu bytes of device memory", n * sizeof(T));
-    if (!h.empty() && hipMemcpy(*d, h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice) != hipSuccess)
-        return fail(MGGX_EHIP, "core plan: upload failed");
-    return MGGX_OK;
-}
-
 }  // namespace
 
 void core_plan_free(CorePlan *p)
@@ -204,6 +329,111 @@ int core_side_stream(hipStream_t *stream, hipEvent_t *fork, hipEvent_t *join)
     *stream = s.side_stream;
     *fork = s.side_fork;
     *join = s.side_join;
+    return MGGX_OK;
+}
+
+namespace {
+
+struct Scratch {  // device temporaries of one plan build, freed on the way out
+    std::vector<void *> ptrs;
+    ~Scratch()
+    {
+        for (void *q : ptrs) (void)hipFree(q);
+    }
+    template <typename T>
+    int get(T **q, size_t count)
+    {
+        void *r = nullptr;
+        if (hipMalloc(&r, std::max<size_t>(count, 1) * sizeof(T)) != hipSuccess) return fail(MGGX_ENOMEM, "core plan: %zu bytes of scratch", count * sizeof(T));
+        ptrs.push_back(r);
+        *q = static_cast<T *>(r);
+        return MGGX_OK;
+    }
+};
+
+template <typename T>
+int device_array(T **q, size_t count)
+{
+    if (hipMalloc((void **)q, std::max<size_t>(count, 1) * sizeof(T)) != hipSuccess) return fail(MGGX_ENOMEM, "core plan: %zu bytes of device memory", count * sizeof(T));
+    return MGGX_OK;
+}
+
+}  // namespace
+
+// The arrays of core_layout_build (mggx_internal.h), made on the GPU from the caller's device CSR: a stable radix sort
+// by falling degree gives the ranking, one pass counts list lengths per (core row, tile), two prefix sums place the
+// blocks and the remaining rows, a second pass fills lists and remaining CSR in edge order.  Only scalars come back to
+// the host.  p->unsuitable is set where the host version refuses (no whole unit of rows, ids out of range).
+static int core_plan_build_device(CorePlan *p, int tc)
+{
+    State &s = state();
+    const int rows = p->rows, lb = p->lb;
+    int core = std::min(p->asked, rows);
+    const int unit = tc > 512 ? tc : 512;
+    core = core / unit * unit;
+    if (core < unit) {
+        p->unsuitable = true;
+        return MGGX_OK;
+    }
+    const int ntiles = core / tc, nslices = core / 64;
+    if (ntiles > 2048) return fail(MGGX_ELIMIT, "core plan: %d core rows", core);
+    Scratch tmp;
+    int *deg = nullptr, *deg_sorted = nullptr, *ids = nullptr, *sorted = nullptr, *keep = nullptr, *chunks = nullptr, *flag = nullptr, *blk = nullptr;
+    unsigned short *cnt = nullptr;
+    int rc;
+    if ((rc = tmp.get(&deg, (size_t)rows)) || (rc = tmp.get(&deg_sorted, (size_t)rows)) || (rc = tmp.get(&ids, (size_t)rows)) ||
+        (rc = tmp.get(&sorted, (size_t)rows)) || (rc = tmp.get(&keep, (size_t)rows)) || (rc = tmp.get(&chunks, (size_t)nslices * ntiles)) ||
+        (rc = tmp.get(&flag, 1)) || (rc = tmp.get(&cnt, (size_t)core * ntiles)) || (rc = tmp.get(&blk, (size_t)nslices * ntiles + 1)))
+        return rc;
+    if ((rc = device_array(&p->d_order, (size_t)core)) || (rc = device_array(&p->d_rank, (size_t)rows)) ||
+        (rc = device_array(&p->d_blk_off, (size_t)nslices * ntiles + 1)) || (rc = device_array(&p->d_rem_ptr, (size_t)rows + 1)))
+        return rc;
+    MGGX_HIP(hipMemsetAsync(flag, 0, sizeof(int), s.stream));
+    const unsigned row_blocks = (unsigned)((rows + 255) / 256);
+    k_core_deg<<<row_blocks, 256, 0, s.stream>>>(p->d_ptr_l, rows, deg, ids);
+    size_t need = 0;
+    MGGX_HIP(rocprim::radix_sort_pairs_desc(nullptr, need, deg, deg_sorted, ids, sorted, (size_t)rows, 0, 32, s.stream));
+    char *sort_tmp = nullptr;
+    if ((rc = tmp.get(&sort_tmp, need))) return rc;
+    MGGX_HIP(rocprim::radix_sort_pairs_desc(sort_tmp, need, deg, deg_sorted, ids, sorted, (size_t)rows, 0, 32, s.stream));
+    k_core_rank<<<row_blocks, 256, 0, s.stream>>>(sorted, rows, core, p->d_order, p->d_rank);
+    const unsigned wave_blocks = (unsigned)std::min<long long>(((long long)rows + BUILD_WAVES - 1) / BUILD_WAVES, 256 * 64);
+    const size_t lds = (size_t)BUILD_WAVES * ntiles * sizeof(int);
+    k_core_count<<<wave_blocks, BUILD_WAVES * 64, lds, s.stream>>>(p->d_ptr_l, p->d_col_l, p->d_rank, rows, lb, ntiles, tc, cnt, keep, flag);
+    MGGX_LAUNCH_CHECK("k_core_count");
+    long long rem_nnz = 0, total_chunks = 0;
+    rc = exclusive_scan_i32(keep, p->d_rem_ptr, rows, &rem_nnz);
+    if (rc) return rc;
+    const long long nblk = (long long)nslices * ntiles;
+    k_core_widths<<<(unsigned)((nblk + 255) / 256), 256, 0, s.stream>>>(cnt, nslices, ntiles, chunks);
+    rc = exclusive_scan_i32(chunks, blk, (int)nblk, &total_chunks);
+    if (rc) return rc;
+    int bad = 0, nnz = 0;
+    MGGX_HIP(hipMemcpyAsync(&bad, flag, sizeof(int), hipMemcpyDeviceToHost, s.stream));
+    MGGX_HIP(hipMemcpyAsync(&nnz, p->d_ptr_l + rows, sizeof(int), hipMemcpyDeviceToHost, s.stream));
+    MGGX_HIP(hipMemcpyAsync(p->d_blk_off, blk, sizeof(int) * ((size_t)nblk + 1), hipMemcpyDeviceToDevice, s.stream));
+    MGGX_HIP(hipStreamSynchronize(s.stream));
+    if (bad) {  // a neighbor id outside [lb, lb + rows), or more than 65534 parallel edges into one tile: not this path's input
+        p->unsuitable = true;
+        return MGGX_OK;
+    }
+    if (total_chunks > (long long)(0xFFFFFFFFull / 64)) return fail(MGGX_ELIMIT, "core plan: %lld list chunks", total_chunks);
+    const size_t idx_elems = std::max<size_t>((size_t)total_chunks * 256, 256);
+    if ((rc = device_array(&p->d_idx, idx_elems)) || (rc = device_array(&p->d_rem_col, (size_t)rem_nnz))) return rc;
+    MGGX_HIP(hipMemsetAsync(p->d_idx, 0xFF, idx_elems * sizeof(unsigned short), s.stream));
+    k_core_fill<<<wave_blocks, BUILD_WAVES * 64, 2 * lds, s.stream>>>(p->d_ptr_l, p->d_col_l, p->d_rank, rows, lb, ntiles, tc, blk, p->d_rem_ptr, p->d_idx,
+                                                                  p->d_rem_col);
+    MGGX_LAUNCH_CHECK("k_core_fill");
+    MGGX_HIP(hipStreamSynchronize(s.stream));
+    p->core = core;
+    p->ntiles = ntiles;
+    p->rem_nnz = rem_nnz;
+    p->core_nnz = (int64_t)nnz - rem_nnz;
+    // segments: enough workgroups to fill the chip a few times over, whole tiles each
+    int nseg = 1;
+    while (nseg * 2 <= ntiles && (ntiles % (nseg * 2)) == 0 && (long long)(core / (CORE_WAVES * 64)) * nseg < 2048) nseg *= 2;
+    p->nseg = nseg;
+    p->bytes = ((size_t)core + 2 * (size_t)rows + 1 + (size_t)rem_nnz + (size_t)nblk + 1) * sizeof(int) + idx_elems * sizeof(unsigned short);
     return MGGX_OK;
 }
 
@@ -233,40 +463,7 @@ int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int 
     p->rows = rows;
     p->lb = lb;
     p->asked = core;
-    int rc = MGGX_OK;
-    try {
-        std::vector<int> ptr((size_t)rows + 1);
-        if (hipMemcpy(ptr.data(), d_ptr_l, ptr.size() * sizeof(int), hipMemcpyDeviceToHost) != hipSuccess) rc = fail(MGGX_EHIP, "core plan: reading the CSR");
-        std::vector<int> col(rc ? 0 : (size_t)std::max(ptr[rows], 0));
-        if (!rc && !col.empty() && hipMemcpy(col.data(), d_col_l, col.size() * sizeof(int), hipMemcpyDeviceToHost) != hipSuccess)
-            rc = fail(MGGX_EHIP, "core plan: reading the CSR");
-        CoreLayout L;
-        if (!rc) {
-            const int lrc = core_layout_build(ptr.data(), col.data(), rows, lb, core, CORE_TC, &L);
-            if (lrc == MGGX_EINVAL) p->unsuitable = true;  // remembered: the caller falls back to the ordinary path
-            else rc = lrc;
-        }
-        if (!rc && !p->unsuitable) {
-            p->core = L.core;
-            p->ntiles = L.ntiles;
-            p->core_nnz = L.core_nnz;
-            p->rem_nnz = (int64_t)L.rem_col.size();
-            // segments: enough workgroups to fill the chip a few times over, whole tiles each
-            int nseg = 1;
-            while (nseg * 2 <= p->ntiles && (p->ntiles % (nseg * 2)) == 0 && (long long)(p->core / (CORE_WAVES * 64)) * nseg < 2048) nseg *= 2;
-            p->nseg = nseg;
-            rc = upload(&p->d_order, L.order);
-            if (!rc) rc = upload(&p->d_rank, L.rank);
-            if (!rc) rc = upload(&p->d_blk_off, L.blk_off);
-            if (!rc) rc = upload(&p->d_idx, L.idx, 256);
-            if (!rc) rc = upload(&p->d_rem_ptr, L.rem_ptr);
-            if (!rc) rc = upload(&p->d_rem_col, L.rem_col);
-            p->bytes = (L.order.size() + L.rank.size() + L.rem_ptr.size() + L.rem_col.size()) * sizeof(int) + L.blk_off.size() * sizeof(unsigned) +
-                       std::max<size_t>(L.idx.size(), 256) * sizeof(unsigned short);
-        }
-    } catch (const std::bad_alloc &) {
-        rc = fail(MGGX_ENOMEM, "core plan: out of host memory");
-    }
+    int rc = core_plan_build_device(p, CORE_TC);
     if (rc) {
         core_plan_free_arrays(p);
         delete p;
@@ -372,3 +569,32 @@ int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const 
 }
 
 }  // namespace mggx
+
+using mggx::fail;
+
+MGGX_EXPORT int mggx_core_layout_device(const int *d_ptr, const int *d_col, int rows, int lb, int core_rows, int64_t *sizes, int *order,
+                                        int *rank, unsigned *blk_off, unsigned short *idx, int *rem_ptr, int *rem_col)
+{
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    if (!sizes) return fail(MGGX_EINVAL, "core_layout_device: NULL sizes");
+    mggx::CorePlan *p = nullptr;
+    rc = mggx::core_plan_get(d_ptr, d_col, rows, lb, core_rows, &p);
+    if (rc) return rc;
+    if (p->unsuitable) return fail(MGGX_EINVAL, "core layout: no core of whole 512-row units in %d rows, or a neighbor id outside [lb, lb + rows)", rows);
+    const int64_t nblk = (int64_t)(p->core / 64) * p->ntiles + 1;
+    unsigned chunks = 0;
+    MGGX_HIP(hipMemcpy(&chunks, p->d_blk_off + (nblk - 1), sizeof(unsigned), hipMemcpyDeviceToHost));
+    sizes[0] = p->core;
+    sizes[1] = nblk;
+    sizes[2] = (int64_t)chunks * 256;
+    sizes[3] = p->rem_nnz;
+    sizes[4] = p->core_nnz;
+    if (order) MGGX_HIP(hipMemcpy(order, p->d_order, sizeof(int) * (size_t)p->core, hipMemcpyDeviceToHost));
+    if (rank) MGGX_HIP(hipMemcpy(rank, p->d_rank, sizeof(int) * (size_t)rows, hipMemcpyDeviceToHost));
+    if (blk_off) MGGX_HIP(hipMemcpy(blk_off, p->d_blk_off, sizeof(unsigned) * (size_t)nblk, hipMemcpyDeviceToHost));
+    if (idx && chunks) MGGX_HIP(hipMemcpy(idx, p->d_idx, sizeof(unsigned short) * (size_t)chunks * 256, hipMemcpyDeviceToHost));
+    if (rem_ptr) MGGX_HIP(hipMemcpy(rem_ptr, p->d_rem_ptr, sizeof(int) * ((size_t)rows + 1), hipMemcpyDeviceToHost));
+    if (rem_col && p->rem_nnz) MGGX_HIP(hipMemcpy(rem_col, p->d_rem_col, sizeof(int) * (size_t)p->rem_nnz, hipMemcpyDeviceToHost));
+    return MGGX_OK;
+}

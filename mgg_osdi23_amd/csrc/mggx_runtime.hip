@@ -280,6 +280,25 @@ __global__ void __launch_bounds__(256) k_copy16(int4 *__restrict__ dst, const in
     for (; i < n16; i += stride) dst[i] = src[i];
 }
 
+// The same copy with streaming hints: four 16-byte non-temporal loads in flight per thread before the first store, one
+// workgroup per 16 KiB, no grid-stride loop.  Second opinion on the copy ceiling.
+__global__ void __launch_bounds__(256) k_copy16_nt(int4 *__restrict__ dst, const int4 *__restrict__ src, size_t n16)
+{
+    typedef int v4i __attribute__((ext_vector_type(4)));
+    const size_t base = (size_t)blockIdx.x * 1024 + threadIdx.x;
+    v4i v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const size_t i = base + 256 * (size_t)j;
+        if (i < n16) v[j] = __builtin_nontemporal_load(reinterpret_cast<const v4i *>(src) + i);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const size_t i = base + 256 * (size_t)j;
+        if (i < n16) __builtin_nontemporal_store(v[j], reinterpret_cast<v4i *>(dst) + i);
+    }
+}
+
 __global__ void __launch_bounds__(256) k_cast_bf16(unsigned short *__restrict__ dst, const float *__restrict__ src, long long n)
 {
     long long i = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -446,6 +465,18 @@ MGGX_EXPORT int mggx_copy_bytes(void *d_dst, const void *d_src, size_t n)
     if (blocks > 256 * 64) blocks = 256 * 64;
     k_copy16<<<dim3((unsigned)blocks), dim3(256), 0, state().stream>>>((int4 *)d_dst, (const int4 *)d_src, n16);
     MGGX_LAUNCH_CHECK("k_copy16");
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_copy_bytes_nt(void *d_dst, const void *d_src, size_t n)
+{
+    if (!d_dst || !d_src || (n % 16)) return fail(MGGX_EINVAL, "copy_bytes_nt: NULL pointer or size not a multiple of 16");
+    if (!n) return MGGX_OK;
+    const size_t n16 = n / 16;
+    const size_t blocks = (n16 + 1023) / 1024;
+    if (blocks > 0x7fffffffull) return fail(MGGX_ELIMIT, "copy_bytes_nt: %zu bytes", n);
+    k_copy16_nt<<<dim3((unsigned)blocks), dim3(256), 0, state().stream>>>((int4 *)d_dst, (const int4 *)d_src, n16);
+    MGGX_LAUNCH_CHECK("k_copy16_nt");
     return MGGX_OK;
 }
 

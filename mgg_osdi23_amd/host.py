@@ -58,10 +58,10 @@ EXPORTS = [
     "mggx_last_error", "mggx_version", "mggx_init", "mggx_device_name", "mggx_set_stream", "mggx_sync",
     "mggx_malloc", "mggx_free", "mggx_memset", "mggx_memcpy_h2d", "mggx_memcpy_d2h", "mggx_memcpy_d2d",
     "mggx_timer_create", "mggx_timer_start", "mggx_timer_stop", "mggx_timer_elapsed_ms", "mggx_timer_destroy",
-    "mggx_release_cached", "mggx_forget", "mggx_set_plan_check", "mggx_cache_stats", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_core_layout_build", "mggx_core_layout_fetch", "mggx_graph_read",
+    "mggx_release_cached", "mggx_forget", "mggx_set_plan_check", "mggx_cache_stats", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_core_layout_build", "mggx_core_layout_fetch", "mggx_core_layout_device", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
     "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_compact_remote_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_sag_parts_static", "mggx_mlp2_xw", "mggx_spmm",
-    "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_gather_probe", "mggx_lds_probe", "mggx_gather_rows", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
+    "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_copy_bytes_nt", "mggx_gather_probe", "mggx_lds_probe", "mggx_gather_rows", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
 ]
 
 
@@ -476,6 +476,10 @@ def copy_bytes(dst, src, nbytes: int) -> None:
     _check(lib().mggx_copy_bytes(_dptr(dst), _dptr(src), C.c_size_t(nbytes)))
 
 
+def copy_bytes_nt(dst, src, nbytes: int) -> None:
+    _check(lib().mggx_copy_bytes_nt(_dptr(dst), _dptr(src), C.c_size_t(nbytes)))
+
+
 def gather_probe(sink, table, rows: int, ld_bytes: int, row_bytes: int, n_gathers: int, seed: int = 1) -> int:
     """Random row gathers from `table` (rows x ld_bytes bytes); `sink` holds 262144 floats.  Returns the number issued."""
     done = C.c_int64(0)
@@ -507,4 +511,19 @@ def core_layout(ptr: np.ndarray, col: np.ndarray, lb: int, core_rows: int, tile_
     _check(lib().mggx_core_layout_fetch(h, _iptr(order), _iptr(rank), blk_off.ctypes.data_as(C.c_void_p),
                                         idx.ctypes.data_as(C.c_void_p), _iptr(rem_ptr), _iptr(rem_col)))
     return dict(core=core, ntiles=core // tile_cols, core_nnz=int(sizes[4]), order=order, rank=rank, blk_off=blk_off, idx=idx,
+                rem_ptr=rem_ptr, rem_col=rem_col)
+
+
+def core_layout_device(d_ptr, d_col, rows: int, lb: int, core_rows: int):
+    """The dense-core layout as the aggregation builds it on the GPU (from device tensors) -> the same dict as core_layout."""
+    sizes = (C.c_int64 * 5)()
+    _pin(d_ptr, d_col)
+    _check(lib().mggx_core_layout_device(_dptr(d_ptr), _dptr(d_col), rows, lb, core_rows, sizes, None, None, None, None, None, None))
+    core = int(sizes[0])
+    order, rank = np.zeros(core, np.int32), np.zeros(rows, np.int32)
+    blk_off, idx = np.zeros(int(sizes[1]), np.uint32), np.zeros(int(sizes[2]), np.uint16)
+    rem_ptr, rem_col = np.zeros(rows + 1, np.int32), np.zeros(int(sizes[3]), np.int32)
+    _check(lib().mggx_core_layout_device(_dptr(d_ptr), _dptr(d_col), rows, lb, core_rows, sizes, _iptr(order), _iptr(rank),
+                                         blk_off.ctypes.data_as(C.c_void_p), idx.ctypes.data_as(C.c_void_p), _iptr(rem_ptr), _iptr(rem_col)))
+    return dict(core=core, ntiles=core // 256, core_nnz=int(sizes[4]), order=order, rank=rank, blk_off=blk_off, idx=idx,
                 rem_ptr=rem_ptr, rem_col=rem_col)

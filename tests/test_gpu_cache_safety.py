@@ -190,3 +190,44 @@ def test_captured_graph_survives_workspace_growth_and_cache_pressure(gpu):
         torch.cuda.synchronize()
         gpu.use_torch_stream()
         gpu.release_cached()
+
+
+# --------------------------------------------------------------------------- dense-core plan built on the GPU
+@pytest.mark.parametrize("shape", ["rmat", "ragged", "unsorted_parallel"])
+def test_core_plan_built_on_the_gpu_is_the_host_layout(gpu, shape):
+    """The plan the aggregation builds on the device (radix sort, counting pass, prefix sums, fill pass) against the host
+    builder, whose arrays the CPU tests check against numpy: every array bit for bit."""
+    rng = np.random.default_rng(5)
+    if shape == "rmat":
+        V, lb, core = 9000, 0, 2048
+        ptr, col = gpu.gen_rmat(14, V, 400_000, seed=17)
+    elif shape == "ragged":  # empty rows, equal degrees (ties by id), a share that starts at lb > 0
+        V, lb, core = 3000, 5000, 1024
+        deg = rng.integers(0, 40, V)
+        deg[rng.random(V) < 0.3] = 0
+        deg[:50] = 700
+        ptr = np.zeros(V + 1, np.int32)
+        ptr[1:] = np.cumsum(deg)
+        col = (np.concatenate([np.sort(rng.choice(V, d, replace=False)) for d in deg]) + lb).astype(np.int32)
+    else:  # neighbor lists in random order with repeated edges
+        V, lb, core = 2500, 0, 512
+        deg = rng.integers(1, 300, V)
+        ptr = np.zeros(V + 1, np.int32)
+        ptr[1:] = np.cumsum(deg)
+        col = rng.integers(0, V, int(ptr[-1])).astype(np.int32)
+    want = gpu.core_layout(ptr, col, lb, core)
+    d_ptr, d_col = to_dev(ptr), to_dev(col)
+    got = gpu.core_layout_device(d_ptr, d_col, V, lb, core)
+    assert got["core"] == want["core"] and got["core_nnz"] == want["core_nnz"] and got["core_nnz"] > 0
+    for k in ("order", "rank", "blk_off", "rem_ptr", "rem_col", "idx"):
+        assert np.array_equal(got[k], want[k]), k
+    gpu.forget(d_ptr)
+
+
+def test_core_plan_refuses_ids_outside_the_share(gpu):
+    ptr = np.arange(0, 2049 * 4, 4, dtype=np.int32)
+    col = np.tile(np.array([0, 1, 2, 5000], np.int32), 2048)  # 5000 is not a row of this share
+    d_ptr, d_col = to_dev(ptr), to_dev(col)
+    with pytest.raises(gpu.MggxError, match="outside"):
+        gpu.core_layout_device(d_ptr, d_col, 2048, 0, 1024)
+    gpu.forget(d_ptr)
