@@ -198,25 +198,37 @@ def load_traffic(kernel_key, args, blk=-1, core=-1):
 
 
 class Knobs:
-    """(ps, wpb, dist, column blocking) of one aggregation shape: the command line's, or, where --wpb and --dist are 0
-    and the search is on, what the library's search measures fastest on this input (once, before the timed region; the
-    reference fixes its setting per dataset from the same kind of sweep, bench_MGG_DSE_*.py)."""
+    """(ps, wpb, dist, column blocking, dense core) of one aggregation shape.  Default: the command line's values, where 0
+    leaves the choice to the library's rules and its cost model for the dense core (no measurement).  With `search`
+    (a callable) the library's search measures the settings on this input instead -- the reference fixes its setting per
+    dataset from the same kind of sweep, bench_MGG_DSE_*.py."""
 
-    def __init__(self, args, tune):
+    def __init__(self, args, search=None):
         self.ps, self.wpb, self.dist, self.blk, self.core = args.ps, args.wpb, args.dist, args.col_block_rows, args.core_rows
-        if args.wpb == 0 and args.dist == 0 and not args.no_tune:
-            k, ms = tune(args.ps, args.col_block_rows, args.core_rows)
+        self.searched_ms = None
+        if search is not None:
+            k, ms = search(args.ps, args.col_block_rows, args.core_rows)
             self.ps, self.wpb, self.dist, self.blk, self.core = k["ps"], k["wpb"], k["dist"], k["col_block_rows"], k["core_rows"]
+            self.searched_ms = ms
             log("search: %s (%.4f ms)" % (self, ms))
-        elif self.core == 0:
-            self.core = -1  # left to the rule: off
+
+    def tuple(self):
+        return (self.ps, self.wpb, self.dist, self.blk, self.core)
 
     def observe(self, host, call):
-        """Where the order was left to the library's rule: run the call once and read back which order it used."""
+        """Where choices were left to the library: run the call once and read back what it used."""
+        call()
+        k = host.last_agg_kernel()
+        m = re.search(r"blocks=(\d+)", k)
         if self.blk == 0:
-            call()
-            m = re.search(r"blocks=(\d+)", host.last_agg_kernel())
             self.blk = 49152 if m and int(m.group(1)) > 1 else -1
+        if self.core == 0:
+            m = re.search(r"core=(\d+)", k)
+            self.core = int(m.group(1)) if m else -1
+        m = re.search(r"wpb=(\d+) dist=(\d+)", k)
+        if m:
+            self.wpb, self.dist = (self.wpb or int(m.group(1))), (self.dist or int(m.group(2)))
+        return k
 
     def __str__(self):
         return "ps=%d wpb=%d dist=%d %s%s" % (self.ps, self.wpb, self.dist,
@@ -282,7 +294,6 @@ def bench_gcn2(args, torch, host):
     # row-major order, no dense core) and (2) the library's rules alone (no search): both timed in this run, so the
     # price of the searched setting below can be set against what it buys.
     lit = (16, 8, 1, -1, -1)
-    st0 = host.cache_stats()
     t0 = time.perf_counter()
     for fn in forward_stages(lit, lit):
         fn()
@@ -296,44 +307,47 @@ def bench_gcn2(args, torch, host):
     for fn in forward_stages(rule, rule):
         fn()
     torch.cuda.synchronize()
-    st1 = host.cache_stats()
     r = time_steps(torch, forward_stages(rule, rule), names, max(3, args.steps // 2), 1)
-    extra["rule_only_fwd_ms"] = round(r["event_median_ms"], 4)
-    extra["rule_only"] = {"knobs": "ps=%d, wpb / dist / order by the library's rules, no dense core, no search" % args.ps,
-                          "stage_ms": {k: round(v, 4) for k, v in r["stage_median"].items()},
-                          "plan_build_ms": round(st1["plan_build_ms"] - st0["plan_build_ms"], 2)}
-    log("literal knobs %.4f ms, rules only %.4f ms" % (extra["literal_knobs"]["fwd_ms"], extra["rule_only_fwd_ms"]))
+    extra["rules_without_dense_core"] = {"fwd_ms": round(r["event_median_ms"], 4),
+                                         "knobs": "ps=%d, wpb / dist / order by the library's rules, dense core off" % args.ps,
+                                         "stage_ms": {k: round(v, 4) for k, v in r["stage_median"].items()}}
+    log("literal knobs %.4f ms, rules without the dense core %.4f ms" % (extra["literal_knobs"]["fwd_ms"], r["event_median_ms"]))
 
-    # (3) the searched setting: what the headline is timed with; its set-up is timed here
+    # (3) the headline: knobs as the command line gives them; by default everything is left to the library -- its rules
+    # for ps / wpb / dist / order and its cost model (degree histogram x row width) for the dense core.  No search, no
+    # measurement; the first forward builds the plans (on the GPU) and is timed as the set-up.  With --tune the
+    # library's search picks the knobs instead, as it does in (4) for comparison.
+    search1 = lambda ps, blk, core: host.tune_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, ps,
+                                                     row_scale_out=d_s, col_block_rows=blk, core_rows=core)
+    search2 = lambda ps, blk, core: host.tune_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, ps,
+                                                     row_scale_out=d_s, col_block_rows=blk, core_rows=core, ld_in=pitch, ld_out=pitch)
+    host.release_cached()   # the plans of (1) and (2) are gone: the set-up below is what a first call costs
     setup = {}
-    marks = [host.cache_stats()]
+    mark = host.cache_stats()
     t0 = time.perf_counter()
-    k1 = Knobs(args, lambda ps, blk, core: host.tune_np_div(d_H1, d_Y1, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, hidden, V, ps,
-                                                      row_scale_out=d_s, col_block_rows=blk, core_rows=core))
-    torch.cuda.synchronize()
-    setup["search_agg1"] = (time.perf_counter() - t0) * 1e3
-    marks.append(host.cache_stats())
-    t0 = time.perf_counter()
-    k2 = Knobs(args, lambda ps, blk, core: host.tune_np_div(d_H2, d_Y2, d_ptr, d_col, d_zero_ptr, d_zero_col, 0, V, ldo, V, ps,
-                                                      row_scale_out=d_s, col_block_rows=blk, core_rows=core, ld_in=pitch, ld_out=pitch))
-    torch.cuda.synchronize()
-    setup["search_agg2"] = (time.perf_counter() - t0) * 1e3
-    marks.append(host.cache_stats())
-    setup["core_plan_build"] = marks[2]["core_plan_build_ms"] - marks[0]["core_plan_build_ms"]
-    setup["plan_build"] = marks[2]["plan_build_ms"] - marks[0]["plan_build_ms"]
-    setup = {k: round(v, 2) for k, v in setup.items()}
-    setup["note"] = "search_agg1 / search_agg2 are whole calls (host clock) and include the plan builds listed beside them"
-    stages = forward_stages((k1.ps, k1.wpb, k1.dist, k1.blk, k1.core), (k2.ps, k2.wpb, k2.dist, k2.blk, k2.core))
+    k1 = Knobs(args, search1 if args.tune else None)
+    k2 = Knobs(args, search2 if args.tune else None)
+    stages = forward_stages(k1.tuple(), k2.tuple())
     k1.observe(host, stages[1])
-    k2.observe(host, stages[3])
-    stages[3]()
-    m = re.search(r"core_nnz=(\d+)", host.last_agg_kernel())
+    kstr = k2.observe(host, stages[3])
+    torch.cuda.synchronize()
+    setup["first_use_of_both_aggregations"] = (time.perf_counter() - t0) * 1e3
+    now = host.cache_stats()
+    setup["core_plan_build"] = now["core_plan_build_ms"] - mark["core_plan_build_ms"]
+    setup["plan_build"] = now["plan_build_ms"] - mark["plan_build_ms"]
+    setup["search"] = now["search_ms"] - mark["search_ms"]
+    setup = {k: round(v, 2) for k, v in setup.items()}
+    setup["note"] = ("host clock; first_use_of_both_aggregations is everything between cold caches and two finished aggregation calls and includes "
+                     "the builds listed beside it" + ("" if args.tune else "; no search ran for the headline"))
+    stages = forward_stages(k1.tuple(), k2.tuple())
+    m = re.search(r"core_nnz=(\d+)", kstr)
     core_edges = int(m.group(1)) if m else 0
 
     r = time_steps(torch, stages, names, args.steps, args.warmup)
     avg, med = r["stage_avg"], r["stage_median"]
     held = host.cache_stats()
     extra["setup_ms"] = setup
+    extra["rule_only_fwd_ms"] = None if args.tune else round(r["event_median_ms"], 4)  # the headline itself: rules and cost model, no search
     extra["device_bytes_held_by_library"] = {k: int(held[k]) for k in ("plan_bytes", "core_plan_bytes", "workspace_bytes", "core_scratch_bytes")}
     log("stage ms (median):", {k: round(v, 4) for k, v in med.items()}, "per forward: events median %.4f, host median %.4f, wall mean %.4f"
         % (r["event_median_ms"], r["host_median_ms"], r["wall_ms"]))
@@ -392,6 +406,22 @@ def bench_gcn2(args, torch, host):
     torch.cuda.synchronize()
     H1_gpu, P_gpu, Y1_gpu = d_H1.cpu().numpy(), d_P.cpu().numpy(), d_Y1.cpu().numpy()
     agg1_ms = avg["agg1"]
+    # (4) the library's search on the same inputs (ps x order x core size x wpb x dist measured on the device), timed in the
+    # same run: what the rules and the cost model leave on the table, and what finding out costs.
+    if not args.tune and not args.no_search:
+        mark = host.cache_stats()
+        t0 = time.perf_counter()
+        s1, s2 = Knobs(args, search1), Knobs(args, search2)
+        torch.cuda.synchronize()
+        search_wall = (time.perf_counter() - t0) * 1e3
+        now = host.cache_stats()
+        rs_ = time_steps(torch, forward_stages(s1.tuple(), s2.tuple()), names, max(3, args.steps // 2), 1)
+        extra["searched"] = {"fwd_ms": round(rs_["event_median_ms"], 4), "width16": str(s1), "width41": str(s2),
+                             "stage_ms": {k: round(v, 4) for k, v in rs_["stage_median"].items()},
+                             "search_wall_ms": round(search_wall, 1),
+                             "of_which_plan_builds_ms": round(now["plan_build_ms"] + now["core_plan_build_ms"] - mark["plan_build_ms"] - mark["core_plan_build_ms"], 1),
+                             "headline_over_searched": round(r["event_median_ms"] / rs_["event_median_ms"], 4)}
+        log("searched: %.4f ms per forward (headline / searched = %.3f), search took %.0f ms" % (rs_["event_median_ms"], extra["searched"]["headline_over_searched"], search_wall))
     host.release_cached()
 
     # The HBM-resident workload of the same run: rank 0's 1/8 share, the kernel the roofline is quoted on.
@@ -472,23 +502,34 @@ def share_record(args, torch, host, with_cpu):
     nbytes = agg_bytes(nnz, R, dim, ptr_arrays=2)
 
     def measure(col_r, table, key):
-        t0 = time.perf_counter()
-        kn = Knobs(args, lambda ps, blk, core: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], col_r, lb, ub, dim, npp, ps, input_remote=table,
-                                                          col_block_rows=blk, core_rows=core))
-        torch.cuda.synchronize()
-        search_ms = (time.perf_counter() - t0) * 1e3
-        call = lambda: host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], col_r, lb, ub, dim, npp, 0, kn.ps, kn.wpb, kn.dist, input_remote=table,
-                                           col_block_rows=kn.blk, core_rows=kn.core)
-        kn.observe(host, call)
-        r = time_steps(torch, [call], ["agg"], args.steps, args.warmup)
-        ms = r["stage_avg"]["agg"]
+        search = lambda ps, blk, core: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], col_r, lb, ub, dim, npp, ps, input_remote=table,
+                                                        col_block_rows=blk, core_rows=core)
+
+        def timed(kn):
+            call = lambda: host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], col_r, lb, ub, dim, npp, 0, kn.ps, kn.wpb, kn.dist, input_remote=table,
+                                               col_block_rows=kn.blk, core_rows=kn.core)
+            kn.observe(host, call)
+            r = time_steps(torch, [call], ["agg"], args.steps, args.warmup)
+            return call, r["stage_avg"]["agg"], r["stage_median"]["agg"]
+
+        kn = Knobs(args, search if args.tune else None)
+        call, ms, med = timed(kn)
         gbps = nbytes / (ms * 1e-3) / 1e9
-        rec = {"avg_launch_ms": round(ms, 4), "median_launch_ms": round(r["stage_median"]["agg"], 4), "achieved": round(gbps, 1),
-               "frac": round(gbps / HBM_PEAK_GBPS, 4), "knobs": str(kn), "search_ms": round(search_ms, 2), "kernel": host.last_agg_kernel().split(" grid")[0],
-               **load_traffic(key, args, kn.blk, kn.core)}
+        rec = {"avg_launch_ms": round(ms, 4), "median_launch_ms": round(med, 4), "achieved": round(gbps, 1),
+               "frac": round(gbps / HBM_PEAK_GBPS, 4), "knobs": str(kn) + (" (searched)" if args.tune else " (library rules, no search)"),
+               "kernel": host.last_agg_kernel().split(" grid")[0], **load_traffic(key, args, kn.blk, kn.core)}
         call()
         torch.cuda.synchronize()
-        return rec, d_out.cpu().numpy()
+        result = d_out.cpu().numpy()
+        if not args.tune and not args.no_search:
+            t0 = time.perf_counter()
+            ks = Knobs(args, search)
+            torch.cuda.synchronize()
+            search_ms = (time.perf_counter() - t0) * 1e3
+            _, ms_s, _ = timed(ks)
+            rec["searched"] = {"avg_launch_ms": round(ms_s, 4), "knobs": str(ks), "search_wall_ms": round(search_ms, 2),
+                               "frac": round(nbytes / (ms_s * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "rules_over_searched": round(ms / ms_s, 4)}
+        return rec, result
 
     glob, out_glob = measure(d[3], d_xr, "share_agg")
     # compact staging: distinct remote ids most referenced first, column array rewritten, rows gathered into a small table
@@ -569,8 +610,8 @@ def compact_variant(args, torch, host, d_out, d_xl, d_xr, d, rc, lb, ub, dim, np
     stage = lambda: host.gather_rows(d_xc, d_xr, d_ids, len(ids), dim * esize)
     stage()
     want = d_out.clone()  # produced from the global-id table by the caller
-    kn = Knobs(args, lambda ps, blk, core: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d_rcc, lb, ub, dim, npp, ps, input_remote=d_xc,
-                                                      col_block_rows=blk, core_rows=core))
+    kn = Knobs(args, None if args.no_tune else lambda ps, blk, core: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d_rcc, lb, ub, dim, npp, ps,
+                                                                                         input_remote=d_xc, col_block_rows=blk, core_rows=core))
     call = lambda: host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], d_rcc, lb, ub, dim, npp, 0, kn.ps, kn.wpb, kn.dist,
                                        input_remote=d_xc, col_block_rows=kn.blk, core_rows=kn.core)
     for _ in range(args.warmup):
@@ -617,7 +658,8 @@ def bench_gin(args, torch, host):
     d_P = torch.empty(V, out_dim, device=dev)
 
     d_Y.zero_()
-    kn = Knobs(args, lambda ps, blk, core: host.tune_np_div(d_H, d_Y, d_ptr, d_col, zp, zc, 0, V, hidden, V, ps, gin_eps=eps, col_block_rows=blk, core_rows=core))
+    kn = Knobs(args, None if args.no_tune else lambda ps, blk, core: host.tune_np_div(d_H, d_Y, d_ptr, d_col, zp, zc, 0, V, hidden, V, ps, gin_eps=eps,
+                                                                                         col_block_rows=blk, core_rows=core))
     stages, names = [lambda: host.dense_forward(d_Y, d_X, d_W0, V, in_dim, hidden)], ["dense0"]
     for l in range(L):
         last = l == L - 1
@@ -710,8 +752,8 @@ def bench_big(args, torch, host):
     W = host.glorot(dim, dim, seed=6)
     d_W = torch.from_numpy(W).to(dev).to(torch.bfloat16)
     d_next = torch.empty(R, dim, device=dev, dtype=torch.bfloat16)
-    kn = Knobs(args, lambda ps, blk, core: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, ps, input_remote=d_xr,
-                                                      col_block_rows=blk, core_rows=core))
+    kn = Knobs(args, None if args.no_tune else lambda ps, blk, core: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, ps,
+                                                                                         input_remote=d_xr, col_block_rows=blk, core_rows=core))
     stages = [
         lambda: host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, kn.ps, kn.wpb, kn.dist, input_remote=d_xr,
                                     col_block_rows=kn.blk, core_rows=kn.core),
@@ -916,8 +958,11 @@ def main():
                          "N = the N highest-degree rows")
     ap.add_argument("--wpb", type=int, default=0, help="wavefronts per workgroup; 0 = let the library choose")
     ap.add_argument("--dist", type=int, default=0, help="interleaved_dist; 0 = let the library choose.  With --wpb 0 --dist 0 (the default) the "
-                         "library's search picks the pair once per aggregation shape before the timed region")
-    ap.add_argument("--no-tune", action="store_true", help="with --wpb 0 --dist 0: use the library's rule of thumb instead of its search")
+                         "library's rules pick them")
+    ap.add_argument("--tune", action="store_true", help="time the setting the library's search measures fastest instead of the one its rules and "
+                         "cost model choose (gcn2 and share otherwise run the search afterwards, for comparison)")
+    ap.add_argument("--no-search", action="store_true", help="gcn2 / share: skip the comparison run of the search")
+    ap.add_argument("--no-tune", action="store_true", help="gin / big: use the library's rules instead of its search")
     ap.add_argument("--share-density", type=int, default=1, help="multiplies the number of RMAT draws of --workload share")
     ap.add_argument("--small", action="store_true", help="tiny graph, for a quick functional run")
     ap.add_argument("--big-scale", type=int, default=0, help="--workload big: divide every size by 2^k")

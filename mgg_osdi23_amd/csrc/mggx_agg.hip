@@ -703,21 +703,17 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         return fail(MGGX_EINVAL, "aggregation: unknown input dtype %d", o.in_dtype);
     }
     const int slots = 64 / lpr;
-    // 0 = let the library choose (from sweeps on the benchmark graphs): 8 wavefronts; with few slots per wavefront
-    // (wide rows) 16 rounds, so a workgroup still covers a few thousand neighbors; otherwise a workgroup tile of
-    // about 8 rows' worth of partitions (most rows then finish inside one workgroup), between 1 and 16 rounds.
-    // Column-blocked plans (long rows by construction): 4 wavefronts, 4 rounds for narrow rows.
-    if (wpb == 0) wpb = blocked ? 4 : 8;
+    // 0 = let the library choose (from sweeps of wpb x dist on the benchmark graphs; each choice within 5 % of the best
+    // setting of its sweep).  Few slots per wavefront (wide rows): 8 wavefronts and 16 rounds, so a workgroup still covers
+    // a few thousand neighbors -- 4 wavefronts for column-blocked plans, whose kernel shares the chip with the dense
+    // core's 4-wavefront workgroups.  Many slots (narrow rows): 4 wavefronts, 4 rounds; 8 rounds where a column-blocked
+    // plan is left with short rows (under 8 partitions per row and block).
+    const double per_row = (double)plan->num_parts / (double)(plan->rows > 0 ? plan->rows : 1);
+    if (wpb == 0) wpb = (blocked || slots > 4) ? 4 : 8;
     if (dist == 0) {
-        if (slots <= 4) {
-            dist = 16;
-        } else if (blocked) {
-            dist = 4;
-        } else {
-            const double per_row = (double)plan->num_parts / (double)plan->rows;
-            const long long want = (long long)(8.0 * per_row / (double)(wpb * slots) + 0.999);
-            dist = (int)(want < 1 ? 1 : (want > 16 ? 16 : want));
-        }
+        if (slots <= 4) dist = 16;
+        else if (blocked && per_row < 8.0) dist = 8;
+        else dist = 4;
     }
     const long long parts_per_wg = (long long)wpb * slots * dist;
     if (parts_per_wg > 0x3fffffffLL) return fail(MGGX_ELIMIT, "aggregation: wpb*dist too large");
@@ -844,8 +840,8 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         }
         MGGX_LAUNCH_CHECK("k_agg_block_reduce");
     }
-    snprintf(st.last_kernel, sizeof(st.last_kernel), "k_agg<%d,%d,%d> grid=%lld block=%d parts=%d blocks=%d", lpr, mode, (int)buf, num_wg,
-             64 * wpb, plan->num_parts, plan->blocks);
+    snprintf(st.last_kernel, sizeof(st.last_kernel), "k_agg<%d,%d,%d> grid=%lld block=%d parts=%d blocks=%d ps=%d wpb=%d dist=%d", lpr, mode, (int)buf,
+             num_wg, 64 * wpb, plan->num_parts, plan->blocks, plan->ps, wpb, dist);
     return MGGX_OK;
 }
 
@@ -872,7 +868,7 @@ struct Knobs {
     int core_rows;                  // > 0: that many highest-degree rows form a dense core served from LDS, -1: none
 };
 
-// The dense-core path pays for a host-built plan and partial rows: worth trying on a local-only fp32 CSR with many rows
+// The dense-core path pays for a plan and partial rows: worth considering on a local-only fp32 CSR with many rows
 // beyond the core and a mean degree of 16 or more (on a power-law graph of mean degree 50 the 32 Ki highest-degree rows
 // already hold enough edges among themselves for a quarter less time).
 bool core_eligible(const GraphInfo &g, int dim, int dtype, int core_rows)
@@ -880,19 +876,31 @@ bool core_eligible(const GraphInfo &g, int dim, int dtype, int core_rows)
     return g.nnz_r == 0 && dtype == MGGX_F32 && dim <= 64 && g.rows >= 2 * (long long)core_rows && g.nnz_l >= 16 * (long long)g.rows;
 }
 
-// Fills in the knobs the caller left at 0: from the search's result for this CSR, width and element type, else by rule.
-Knobs resolve_knobs(const GraphInfo &g, int dim, int dtype, int ps, int wpb, int dist, int block_rows, int core_rows)
+// Fills in the knobs the caller left at 0: from the search's result for this CSR, width and element type where there is
+// one, else by rule -- ps 16; the column-blocked order for long sorted rows; the dense core where the cost model over the
+// degree histogram predicts a gain (its size too).  wpb and dist left at 0 are settled per plan in run_agg.
+int resolve_knobs(GraphInfo &g, int dim, int dtype, int ps, int wpb, int dist, int block_rows, int core_rows, unsigned long long table_bytes,
+                  Knobs *out)
 {
     const GraphInfo::Tuned *t = nullptr;
     for (const GraphInfo::Tuned &e : g.tuned)
         if (e.dim == dim && e.dtype == dtype) t = &e;
     Knobs k{ps, wpb, dist, block_rows, core_rows};
-    if (t && (ps == 0 || ps == t->ps) && wpb == 0 && dist == 0 && block_rows == 0 && core_rows == 0)
-        return Knobs{t->ps, t->wpb, t->dist, t->block_rows, t->core_rows};
+    if (t && (ps == 0 || ps == t->ps) && wpb == 0 && dist == 0 && block_rows == 0 && core_rows == 0) {
+        *out = Knobs{t->ps, t->wpb, t->dist, t->block_rows, t->core_rows};
+        return MGGX_OK;
+    }
     if (k.ps == 0) k.ps = 16;
     if (k.block_rows == 0) k.block_rows = blocking_eligible(g, DEFAULT_BLOCK_ROWS) ? DEFAULT_BLOCK_ROWS : -1;
-    if (k.core_rows == 0) k.core_rows = -1;  // by rule: off (its plan is built on the host); the search turns it on where it wins
-    return k;
+    if (k.core_rows == 0) {
+        k.core_rows = -1;
+        if (core_eligible(g, dim, dtype, 8192)) {
+            const int rc = predict_core_rows(g, dim, table_bytes, &k.core_rows);
+            if (rc) return rc;
+        }
+    }
+    *out = k;
+    return MGGX_OK;
 }
 
 // `gate`: the call's content check of the caller's CSR arrays; every kernel launched below looks at it first.
@@ -992,7 +1000,10 @@ MGGX_EXPORT int mggx_sag_np_div(float *d_out, const void *d_in_local, const void
     mggx::Gate gate;
     rc = mggx::guard_check(g->guard, &gate);
     if (rc) return rc;
-    const mggx::Knobs k = mggx::resolve_knobs(*g, dim, o.in_dtype, ps, wpb, dist, o.col_block_rows, o.core_rows);
+    mggx::Knobs k;
+    rc = mggx::resolve_knobs(*g, dim, o.in_dtype, ps, wpb, dist, o.col_block_rows, o.core_rows,
+                             (unsigned long long)(ub - lb) * (unsigned long long)(o.ld_in ? o.ld_in : dim) * (o.in_dtype == MGGX_BF16 ? 2 : 4), &k);
+    if (rc) return rc;
     return mggx::run_knobs(*g, k, d_out, d_in_local, d_in_remote, d_ptr_l, d_col_l, d_ptr_r, d_col_r, lb, ub, dim, o, gate);
 }
 
@@ -1177,6 +1188,8 @@ MGGX_EXPORT int mggx_spmm(float *d_out, const float *d_in, const int *d_row_ptr,
     rc = mggx::guard_check(g->guard, &gate);
     if (rc) return rc;
     // the whole graph on one GPU: the same knob rules (and column-blocked order for long rows) as mggx_sag_np_div
-    mggx::Knobs k = mggx::resolve_knobs(*g, dim, MGGX_F32, ps, wpb, 0, 0, 0);
+    mggx::Knobs k;
+    rc = mggx::resolve_knobs(*g, dim, MGGX_F32, ps, wpb, 0, 0, 0, (unsigned long long)num_nodes * dim * 4, &k);
+    if (rc) return rc;
     return mggx::run_knobs(*g, k, d_out, d_in, nullptr, d_row_ptr, d_col, nullptr, nullptr, 0, num_nodes, dim, o, gate);
 }

@@ -9,6 +9,7 @@
 // the partial rows to the output the aggregation wrote.
 #include <algorithm>
 #include <chrono>
+#include <cmath>
 #include <new>
 
 #include <rocprim/device/device_radix_sort.hpp>
@@ -565,6 +566,154 @@ int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const 
                                                                                     p->nseg, relu, all_rows, gate);
     }
     MGGX_LAUNCH_CHECK("k_core_finish");
+    return MGGX_OK;
+}
+
+}  // namespace mggx
+
+// ---------------------------------------------------------------------------
+// Cost model: which core size pays.
+//
+// Rows are ranked by degree.  Under the configuration model an edge joins ranks i and j with probability
+// d_i d_j / nnz, so the list of a row of rank i for the tile of columns [256 t, 256 t + 256) holds lambda = d_i D_t / nnz
+// entries on average (D_t = degree sum of the tile's columns, at most 256), and the 64 lists of a slice are padded to
+// the longest of them, rounded up to 4: E[4 ceil(max of 64 Poisson(lambda) / 4)], tabulated once.  That gives the
+// useful and the padded entries of any core size from the degree histogram alone (within 3 % of the built plans on the
+// benchmark graphs).  Growing the core by a band of rows pays while the band's useful entries per padded entry stay
+// above theta = (cost of one padded entry in the LDS kernel) / (cost of one edge in the gather kernel)
+//             = ALPHA x ceil(dim/4) / (BETA x 64-byte sectors of a row x (1 or HBM_FACTOR)),
+// constants fitted to sweeps of the core size on the 233 K-node width-16 / width-44 and the 2.45 M-node width-64
+// graphs (ALPHA 1.1 ps per padded 16-byte piece; BETA 9 ps per 64-byte sector of a gathered row while the table fits
+// the 256 MB last-level cache, 1.9 x that beyond).
+namespace mggx {
+namespace {
+
+constexpr int PROFILE_SLICES = 1024;  // 65536 ranks
+constexpr double ALPHA_PS = 1.1, BETA_PS = 9.0, HBM_FACTOR = 1.9;
+constexpr unsigned long long LAST_LEVEL_CACHE_BYTES = 256ull << 20;
+constexpr int MODEL_STEP = 4096, MODEL_MAX_CORE = 57344;
+
+__global__ void __launch_bounds__(256) k_degrees(const int *__restrict__ ptr, int rows, int *__restrict__ deg)
+{
+    const int v = blockIdx.x * 256 + threadIdx.x;
+    if (v < rows) deg[v] = ptr[v + 1] - ptr[v];
+}
+
+// slice_sum[s] = sum of sorted[64 s .. 64 s + 63] (sorted: falling degrees), one wavefront per slice
+__global__ void __launch_bounds__(256) k_slice_sums(const int *__restrict__ sorted, int rows, int slices, float *__restrict__ slice_sum)
+{
+    const int s = blockIdx.x * 4 + (int)(threadIdx.x >> 6), lane = (int)(threadIdx.x & 63u);
+    if (s >= slices) return;
+    const int i = s * 64 + lane;
+    float d = i < rows ? (float)sorted[i] : 0.f;
+    for (int o = 32; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+    if (lane == 0) slice_sum[s] = d;
+}
+
+// E[4 ceil(max of 64 independent Poisson(lambda) / 4)] on a logarithmic grid of lambda
+struct PaddingTable {
+    static constexpr int N = 96;
+    double lo = 1e-3, hi = 300.0, v[N];
+    PaddingTable()
+    {
+        for (int i = 0; i < N; ++i) {
+            const double lam = lo * std::pow(hi / lo, (double)i / (N - 1));
+            // P(X <= m) by the recurrence of the Poisson terms; E = sum_j 4 (1 - F(4 j)^64)
+            double term = std::exp(-lam), cdf = term, e = 0.0;
+            int m = 0;
+            for (int j = 0; j < 400; ++j) {
+                while (m < 4 * j) {
+                    ++m;
+                    term *= lam / m;
+                    cdf += term;
+                }
+                const double miss = 1.0 - std::pow(std::min(cdf, 1.0), 64.0);
+                e += 4.0 * miss;
+                if (miss < 1e-12 && 4 * j > lam) break;
+            }
+            v[i] = e;
+        }
+    }
+    double operator()(double lam) const
+    {
+        if (lam <= lo) return 256.0 * lam;  // 4 P(some lane has an entry) ~ 4 x 64 lambda
+        if (lam >= hi) return lam + 4.0 * std::sqrt(lam);
+        const double x = std::log(lam / lo) / std::log(hi / lo) * (N - 1);
+        const int i = std::min((int)x, N - 2);
+        return v[i] + (v[i + 1] - v[i]) * (x - i);
+    }
+};
+
+int fetch_degree_profile(GraphInfo &g)
+{
+    State &s = state();
+    if (g.have_profile) return MGGX_OK;
+    if (capturing()) return fail(MGGX_EINVAL, "cost model: first use of these CSR arrays inside a stream capture; call once outside the capture first");
+    const int rows = g.rows;
+    const int slices = std::min(PROFILE_SLICES, (rows + 63) / 64);
+    Scratch tmp;
+    int *deg = nullptr, *sorted = nullptr;
+    float *d_sum = nullptr;
+    char *sort_tmp = nullptr;
+    int rc;
+    if ((rc = tmp.get(&deg, (size_t)rows)) || (rc = tmp.get(&sorted, (size_t)rows)) || (rc = tmp.get(&d_sum, (size_t)slices))) return rc;
+    k_degrees<<<(unsigned)((rows + 255) / 256), 256, 0, s.stream>>>(g.d_ptr_l, rows, deg);
+    size_t need = 0;
+    MGGX_HIP(rocprim::radix_sort_keys_desc(nullptr, need, deg, sorted, (size_t)rows, 0, 32, s.stream));
+    if ((rc = tmp.get(&sort_tmp, need))) return rc;
+    MGGX_HIP(rocprim::radix_sort_keys_desc(sort_tmp, need, deg, sorted, (size_t)rows, 0, 32, s.stream));
+    k_slice_sums<<<(unsigned)((slices + 3) / 4), 256, 0, s.stream>>>(sorted, rows, slices, d_sum);
+    MGGX_LAUNCH_CHECK("k_slice_sums");
+    g.slice_deg.assign((size_t)slices, 0.f);
+    MGGX_HIP(hipMemcpyAsync(g.slice_deg.data(), d_sum, sizeof(float) * (size_t)slices, hipMemcpyDeviceToHost, s.stream));
+    MGGX_HIP(hipStreamSynchronize(s.stream));
+    g.have_profile = true;
+    return MGGX_OK;
+}
+
+}  // namespace
+
+int predict_core_rows(GraphInfo &g, int dim, unsigned long long table_bytes, int *core_rows)
+{
+    static const PaddingTable padded;
+    *core_rows = -1;
+    if (g.rows < 2 * MODEL_STEP || g.nnz_l <= 0) return MGGX_OK;
+    const bool beyond_cache = table_bytes > LAST_LEVEL_CACHE_BYTES;
+    for (const GraphInfo::Predicted &p : g.predicted)
+        if (p.dim == dim && p.beyond_cache == beyond_cache) {
+            *core_rows = p.core_rows;
+            return MGGX_OK;
+        }
+    int rc = fetch_degree_profile(g);
+    if (rc) return rc;
+    const int n4 = (dim + 3) / 4;
+    const int sectors = (dim * 4 + 63) / 64;
+    const double theta = ALPHA_PS * n4 / (BETA_PS * sectors * (beyond_cache ? HBM_FACTOR : 1.0));
+    const double nnz = (double)g.nnz_l;
+    const int max_core = std::min({MODEL_MAX_CORE, g.rows / 2 / MODEL_STEP * MODEL_STEP, (int)g.slice_deg.size() * 64 / MODEL_STEP * MODEL_STEP});
+    // useful and padded entries of the block (slices [s0, s1) x tiles [t0, t1))
+    const auto block = [&](int s0, int s1, int t0, int t1, double *useful, double *pad) {
+        for (int sl = s0; sl < s1; ++sl) {
+            const double d = g.slice_deg[(size_t)sl] / 64.0;
+            for (int t = t0; t < t1; ++t) {
+                const double dt = (double)g.slice_deg[4 * (size_t)t] + g.slice_deg[4 * (size_t)t + 1] + g.slice_deg[4 * (size_t)t + 2] + g.slice_deg[4 * (size_t)t + 3];
+                const double lam = std::min(d * dt / nnz, 256.0);
+                *useful += 64.0 * lam;
+                *pad += 64.0 * padded(lam);
+            }
+        }
+    };
+    int best = 0;
+    for (int k = MODEL_STEP; k <= max_core; k += MODEL_STEP) {
+        // the band the core grows by: new rows x all tiles, old rows x new tiles
+        double useful = 0.0, pad = 0.0;
+        block((k - MODEL_STEP) / 64, k / 64, 0, k / 256, &useful, &pad);
+        block(0, (k - MODEL_STEP) / 64, (k - MODEL_STEP) / 256, k / 256, &useful, &pad);
+        if (pad <= 0.0 || useful / pad < theta) break;
+        best = k;
+    }
+    if (best >= 2 * MODEL_STEP) *core_rows = best;
+    g.predicted.push_back({dim, beyond_cache, *core_rows});
     return MGGX_OK;
 }
 

@@ -139,6 +139,12 @@ struct GraphInfo {
     const int *d_col_l = nullptr;
     const int *d_col_r = nullptr;
     int rows = 0;
+    // degree profile for the dense-core cost model: sum of the degrees of ranks [64 s, 64 s + 64) for the 1024 highest-degree
+    // slices (rows ranked by falling degree), fetched once per record
+    std::vector<float> slice_deg;
+    bool have_profile = false;
+    struct Predicted { int dim; bool beyond_cache; int core_rows; };
+    std::vector<Predicted> predicted;  // what the cost model said for a row width (evaluated once, a millisecond of host time)
     bool internal = false;  // arrays owned by the library (the remainder CSR of a dense-core plan): no content check
     bool pinned = false;    // used inside a stream capture: never evicted
     Guard guard;
@@ -205,6 +211,10 @@ int static_scratch_ptr(unsigned char **out);
 void plan_free(Plan *p);
 int forget_pointer(const void *d_ptr);
 int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, CorePlan **out);
+// Cost model of the dense core (degree histogram x row width): the core size that is predicted to pay for this CSR, a
+// multiple of 4096, or -1 for none.  table_bytes = rows x row pitch of the feature table.  Fetches the record's degree
+// profile on first use (one sort of the degrees on the device, 4 KiB to the host; synchronises).
+int predict_core_rows(GraphInfo &g, int dim, unsigned long long table_bytes, int *core_rows);
 void core_plan_free(CorePlan *p);
 int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, const Gate &gate, hipStream_t stream);
 int run_core_sums(CorePlan *p, int dim, const Gate &gate, hipStream_t stream);

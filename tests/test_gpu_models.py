@@ -267,10 +267,11 @@ def test_full_size_share_of_eight(gpu):
     d = [to_dev(a) for a in (lp, lc, rp, rc)]
     d_xl, d_xr = to_dev(xl), to_dev(x)
     out = torch.empty(ub - lb, dim, device="cuda")
-    for ps, wpb, dist in [(16, 8, 1), (4, 4, 4), (32, 16, 2)]:
+    for ps, wpb, dist in [(16, 8, 1), (4, 4, 4), (32, 16, 2), (0, 0, 0)]:
         out.fill_(-3.0)
         gpu.mgg_SAG_np_div(out, d_xl, d[0], d[1], d[2], d[3], lb, ub, dim, npp, 0, ps, wpb, dist, input_remote=d_xr)
         gpu.sync()
+        assert "core=" not in gpu.last_agg_kernel()  # remote edges: the dense-core path is not for a split share
         check_sampled_rows(gpu, out.cpu().numpy(), sh, xl, x, dim)
     # size-independent properties: ones -> degree (exact); linearity: A(x) + A(y) == A(x + y) within rounding
     ones = torch.ones(n * npp, dim, device="cuda")
