@@ -53,7 +53,10 @@ extern "C" {
 /* aggregation flags */
 #define MGGX_AGG_ACCUMULATE 1u /* out += result (mgg_SAG_np_div never zeroes out, neighbor_utils.cuh:1458) */
 #define MGGX_AGG_GIN 2u        /* out = (1+eps)*x_self + sum (mgg_GIN_np_div_cuda, neighbor_utils.cuh:1660-1665) */
-#define MGGX_AGG_RELU 4u       /* max(0, .) applied last (not in the reference; off by default) */
+#define MGGX_AGG_RELU 4u       /* max(0, .) applied after the sum (not in the reference; off by default) */
+#define MGGX_AGG_SOFTMAX 8u    /* row softmax over the dim columns applied last, inside the kernels that finish a row: the
+                                * aggregation and the softmax_forward that follows it in the reference's last layer
+                                * (src/mgg_np_div_mem.cu:221-225, include/gnn_layer.cuh:36-40) as one call */
 
 /* feature element types */
 #define MGGX_F32 0

@@ -198,15 +198,42 @@ __device__ __forceinline__ float load_self(const AggArgs &a, int row, int d)
     return static_cast<const float *>(a.in_l)[(long long)row * a.ld_in + d];
 }
 
-// Finishes one output element: scale, GIN self term, accumulate, ReLU, store.
-__device__ __forceinline__ void finish_elem(const AggArgs &a, int row, int d, float sum)
+// One finished output element before the store: scale, GIN self term, accumulate, ReLU.
+__device__ __forceinline__ float epilogue_value(const AggArgs &a, int row, int d, float sum)
 {
     float v = a.rs_out ? sum * a.rs_out[row] : sum;
     if (a.flags & MGGX_AGG_GIN) v += (1.0f + a.eps) * load_self(a, row, d);
-    float *o = a.out + (long long)row * a.ld_out + d;
-    if (a.flags & MGGX_AGG_ACCUMULATE) v += *o;
+    if (a.flags & MGGX_AGG_ACCUMULATE) v += a.out[(long long)row * a.ld_out + d];
     if (a.flags & MGGX_AGG_RELU) v = fmaxf(v, 0.0f);
-    *o = v;
+    return v;
+}
+
+__device__ __forceinline__ void finish_elem(const AggArgs &a, int row, int d, float sum)
+{
+    a.out[(long long)row * a.ld_out + d] = epilogue_value(a, row, d, sum);
+}
+
+// Row softmax over values spread across a group of G adjacent lanes (G a power of two, the group aligned to G), NPL values
+// per lane, `on[i]` false for slots past the row width: v[i] <- exp(v[i] - max) / sum.  Every lane of the group must be
+// active.  The epilogue of the last layer (MGGX_AGG_SOFTMAX), so that the logits never make a round trip through memory.
+template <int NPL>
+__device__ __forceinline__ void group_softmax(float (&v)[NPL], const bool (&on)[NPL], int G)
+{
+    const int lane = lane_id();
+    float m = -3.0e38f;
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) m = on[i] ? fmaxf(m, v[i]) : m;
+    for (int o = 1; o < G; o <<= 1) m = fmaxf(m, lane_read(m, lane ^ o));
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+        v[i] = on[i] ? __expf(v[i] - m) : 0.f;
+        sum += v[i];
+    }
+    for (int o = 1; o < G; o <<= 1) sum += lane_read(sum, lane ^ o);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) v[i] *= inv;
 }
 
 // Output rows are written once and not read again by the aggregation: stored with the streaming hint.
@@ -221,6 +248,21 @@ template <int LPR, int MODE>
 __device__ __forceinline__ void finish_row(const AggArgs &a, int row, int l, const float (&acc)[ModeTraits<MODE>::NV])
 {
     constexpr int NV = ModeTraits<MODE>::NV;
+    if (a.flags & MGGX_AGG_SOFTMAX) {  // the slot's LPR lanes hold the whole row: softmax across them, then the store
+        float v[NV];
+        bool on[NV];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int d = elem_of<LPR, MODE>(l, i);
+            on[i] = d < a.dim;
+            v[i] = on[i] ? epilogue_value(a, row, d, acc[i]) : 0.f;
+        }
+        group_softmax<NV>(v, on, LPR);
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            if (on[i]) a.out[(long long)row * a.ld_out + elem_of<LPR, MODE>(l, i)] = v[i];
+        return;
+    }
     if constexpr (MODE == MODE_F32_VEC4) {
         if (a.flags == 0 && a.rs_out == nullptr) {
             if (NV * l < a.dim)
@@ -496,10 +538,24 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     int orow = -1;
     auto emit = [&](bool ends) {
         if (started && ends) {
+            if (a.flags & MGGX_AGG_SOFTMAX) {
+                float v[4];
+                bool on[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int dd = lane + 64 * i;
-                if (dd < a.dim) finish_elem(a, orow, dd, s[i]);
+                for (int i = 0; i < 4; ++i) {
+                    on[i] = lane + 64 * i < a.dim;
+                    v[i] = on[i] ? epilogue_value(a, orow, lane + 64 * i, s[i]) : 0.f;
+                }
+                group_softmax<4>(v, on, 64);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (on[i]) a.out[(long long)orow * a.ld_out + lane + 64 * i] = v[i];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int dd = lane + 64 * i;
+                    if (dd < a.dim) finish_elem(a, orow, dd, s[i]);
+                }
             }
         } else {
             const int e = started ? 2 * wg + 1 : 2 * wg;
@@ -549,90 +605,135 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     if (open) emit(false);
 }
 
-// Rows that cross workgroups: the workgroup where the row starts left a tail entry; every later workgroup up to
-// the one where it ends left a head entry.  A wavefront finishes 64/comp_lanes consecutive workgroup slots at once:
-// lane = (walker, component) with `comp_lanes` = power of two >= dim (<= 64); a walker whose slot holds a tail sums
-// that row's chain of head entries in order, four loads in flight.  Wider rows (dim > 64) use one walker per
-// wavefront and several components per lane.
-__global__ void __launch_bounds__(256) k_agg_fixup(const AggArgs a, int num_wg, int comp_lanes)
+// What the main kernel leaves open, in one launch.  Workgroups [0, fix_blocks): rows that cross workgroups -- the
+// workgroup where such a row starts left a tail entry, every later workgroup up to the one where it ends a head entry.
+// A wavefront finishes 64/comp_lanes consecutive workgroup slots at once: lane = (walker, component) with `comp_lanes` a
+// power of two >= dim (<= 64; wider rows use one walker per wavefront and up to four components per lane); a walker whose
+// slot holds a tail sums that row's chain of head entries in order, four loads in flight.  Workgroups from fix_blocks
+// on: rows with no neighbor at all (their sum is zero), one group of comp_lanes lanes per row.
+__global__ void __launch_bounds__(256) k_agg_tail(const AggArgs a, int num_wg, int comp_lanes, int fix_blocks, const int *__restrict__ empty_rows,
+                                                  int n_empty)
 {
     if (gate_closed(a.gate)) return;
     const int lane = lane_id();
     const int group = 64 / comp_lanes;
-    const long long b = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * group + lane / comp_lanes;
-    if (b >= num_wg - 1) return;
-    const int2 t = a.c_hdr[2 * b + 1];
-    if (!(t.y & HDR_VALID)) return;
-    const int row = t.x;
-    const int n = (a.off[row + 1] - 1) / a.parts_per_wg - (int)b;  // head entries of workgroups b+1 .. b+n
-    for (int c = lane % comp_lanes; c < a.dim; c += comp_lanes) {
-        float total = a.c_val[(size_t)(2 * b + 1) * a.cpad + c];
-        int k = 0;
-        for (; k + 4 <= n; k += 4) {
-            const float v0 = a.c_val[(size_t)(2 * (b + 1 + k)) * a.cpad + c];
-            const float v1 = a.c_val[(size_t)(2 * (b + 2 + k)) * a.cpad + c];
-            const float v2 = a.c_val[(size_t)(2 * (b + 3 + k)) * a.cpad + c];
-            const float v3 = a.c_val[(size_t)(2 * (b + 4 + k)) * a.cpad + c];
-            total += v0;
-            total += v1;
-            total += v2;
-            total += v3;
+    const int c0 = lane % comp_lanes;
+    float total[4] = {0.f, 0.f, 0.f, 0.f};
+    int row;
+    if ((int)blockIdx.x < fix_blocks) {
+        const long long b = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * group + lane / comp_lanes;
+        if (b >= num_wg - 1) return;
+        const int2 t = a.c_hdr[2 * b + 1];
+        if (!(t.y & HDR_VALID)) return;
+        row = t.x;
+        const int n = (a.off[row + 1] - 1) / a.parts_per_wg - (int)b;  // head entries of workgroups b+1 .. b+n
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = c0 + i * comp_lanes;
+            if (c >= a.dim) break;
+            float tot = a.c_val[(size_t)(2 * b + 1) * a.cpad + c];
+            int k = 0;
+            for (; k + 4 <= n; k += 4) {
+                const float v0 = a.c_val[(size_t)(2 * (b + 1 + k)) * a.cpad + c];
+                const float v1 = a.c_val[(size_t)(2 * (b + 2 + k)) * a.cpad + c];
+                const float v2 = a.c_val[(size_t)(2 * (b + 3 + k)) * a.cpad + c];
+                const float v3 = a.c_val[(size_t)(2 * (b + 4 + k)) * a.cpad + c];
+                tot += v0;
+                tot += v1;
+                tot += v2;
+                tot += v3;
+            }
+            for (; k < n; ++k) tot += a.c_val[(size_t)(2 * (b + 1 + k)) * a.cpad + c];
+            total[i] = tot;
         }
-        for (; k < n; ++k) total += a.c_val[(size_t)(2 * (b + 1 + k)) * a.cpad + c];
-        finish_elem(a, row, c, total);
+    } else {
+        const long long e = ((long long)((int)blockIdx.x - fix_blocks) * 4 + (threadIdx.x >> 6)) * group + lane / comp_lanes;
+        if (e >= n_empty) return;
+        row = empty_rows[e];
     }
+    float v[4];
+    bool on[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = c0 + i * comp_lanes;
+        on[i] = c < a.dim;
+        v[i] = on[i] ? epilogue_value(a, row, c, total[i]) : 0.f;
+    }
+    if (a.flags & MGGX_AGG_SOFTMAX) group_softmax<4>(v, on, comp_lanes);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (on[i]) a.out[(long long)row * a.ld_out + c0 + i * comp_lanes] = v[i];
 }
 
-// Rows with no neighbor at all: the sum is zero.
-__global__ void __launch_bounds__(256) k_agg_empty_rows(const AggArgs a, const int *__restrict__ rows, int n_rows)
+// What a column-blocked plan leaves open, in one launch: out[v] = epilogue(sum over blocks c of the partial row of
+// virtual row c * rows + v, blocks in order [+ the dense core's partial rows of v]).  A virtual row that the main kernel
+// finished lies in `part`; one that crossed workgroups is the sum of its chain in the carry buffer (the tail entry of the
+// workgroup it starts in, then the head entries of the following ones); one without neighbors is zero -- all told by the
+// plan's row offsets, so no fix-up pass, no zero fill and no separate reduction run.  G lanes per row (a power of two
+// >= dim/4), lane q holds columns 4 q .. 4 q + 3; the epilogue is the caller's (row scale, accumulate, ReLU, softmax).
+struct CoreMergeArgs {
+    const float4 *partial;  // [nseg][core][n4] or NULL
+    const int *rank;        // [rows]: rank in the core or -1
+    int core, nseg;
+};
+
+__global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp, int G,
+                                                            const CoreMergeArgs cm)
 {
     if (gate_closed(a.gate)) return;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (long long)n_rows * a.dim) return;
-    const int r = rows[idx / a.dim];
-    const int d = (int)(idx % a.dim);
-    finish_elem(a, r, d, 0.0f);
-}
-
-// Column-blocked plans: out[v] = epilogue(sum over blocks c of P[c * rows + v]), blocks summed in order.
-__global__ void __launch_bounds__(256) k_agg_block_reduce(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp)
-{
-    if (gate_closed(a.gate)) return;
-    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (long long)rows * a.dim) return;
-    const int v = (int)(idx / a.dim), d = (int)(idx % a.dim);
-    float total = 0.0f;
-    for (int c = 0; c < blocks; ++c) total += part[((long long)c * rows + v) * ldp + d];
-    finish_elem(a, v, d, total);
-}
-
-// The same with four columns per thread, for outputs that take 16-byte stores and epilogues without a read of
-// other tables (row scale, accumulation and ReLU only).
-__global__ void __launch_bounds__(256) k_agg_block_reduce4(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp)
-{
-    if (gate_closed(a.gate)) return;
-    const int q = a.dim >> 2;  // float4 per row
-    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (long long)rows * q) return;
-    const int v = (int)(idx / q), d = 4 * (int)(idx % q);
+    const long long v_ll = idx / G;
+    const int q = (int)(idx % G);
+    const int n4 = (a.dim + 3) >> 2;
+    if (v_ll >= rows) return;  // G divides 64: the lanes of a row leave together
+    const int v = (int)v_ll;
     float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int c = 0; c < blocks; ++c) {
-        const float4 p = *reinterpret_cast<const float4 *>(part + ((long long)c * rows + v) * ldp + d);
-        t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
+    const bool lane_on = q < n4;
+    if (lane_on) {
+        for (int c = 0; c < blocks; ++c) {
+            const long long vr = (long long)c * rows + v;
+            const int o0 = a.off[vr], o1 = a.off[vr + 1];
+            if (o1 == o0) continue;
+            const int w0 = o0 / a.parts_per_wg, w1 = (o1 - 1) / a.parts_per_wg;
+            float4 p;
+            if (w0 == w1) {
+                p = *reinterpret_cast<const float4 *>(part + vr * ldp + 4 * q);
+            } else {
+                p = *reinterpret_cast<const float4 *>(a.c_val + (size_t)(2 * w0 + 1) * a.cpad + 4 * q);
+                for (int w = w0 + 1; w <= w1; ++w) {
+                    const float4 h = *reinterpret_cast<const float4 *>(a.c_val + (size_t)(2 * w) * a.cpad + 4 * q);
+                    p.x += h.x; p.y += h.y; p.z += h.z; p.w += h.w;
+                }
+            }
+            t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
+        }
+        if (cm.partial) {
+            const int r = cm.rank[v];
+            if (r >= 0)
+                for (int seg = 0; seg < cm.nseg; ++seg) {
+                    const float4 p = cm.partial[((size_t)seg * cm.core + r) * n4 + q];
+                    t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
+                }
+        }
     }
-    if (a.rs_out) {
-        const float s = a.rs_out[v];
-        t.x *= s; t.y *= s; t.z *= s; t.w *= s;
+    float val[4] = {t.x, t.y, t.z, t.w};
+    bool on[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        on[i] = lane_on && 4 * q + i < a.dim;
+        val[i] = on[i] ? epilogue_value(a, v, 4 * q + i, val[i]) : 0.f;
     }
-    float4 *o = reinterpret_cast<float4 *>(a.out + (long long)v * a.ld_out + d);
-    if (a.flags & MGGX_AGG_ACCUMULATE) {
-        const float4 p = *o;
-        t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
+    if (a.flags & MGGX_AGG_SOFTMAX) group_softmax<4>(val, on, G);
+    float *o = a.out + (long long)v * a.ld_out + 4 * q;
+    if (lane_on) {
+        if (4 * q + 3 < a.dim && (a.ld_out & 3) == 0 && (reinterpret_cast<uintptr_t>(a.out) & 15u) == 0) {
+            *reinterpret_cast<float4 *>(o) = make_float4(val[0], val[1], val[2], val[3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (on[i]) o[i] = val[i];
+        }
     }
-    if (a.flags & MGGX_AGG_RELU) {
-        t.x = fmaxf(t.x, 0.f); t.y = fmaxf(t.y, 0.f); t.z = fmaxf(t.z, 0.f); t.w = fmaxf(t.w, 0.f);
-    }
-    *o = t;
 }
 
 int pow2_ceil(int x)
@@ -672,9 +773,22 @@ struct FixedScratch {
     const int *nnz_l_dev;
 };
 
+// The dense core's side of a call, handed to the aggregation of the remaining CSR: where a column-blocked plan ends in
+// its finish kernel anyway, that kernel also waits for the core block (event `join`), adds its partial rows and applies
+// the caller's whole epilogue (`merged` is set); otherwise the post-operations (ReLU, softmax) are left out here and the
+// caller adds the core afterwards.
+struct CoreMerge {
+    const float4 *partial;
+    const int *rank;
+    int core, nseg;
+    hipEvent_t join;
+    bool merged;
+};
+
 int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, const int *d_col_l, const int *d_col_r,
-            int lb, int dim, int wpb, int dist, const mggx_agg_opts &o, const Gate &gate, const FixedScratch *fixed = nullptr)
+            int lb, int dim, int wpb, int dist, const mggx_agg_opts &o_in, const Gate &gate, const FixedScratch *fixed = nullptr, CoreMerge *cm = nullptr)
 {
+    mggx_agg_opts o = o_in;
     State &st = state();
     if (dim < 1 || dim > 256) return fail(MGGX_ELIMIT, "aggregation: dim %d outside 1..256", dim);
     if (wpb < 0 || wpb > 16) return fail(MGGX_EINVAL, "aggregation: wpb %d outside 0..16 (0 = choose)", wpb);
@@ -683,7 +797,8 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     if (ld_in < dim || ld_out < dim) return fail(MGGX_EINVAL, "aggregation: row stride smaller than dim");
     if (plan->rows == 0) return MGGX_OK;
     if (!d_out || !d_in_l) return fail(MGGX_EINVAL, "aggregation: NULL feature pointer");
-    const bool blocked = plan->blocks > 1;
+    const bool blocked = plan->blocks > 1 && plan->num_parts > 0;
+    if (cm && !blocked) o.flags &= ~(MGGX_AGG_RELU | MGGX_AGG_SOFTMAX);  // the caller applies them after adding the core
     if (plan->nnz_r > 0 && (!d_in_r || !d_col_r)) return fail(MGGX_EINVAL, "aggregation: remote edges but no remote table");
     if (plan->nnz_l > 0 && !d_col_l) return fail(MGGX_EINVAL, "aggregation: local edges but no column array");
 
@@ -809,36 +924,39 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         }
         if (rc) return rc;
         MGGX_LAUNCH_CHECK("k_agg");
-        if (num_wg > 1) {
-            const int comp_lanes = dim >= 64 ? 64 : pow2_ceil(dim);
-            const long long fix_slots_per_block = 4 * (64 / comp_lanes);
-            const long long fix_blocks = (num_wg - 1 + fix_slots_per_block - 1) / fix_slots_per_block;
-            k_agg_fixup<<<dim3((unsigned)fix_blocks), dim3(256), 0, st.stream>>>(a, (int)num_wg, comp_lanes);
-            MGGX_LAUNCH_CHECK("k_agg_fixup");
-        }
-    }
-    const bool touch_empty = blocked || !(o.flags & MGGX_AGG_ACCUMULATE) || (o.flags & (MGGX_AGG_GIN | MGGX_AGG_RELU));
-    if (plan->num_empty > 0 && touch_empty) {
-        const long long n = (long long)plan->num_empty * dim;
-        k_agg_empty_rows<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(a, plan->d_empty_rows, plan->num_empty);
-        MGGX_LAUNCH_CHECK("k_agg_empty_rows");
     }
     if (blocked) {
-        AggArgs r = a;  // the real output and epilogue
+        // one kernel finishes a column-blocked call: per-block partial rows and carry chains summed per row, the dense
+        // core's partial rows on top where there are any, then the caller's epilogue
+        AggArgs r = a;
         const float *part = a.out;
         r.out = d_out;
         r.ld_out = ld_out;
         r.rs_out = o.d_row_scale_out;
         r.flags = o.flags;
-        const bool vec4 = dim % 4 == 0 && ld_out % 4 == 0 && aligned16(d_out) && !(o.flags & MGGX_AGG_GIN);
-        if (vec4) {
-            const long long n = (long long)plan->real_rows * (dim / 4);
-            k_agg_block_reduce4<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(r, part, plan->real_rows, plan->blocks, ldp);
-        } else {
-            const long long n = (long long)plan->real_rows * dim;
-            k_agg_block_reduce<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(r, part, plan->real_rows, plan->blocks, ldp);
+        CoreMergeArgs cma{nullptr, nullptr, 0, 0};
+        if (cm) {
+            MGGX_HIP(hipStreamWaitEvent(st.stream, cm->join, 0));
+            cma = CoreMergeArgs{cm->partial, cm->rank, cm->core, cm->nseg};
+            cm->merged = true;
         }
-        MGGX_LAUNCH_CHECK("k_agg_block_reduce");
+        const int G = pow2_ceil((dim + 3) / 4);
+        const long long n = (long long)plan->real_rows * G;
+        k_agg_finish_blocked<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(r, part, plan->real_rows, plan->blocks, ldp, G, cma);
+        MGGX_LAUNCH_CHECK("k_agg_finish_blocked");
+    } else {
+        // rows that cross workgroups and rows without neighbors, in one launch
+        const bool touch_empty = !(o.flags & MGGX_AGG_ACCUMULATE) || (o.flags & (MGGX_AGG_GIN | MGGX_AGG_RELU | MGGX_AGG_SOFTMAX));
+        const int n_empty = touch_empty ? plan->num_empty : 0;
+        const int comp_lanes = dim >= 64 ? 64 : pow2_ceil(dim);
+        const long long per_block = 4 * (64 / comp_lanes);
+        const long long fix_blocks = num_wg > 1 ? (num_wg - 1 + per_block - 1) / per_block : 0;
+        const long long empty_blocks = (n_empty + per_block - 1) / per_block;
+        if (fix_blocks + empty_blocks > 0) {
+            k_agg_tail<<<dim3((unsigned)(fix_blocks + empty_blocks)), dim3(256), 0, st.stream>>>(a, (int)num_wg, comp_lanes, (int)fix_blocks,
+                                                                                               plan->d_empty_rows, n_empty);
+            MGGX_LAUNCH_CHECK("k_agg_tail");
+        }
     }
     snprintf(st.last_kernel, sizeof(st.last_kernel), "k_agg<%d,%d,%d> grid=%lld block=%d parts=%d blocks=%d ps=%d wpb=%d dist=%d", lpr, mode, (int)buf,
              num_wg, 64 * wpb, plan->num_parts, plan->blocks, plan->ps, wpb, dist);
@@ -905,7 +1023,7 @@ int resolve_knobs(GraphInfo &g, int dim, int dtype, int ps, int wpb, int dist, i
 
 // `gate`: the call's content check of the caller's CSR arrays; every kernel launched below looks at it first.
 int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in_local, const void *d_in_remote, const int *d_ptr_l,
-              const int *d_col_l, const int *d_ptr_r, const int *d_col_r, int lb, int ub, int dim, const mggx_agg_opts &o, const Gate &gate)
+              const int *d_col_l, const int *d_ptr_r, const int *d_col_r, int lb, int ub, int dim, const mggx_agg_opts &o, const Gate &gate, CoreMerge *cm = nullptr)
 {
     Plan *plan = nullptr;
     int rc;
@@ -916,8 +1034,10 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
         if (rc) return rc;
         if (!cp->unsuitable) {
             // The core block is bound by the LDS, the rest of the CSR by the caches: they run side by side.  The core's sums
-            // go to partial rows on a second stream; the rest of the CSR runs here with the caller's epilogue except the
-            // ReLU; then the partial rows are added (with the row scale) and the ReLU comes last.
+            // go to partial rows on a second stream while the rest of the CSR runs here.  Where that rest ends in the finish
+            // kernel of a column-blocked plan, the same kernel joins the side stream, adds the core's partial rows and
+            // applies the caller's epilogue; otherwise the rest runs with the epilogue except its post-operations (ReLU,
+            // softmax), and k_core_finish adds the partial rows (times the row scale) and applies those last.
             const long long ld_in = o.ld_in ? o.ld_in : dim, ld_out = o.ld_out ? o.ld_out : dim;
             if (ld_in < dim || ld_out < dim) return fail(MGGX_EINVAL, "aggregation: row stride smaller than dim");
             State &st0 = state();
@@ -933,26 +1053,29 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
             const hipError_t er = hipEventRecord(join, side);
             int rc2 = MGGX_OK;
             GraphInfo *gr = nullptr;
-            if (!rc) rc2 = graph_info(cp->d_rem_ptr, nullptr, cp->d_rem_col, nullptr, ub - lb, true, &gr);
-            if (!rc && !rc2) {
-                mggx_agg_opts o2 = o;
-                o2.flags &= ~MGGX_AGG_RELU;
+            CoreMerge cm{nullptr, cp->d_rank, cp->core, cp->nseg, join, false};
+            if (!rc) rc2 = core_partial_rows(cp, dim, &cm.partial);
+            if (!rc && !rc2) rc2 = graph_info(cp->d_rem_ptr, nullptr, cp->d_rem_col, nullptr, ub - lb, true, &gr);
+            if (!rc && !rc2 && er == hipSuccess) {
                 Knobs k2 = k;
                 k2.core_rows = -1;
                 if (k2.block_rows > 0 && !blocking_eligible(*gr, k2.block_rows)) k2.block_rows = -1;
-                rc2 = run_knobs(*gr, k2, d_out, d_in_local, nullptr, cp->d_rem_ptr, cp->d_rem_col, nullptr, nullptr, lb, ub, dim, o2, gate);
+                rc2 = run_knobs(*gr, k2, d_out, d_in_local, nullptr, cp->d_rem_ptr, cp->d_rem_col, nullptr, nullptr, lb, ub, dim, o, gate, &cm);
             }
             // the caller's stream takes the side stream back in whatever happened, so no work of this call outlives it unordered
-            const hipError_t ew = er == hipSuccess ? hipStreamWaitEvent(st0.stream, join, 0) : er;
+            const hipError_t ew = er == hipSuccess ? (cm.merged ? hipSuccess : hipStreamWaitEvent(st0.stream, join, 0)) : er;
             if (rc) return rc;
             if (rc2) return rc2;
             if (ew != hipSuccess) return fail(MGGX_EHIP, "aggregation: joining the side stream: %s", hipGetErrorString(ew));
-            rc = run_core_finish(cp, d_out, dim, ld_out, o.d_row_scale_out, (o.flags & MGGX_AGG_RELU) ? 1 : 0, gate, st0.stream);
-            if (rc) return rc;
+            if (!cm.merged) {
+                rc = run_core_finish(cp, d_out, dim, ld_out, o.d_row_scale_out, (o.flags & MGGX_AGG_RELU) ? 1 : 0, (o.flags & MGGX_AGG_SOFTMAX) ? 1 : 0, gate,
+                                     st0.stream);
+                if (rc) return rc;
+            }
             State &st = state();
             const size_t n = strlen(st.last_kernel);
-            snprintf(st.last_kernel + n, sizeof(st.last_kernel) - n, " core=%d core_nnz=%lld rem_nnz=%lld", cp->core, (long long)cp->core_nnz,
-                     (long long)cp->rem_nnz);
+            snprintf(st.last_kernel + n, sizeof(st.last_kernel) - n, " core=%d core_nnz=%lld rem_nnz=%lld%s", cp->core, (long long)cp->core_nnz,
+                     (long long)cp->rem_nnz, cm.merged ? " merged_finish" : "");
             return MGGX_OK;
         }
     }
@@ -965,7 +1088,7 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
         rc = plan_get(d_ptr_l, d_ptr_r, d_col_r, ub - lb, k.ps, &plan);
         if (rc) return rc;
     }
-    return run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, k.wpb, k.dist, o, gate);
+    return run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, k.wpb, k.dist, o, gate, nullptr, cm);
 }
 
 int check_np_div_args(const char *who, const int *d_ptr_l, int lb, int ub, int nodes_per_pe, int &ps, int block_rows, int core_rows)

@@ -103,49 +103,63 @@ __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *_
 }
 
 // Adds the core block's sums to output rows that already hold the rest of the aggregation:
-// out[v][d] = act(out[v][d] + scale[v] * sum over segments of the partial rows of v).  all_rows = 0: one thread per
-// element of the core rows only (idx -> rank -> row); all_rows = 1: every row (needed when act is the ReLU).
-__global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, const float *__restrict__ partial, const int *__restrict__ rank,
+// out[v] = post(out[v] + scale[v] * sum over segments of the partial rows of v), post = ReLU and / or row softmax.
+// G lanes per row (a power of two >= ceil(dim/4)), lane q holds columns 4 q .. 4 q + 3.  all_rows = 0: the core rows only
+// (index -> rank -> row); all_rows = 1: every row (needed when there is a post-operation).
+__global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, const v4f *__restrict__ partial, const int *__restrict__ rank,
                                                      const int *__restrict__ order, const float *__restrict__ rs, int rows, int dim,
-                                                     long long ld_out, int core, int n4, int nseg, int relu, int all_rows, const Gate gate)
+                                                     long long ld_out, int core, int nseg, int G, int relu, int softmax, int all_rows, const Gate gate)
 {
     if (gate_closed(gate)) return;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (long long)(all_rows ? rows : core) * dim) return;
-    const int i = (int)(idx / dim), d = (int)(idx % dim);
+    const long long i_ll = idx / G;
+    const int q = (int)(idx % G), n4 = (dim + 3) >> 2;
+    if (i_ll >= (all_rows ? rows : core)) return;  // G divides 64: the lanes of a row leave together
+    const int i = (int)i_ll;
     const int v = all_rows ? i : order[i];
     const int r = all_rows ? rank[i] : i;
-    float sum = 0.f;
-    if (r >= 0) {
-        for (int seg = 0; seg < nseg; ++seg) sum += partial[(((size_t)seg * core + r) * n4 + (d >> 2)) * 4 + (d & 3)];
-        if (rs) sum *= rs[v];
+    const bool lane_on = q < n4;
+    float val[4] = {0.f, 0.f, 0.f, 0.f};
+    bool on[4];
+    float *o = out + (long long)v * ld_out + 4 * q;
+    if (lane_on) {
+        v4f sum = {0.f, 0.f, 0.f, 0.f};
+        if (r >= 0) {
+            for (int seg = 0; seg < nseg; ++seg) sum += partial[((size_t)seg * core + r) * n4 + q];
+            if (rs) sum *= rs[v];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            on[j] = 4 * q + j < dim;
+            val[j] = on[j] ? o[j] + sum[j] : 0.f;
+            if (relu) val[j] = fmaxf(val[j], 0.f);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) on[j] = false;
     }
-    float *o = out + (long long)v * ld_out + d;
-    float t = *o + sum;
-    if (relu) t = fmaxf(t, 0.f);
-    *o = t;
-}
-
-// The same, four columns per thread, where the output rows take 16-byte accesses.
-__global__ void __launch_bounds__(256) k_core_finish4(float *__restrict__ out, const v4f *__restrict__ partial, const int *__restrict__ rank,
-                                                      const int *__restrict__ order, const float *__restrict__ rs, int rows, int n4,
-                                                      long long ld_out, int core, int nseg, int relu, int all_rows, const Gate gate)
-{
-    if (gate_closed(gate)) return;
-    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (long long)(all_rows ? rows : core) * n4) return;
-    const int i = (int)(idx / n4), q = (int)(idx % n4);
-    const int v = all_rows ? i : order[i];
-    const int r = all_rows ? rank[i] : i;
-    v4f sum = {0.f, 0.f, 0.f, 0.f};
-    if (r >= 0) {
-        for (int seg = 0; seg < nseg; ++seg) sum += partial[((size_t)seg * core + r) * n4 + q];
-        if (rs) sum *= rs[v];
+    if (softmax) {
+        const int lane = (int)(threadIdx.x & 63u);
+        float m = -3.0e38f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) m = on[j] ? fmaxf(m, val[j]) : m;
+        for (int s = 1; s < G; s <<= 1) m = fmaxf(m, __shfl(m, lane ^ s, 64));
+        float tot = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            val[j] = on[j] ? __expf(val[j] - m) : 0.f;
+            tot += val[j];
+        }
+        for (int s = 1; s < G; s <<= 1) tot += __shfl(tot, lane ^ s, 64);
+        const float inv = 1.0f / tot;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) val[j] *= inv;
     }
-    v4f *o = reinterpret_cast<v4f *>(out + (long long)v * ld_out + 4 * q);
-    v4f t = *o + sum;
-    if (relu) { t.x = fmaxf(t.x, 0.f); t.y = fmaxf(t.y, 0.f); t.z = fmaxf(t.z, 0.f); t.w = fmaxf(t.w, 0.f); }
-    *o = t;
+    if (lane_on) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (on[j]) o[j] = val[j];
+    }
 }
 
 // ---- the plan, built on the GPU (same arrays, bit for bit, as core_layout_build makes on the host) ----
@@ -546,26 +560,31 @@ int run_core_sums(CorePlan *p, int dim, const Gate &gate, hipStream_t stream)
     return rc;
 }
 
-// out += scale * (partial rows of the core), then the ReLU if asked for, on `stream`.
-int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, const Gate &gate, hipStream_t stream)
+// out += scale * (partial rows of the core), then the ReLU and / or the row softmax if asked for, on `stream`.
+int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, int softmax, const Gate &gate,
+                    hipStream_t stream)
 {
     const int n4 = (dim + 3) / 4;
     v4f *tab = nullptr, *partial = nullptr;
     int rc = core_scratch(p, n4, &tab, &partial);  // sized by run_core_sums already: only hands the pointers out
     if (rc) return rc;
-    const int all_rows = relu ? 1 : 0;
-    const long long nrows = all_rows ? p->rows : p->core;
-    if (dim % 4 == 0 && ld_out % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0) {
-        const long long n = nrows * n4;
-        k_core_finish4<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(d_out, partial, p->d_rank, p->d_order, d_row_scale, p->rows, n4,
-                                                                                     ld_out, p->core, p->nseg, relu, all_rows, gate);
-    } else {
-        const long long n = nrows * dim;
-        k_core_finish<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(d_out, reinterpret_cast<const float *>(partial), p->d_rank,
-                                                                                    p->d_order, d_row_scale, p->rows, dim, ld_out, p->core, n4,
-                                                                                    p->nseg, relu, all_rows, gate);
-    }
+    const int all_rows = (relu || softmax) ? 1 : 0;
+    int G = 1;
+    while (G < n4) G <<= 1;
+    const long long n = (long long)(all_rows ? p->rows : p->core) * G;
+    k_core_finish<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(d_out, partial, p->d_rank, p->d_order, d_row_scale, p->rows, dim, ld_out,
+                                                                                p->core, p->nseg, G, relu, softmax, all_rows, gate);
     MGGX_LAUNCH_CHECK("k_core_finish");
+    return MGGX_OK;
+}
+
+int core_partial_rows(CorePlan *p, int dim, const float4 **partial_out)
+{
+    const int n4 = (dim + 3) / 4;
+    v4f *tab = nullptr, *partial = nullptr;
+    const int rc = core_scratch(p, n4, &tab, &partial);
+    if (rc) return rc;
+    *partial_out = reinterpret_cast<const float4 *>(partial);
     return MGGX_OK;
 }
 

@@ -218,7 +218,10 @@ int predict_core_rows(GraphInfo &g, int dim, unsigned long long table_bytes, int
 void core_plan_free(CorePlan *p);
 int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, const Gate &gate, hipStream_t stream);
 int run_core_sums(CorePlan *p, int dim, const Gate &gate, hipStream_t stream);
-int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, const Gate &gate, hipStream_t stream);
+int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, int softmax, const Gate &gate,
+                    hipStream_t stream);
+// Where run_core_sums leaves the core block's sums: [segment][rank][ceil(dim/4)] float4.
+int core_partial_rows(CorePlan *p, int dim, const float4 **partial);
 // Second stream of the dense-core path (created on first use, default priority) and the two events that fork and join it.
 int core_side_stream(hipStream_t *stream, hipEvent_t *fork, hipEvent_t *join);
 

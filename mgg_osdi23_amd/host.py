@@ -19,6 +19,7 @@ LIB_PATH = os.path.join(_PKG, "libmggx.so")
 AGG_ACCUMULATE = 1
 AGG_GIN = 2
 AGG_RELU = 4
+AGG_SOFTMAX = 8
 F32 = 0
 BF16 = 1
 
@@ -389,11 +390,12 @@ def tune_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, c
 
 def mgg_SAG_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb, ub, dim,
                    nodePerPE, peid, np_size, warpPerBlock, interleaved_dist, *, input_remote=None, accumulate=False,
-                   ld_in=0, ld_out=0, row_scale_out=None, relu=False, col_block_rows=0, core_rows=0):
+                   ld_in=0, ld_out=0, row_scale_out=None, relu=False, softmax=False, col_block_rows=0, core_rows=0):
     """Argument order of the reference's mgg_SAG_np_div.  `input` is this rank's table; `input_remote` the
     global-id-indexed table the reference reaches with remote GETs (defaults to `input`, the single-GPU case).
-    The reference adds into `output`; pass accumulate=True for that, the default overwrites."""
-    flags = (AGG_ACCUMULATE if accumulate else 0) | (AGG_RELU if relu else 0)
+    The reference adds into `output`; pass accumulate=True for that, the default overwrites.  softmax=True applies the row
+    softmax of the reference's last layer (softmax_forward) inside the same call."""
+    flags = (AGG_ACCUMULATE if accumulate else 0) | (AGG_RELU if relu else 0) | (AGG_SOFTMAX if softmax else 0)
     _agg(output, input, input_remote if input_remote is not None else input, row_pointers_l, column_index_l,
          row_pointers_r, column_index_r, lb, ub, dim, nodePerPE, np_size, warpPerBlock, interleaved_dist, flags, 0.0,
          ld_in, ld_out, row_scale_out, col_block_rows, core_rows)

@@ -841,3 +841,62 @@ def test_dense_update_bf16(gpu, n, d1, d2, x_bf16, out_bf16):
     want_f = orc.dense(x, w, f64=True)
     mag_f = np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64)
     assert_close_to_oracle(got, want_f, mag_f, BF16_TOL, "bf16 MFMA vs unrounded inputs")
+
+
+# --------------------------------------------------------------------------- softmax inside the aggregation
+def _softmax_want(sh, xl, x, dim, s):
+    """softmax_forward(aggregate(...)) as the reference runs them back to back (src/mgg_np_div_mem.cu:221-225), in double."""
+    want, mag = oracle_agg(sh, xl, x, dim, rs_out=s)
+    w = want.astype(np.float64)
+    e = np.exp(w - w.max(1, keepdims=True))
+    return e / e.sum(1, keepdims=True), mag
+
+
+@pytest.mark.parametrize("dim,ld", [(16, 16), (41, 41), (41, 48), (47, 47), (100, 100), (7, 7)])
+@pytest.mark.parametrize("path", ["plain", "blocked", "core", "core+blocked"])
+def test_softmax_epilogue_on_every_path(gpu, rmat_graph, dim, ld, path):
+    """MGGX_AGG_SOFTMAX: rows finished inside a slot, across the wavefronts of a workgroup, across workgroups (tiny
+    workgroups force long carry chains), rows without neighbors, the column-blocked finish and both dense-core finishes
+    must all give softmax(row scale x sum) -- against the oracle's aggregation followed by a softmax in double."""
+    import torch
+    if path.startswith("core") and dim > 64:
+        pytest.skip("the dense core takes rows of at most 64 columns")
+    V, ptr0, col0 = rmat_graph
+    if path == "core+blocked":  # dense enough that what the core leaves still has long rows per column block
+        V = 4000
+        ptr0, col0 = gpu.gen_rmat(12, V, 1_500_000, seed=15)
+    # a few rows without neighbors, so the empty-row branch runs
+    deg = np.diff(ptr0)
+    keep = np.ones(V, bool)
+    keep[[5, 77, V - 1]] = False
+    ptr = np.zeros(V + 1, np.int32)
+    ptr[1:] = np.cumsum(np.where(keep, deg, 0))
+    col = np.concatenate([col0[ptr0[v]:ptr0[v + 1]] for v in range(V) if keep[v]]).astype(np.int32)
+    sh = share_of(ptr, col, V, 1, 0)
+    x = (gpu.fill_normal((V, dim), seed=300 + dim) * 0.3).astype(np.float32)
+    s = (1.0 / np.sqrt(np.maximum(np.diff(ptr), 1))).astype(np.float32)
+    want, mag = _softmax_want(sh, x, x, dim, s)
+    xp = np.zeros((V, ld), np.float32)
+    xp[:, :dim] = x
+    d_ptr, d_col, d_x, d_s = to_dev(ptr), to_dev(col), to_dev(xp), to_dev(s)
+    z, zc = torch.zeros(V + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    blk = 1500 if "blocked" in path else -1
+    core = 1024 if path.startswith("core") else -1
+    for ps, wpb, dist in [(16, 4, 2), (4, 1, 1), (16, 8, 16)]:
+        out = torch.full((V, ld), 7.5, device="cuda")
+        gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, z, zc, 0, V, dim, V, 0, ps, wpb, dist, ld_in=ld, ld_out=ld, row_scale_out=d_s, softmax=True,
+                           col_block_rows=blk, core_rows=core)
+        gpu.sync()
+        k = gpu.last_agg_kernel()
+        assert ("core=1024" in k) == (core > 0) and (("blocks=1 " in k + " ") == (blk < 0)), k
+        if path == "core+blocked":
+            assert "merged_finish" in k
+        got = out.cpu().numpy()
+        # d softmax_i / d logit_j is bounded by 1/4: an error of FP32_TOL * mag in the logits gives at most that in the output
+        bound = FP32_TOL * (mag.max(1, keepdims=True) + 1.0)
+        assert np.all(np.abs(got[:, :dim] - want) <= bound), (path, dim, ps, wpb, dist, float(np.abs(got[:, :dim] - want).max()))
+        assert np.allclose(got[:, :dim].sum(1), 1.0, atol=1e-5)
+        if ld > dim:
+            assert np.all(got[:, dim:] == 7.5)  # padding columns are not touched
+        assert np.allclose(got[5, :dim], 1.0 / dim, atol=1e-7)  # a row without neighbors: uniform
+    gpu.forget(d_ptr)
