@@ -243,12 +243,14 @@ __device__ __forceinline__ void store_row16(float *p, float x, float y, float z,
     __builtin_nontemporal_store((v4f_s){x, y, z, w}, reinterpret_cast<v4f_s *>(p));
 }
 
-// Finishes this lane's NV elements of a complete row held in registers.
-template <int LPR, int MODE>
+// Finishes this lane's NV elements of a complete row held in registers.  SMX: the kernel variant that serves calls with
+// the softmax epilogue (a variant of its own: inlined into every kernel, the few registers of this branch cost the wide-row
+// kernels a wavefront of occupancy per SIMD on every call).
+template <int LPR, int MODE, bool SMX>
 __device__ __forceinline__ void finish_row(const AggArgs &a, int row, int l, const float (&acc)[ModeTraits<MODE>::NV])
 {
     constexpr int NV = ModeTraits<MODE>::NV;
-    if (a.flags & MGGX_AGG_SOFTMAX) {  // the slot's LPR lanes hold the whole row: softmax across them, then the store
+    if constexpr (SMX) {  // the slot's LPR lanes hold the whole row: softmax across them, then the store
         float v[NV];
         bool on[NV];
 #pragma unroll
@@ -265,8 +267,14 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int row, int l, con
     }
     if constexpr (MODE == MODE_F32_VEC4) {
         if (a.flags == 0 && a.rs_out == nullptr) {
-            if (NV * l < a.dim)
+            if (NV * l + 3 < a.dim) {
                 store_row16(a.out + (long long)row * a.ld_out + 4 * l, acc[0], acc[1], acc[2], acc[3]);
+            } else if (NV * l < a.dim) {  // the last, partial piece of a row whose width is not a multiple of 4
+                float *o = a.out + (long long)row * a.ld_out + 4 * l;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (4 * l + i < a.dim) o[i] = acc[i];
+            }
             return;
         }
     }
@@ -298,7 +306,14 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int row, int l, con
             if (a.flags & MGGX_AGG_RELU) {
                 v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f);
             }
-            store_row16(reinterpret_cast<float *>(o), v.x, v.y, v.z, v.w);
+            if (NV * l + 3 < a.dim) {
+                store_row16(reinterpret_cast<float *>(o), v.x, v.y, v.z, v.w);
+            } else {
+                const float t[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (4 * l + i < a.dim) reinterpret_cast<float *>(o)[i] = t[i];
+            }
         }
         return;
     }
@@ -311,7 +326,7 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int row, int l, con
 
 // One wavefront-wide aggregation kernel; see the file header for the scheme.
 // Dynamic LDS: int2 hdr[2*wpb] (head, tail per wavefront), then float vals[2*wpb][cpad].
-template <int LPR, int MODE, bool BUF>
+template <int LPR, int MODE, bool BUF, bool SMX>
 __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
 {
     constexpr int NV = ModeTraits<MODE>::NV;
@@ -505,7 +520,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
         bool keep_open = false;
         if (run_last) {
             if (row_done && has_first) {
-                finish_row<LPR, MODE>(a, row, l, acc);
+                finish_row<LPR, MODE, SMX>(a, row, l, acc);
             } else if (!row_done && !last_round) {
                 keep_open = true;  // slot S-1 only: continues in the next round
             } else {
@@ -538,7 +553,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     int orow = -1;
     auto emit = [&](bool ends) {
         if (started && ends) {
-            if (a.flags & MGGX_AGG_SOFTMAX) {
+            if (SMX) {
                 float v[4];
                 bool on[4];
 #pragma unroll
@@ -690,22 +705,36 @@ __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, con
     float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
     const bool lane_on = q < n4;
     if (lane_on) {
-        for (int c = 0; c < blocks; ++c) {
-            const long long vr = (long long)c * rows + v;
-            const int o0 = a.off[vr], o1 = a.off[vr + 1];
-            if (o1 == o0) continue;
-            const int w0 = o0 / a.parts_per_wg, w1 = (o1 - 1) / a.parts_per_wg;
-            float4 p;
-            if (w0 == w1) {
-                p = *reinterpret_cast<const float4 *>(part + vr * ldp + 4 * q);
-            } else {
-                p = *reinterpret_cast<const float4 *>(a.c_val + (size_t)(2 * w0 + 1) * a.cpad + 4 * q);
-                for (int w = w0 + 1; w <= w1; ++w) {
-                    const float4 h = *reinterpret_cast<const float4 *>(a.c_val + (size_t)(2 * w) * a.cpad + 4 * q);
-                    p.x += h.x; p.y += h.y; p.z += h.z; p.w += h.w;
-                }
+        // four blocks at a time: their row offsets first, then their partial rows, all in flight before the first sum
+        for (int c0 = 0; c0 < blocks; c0 += 4) {
+            int o0[4], o1[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const long long vr = (long long)min(c0 + j, blocks - 1) * rows + v;
+                o0[j] = a.off[vr];
+                o1[j] = a.off[vr + 1];
             }
-            t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
+            float4 p[4];
+            bool chain[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool there = c0 + j < blocks && o1[j] > o0[j];
+                chain[j] = there && o0[j] / a.parts_per_wg != (o1[j] - 1) / a.parts_per_wg;
+                p[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (there && !chain[j]) p[j] = *reinterpret_cast<const float4 *>(part + ((long long)(c0 + j) * rows + v) * ldp + 4 * q);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (chain[j]) {  // the row crossed workgroups in this block: tail entry of the first, head entries of the others
+                    const int w0 = o0[j] / a.parts_per_wg, w1 = (o1[j] - 1) / a.parts_per_wg;
+                    p[j] = *reinterpret_cast<const float4 *>(a.c_val + (size_t)(2 * w0 + 1) * a.cpad + 4 * q);
+                    for (int w = w0 + 1; w <= w1; ++w) {
+                        const float4 h = *reinterpret_cast<const float4 *>(a.c_val + (size_t)(2 * w) * a.cpad + 4 * q);
+                        p[j].x += h.x; p[j].y += h.y; p[j].z += h.z; p[j].w += h.w;
+                    }
+                }
+                t.x += p[j].x; t.y += p[j].y; t.z += p[j].z; t.w += p[j].w;
+            }
         }
         if (cm.partial) {
             const int r = cm.rank[v];
@@ -743,13 +772,13 @@ int pow2_ceil(int x)
     return p;
 }
 
-template <int MODE, bool BUF>
+template <int MODE, bool BUF, bool SMX>
 int launch_agg(int lpr, dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream, const AggArgs &a)
 {
     switch (lpr) {
 #define MGGX_CASE(L)                                                      \
     case L:                                                               \
-        k_agg<L, MODE, BUF><<<grid, block, lds_bytes, stream>>>(a);       \
+        k_agg<L, MODE, BUF, SMX><<<grid, block, lds_bytes, stream>>>(a);  \
         break;
         MGGX_CASE(1)
         MGGX_CASE(2)
@@ -807,11 +836,16 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     if (o.in_dtype == MGGX_BF16) {
         if (dim % 8 || ld_in % 8 || ld_out % 4 || !aligned16(d_in_l) || (d_in_r && !aligned16(d_in_r)) || !aligned16(d_out))
             return fail(MGGX_EINVAL, "aggregation: bf16 tables need dim %% 8 == 0, ld_in %% 8 == 0 and 16-byte alignment");
+        if (o.flags & MGGX_AGG_SOFTMAX) return fail(MGGX_EINVAL, "aggregation: the softmax epilogue takes fp32 tables (the last layer's logits)");
         mode = MODE_BF16_VEC8;
         lpr = pow2_ceil(dim / 8);
     } else if (o.in_dtype == MGGX_F32) {
-        const bool out_ok = blocked || (ld_out % 4 == 0 && aligned16(d_out));  // blocked plans write their own partial rows
-        const bool vec = dim % 4 == 0 && ld_in % 4 == 0 && out_ok && aligned16(d_in_l) && (!d_in_r || aligned16(d_in_r));
+        // 16-byte accesses per lane wherever the tables allow them: rows that start on 16-byte boundaries and are at least
+        // ceil(dim/4) pieces long (a width that is not a multiple of 4 reads up to three padding columns of its own row
+        // pitch and never stores them)
+        const long long dim4 = (dim + 3) & ~3;
+        const bool out_ok = blocked || (ld_out % 4 == 0 && ld_out >= dim4 && aligned16(d_out));  // blocked plans write their own partial rows
+        const bool vec = ld_in % 4 == 0 && ld_in >= dim4 && out_ok && aligned16(d_in_l) && (!d_in_r || aligned16(d_in_r));
         mode = vec ? MODE_F32_VEC4 : MODE_F32_STRIDED;
         lpr = pow2_ceil((dim + 3) / 4);
     } else {
@@ -913,14 +947,19 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         }
         const size_t lds_bytes = (size_t)wpb * 2 * sizeof(int2) + (size_t)wpb * 2 * cpad * sizeof(float);
         const dim3 grid((unsigned)num_wg), block((unsigned)(64 * wpb));
+        const bool smx = (a.flags & MGGX_AGG_SOFTMAX) != 0;  // fp32 tables only (checked above)
         if (buf) {
-            if (mode == MODE_F32_VEC4) rc = launch_agg<MODE_F32_VEC4, true>(lpr, grid, block, lds_bytes, st.stream, a);
-            else if (mode == MODE_F32_STRIDED) rc = launch_agg<MODE_F32_STRIDED, true>(lpr, grid, block, lds_bytes, st.stream, a);
-            else rc = launch_agg<MODE_BF16_VEC8, true>(lpr, grid, block, lds_bytes, st.stream, a);
+            if (mode == MODE_F32_VEC4) rc = smx ? launch_agg<MODE_F32_VEC4, true, true>(lpr, grid, block, lds_bytes, st.stream, a)
+                                                : launch_agg<MODE_F32_VEC4, true, false>(lpr, grid, block, lds_bytes, st.stream, a);
+            else if (mode == MODE_F32_STRIDED) rc = smx ? launch_agg<MODE_F32_STRIDED, true, true>(lpr, grid, block, lds_bytes, st.stream, a)
+                                                        : launch_agg<MODE_F32_STRIDED, true, false>(lpr, grid, block, lds_bytes, st.stream, a);
+            else rc = launch_agg<MODE_BF16_VEC8, true, false>(lpr, grid, block, lds_bytes, st.stream, a);
         } else {
-            if (mode == MODE_F32_VEC4) rc = launch_agg<MODE_F32_VEC4, false>(lpr, grid, block, lds_bytes, st.stream, a);
-            else if (mode == MODE_F32_STRIDED) rc = launch_agg<MODE_F32_STRIDED, false>(lpr, grid, block, lds_bytes, st.stream, a);
-            else rc = launch_agg<MODE_BF16_VEC8, false>(lpr, grid, block, lds_bytes, st.stream, a);
+            if (mode == MODE_F32_VEC4) rc = smx ? launch_agg<MODE_F32_VEC4, false, true>(lpr, grid, block, lds_bytes, st.stream, a)
+                                                : launch_agg<MODE_F32_VEC4, false, false>(lpr, grid, block, lds_bytes, st.stream, a);
+            else if (mode == MODE_F32_STRIDED) rc = smx ? launch_agg<MODE_F32_STRIDED, false, true>(lpr, grid, block, lds_bytes, st.stream, a)
+                                                        : launch_agg<MODE_F32_STRIDED, false, false>(lpr, grid, block, lds_bytes, st.stream, a);
+            else rc = launch_agg<MODE_BF16_VEC8, false, false>(lpr, grid, block, lds_bytes, st.stream, a);
         }
         if (rc) return rc;
         MGGX_LAUNCH_CHECK("k_agg");

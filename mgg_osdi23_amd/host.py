@@ -363,15 +363,15 @@ def _agg(out, in_local, in_remote, ptr_l, col_l, ptr_r, col_r, lb, ub, dim, npp,
 
 
 def tune_np_div(output, input, row_pointers_l, column_index_l, row_pointers_r, column_index_r, lb, ub, dim, nodePerPE,
-                np_size, *, input_remote=None, gin_eps=None, ld_in=0, ld_out=0, row_scale_out=None, relu=False, col_block_rows=0,
-                core_rows=0):
+                np_size, *, input_remote=None, gin_eps=None, ld_in=0, ld_out=0, row_scale_out=None, relu=False, softmax=False,
+                col_block_rows=0, core_rows=0):
     """The search of the reference's bench_MGG_DSE_dist_ps.py / bench_MGG_DSE_dist_wpb.py in one call: times
     partSize (as given, or 16 and 32 when 0) x plain / column-blocked order x without / with a dense core x warpPerBlock x
     interleaved_dist on this input, returns ({"ps", "wpb", "dist", "col_block_rows", "core_rows"}, ms) of the fastest and makes later calls that leave the
     knobs at 0 on the same CSR tensors use it."""
     import torch
     o = _AggOpts()
-    o.flags = (AGG_RELU if relu else 0) | (AGG_GIN if gin_eps is not None else 0)
+    o.flags = (AGG_RELU if relu else 0) | (AGG_GIN if gin_eps is not None else 0) | (AGG_SOFTMAX if softmax else 0)
     o.eps = float(gin_eps or 0.0)
     o.ld_in = ld_in
     o.ld_out = ld_out
