@@ -241,8 +241,8 @@ __global__ void __launch_bounds__(256) k_core_widths(const unsigned short *__res
 
 // Pass 2, one wavefront per row, 64 neighbors at a time in edge order: neighbors that stay go to the remaining CSR (order
 // kept); a core row's core neighbors go to the list of their tile, the k-th of a tile (in edge order) to list position k.
-// Inside a group of 64 every lane counts the lanes before it with the same tile (64 lane reads, no memory); the counts so
-// far per tile and the row's block offsets sit in LDS, so the loop over a long row never waits for global memory.
+// Inside a group of 64 every lane finds the lanes with the same tile by one ballot per bit of the tile number; the counts
+// so far per tile and the row's block offsets sit in LDS, and the next group's ids and ranks are fetched ahead.
 __global__ void __launch_bounds__(BUILD_WAVES * 64) k_core_fill(const int *__restrict__ ptr, const int *__restrict__ col,
                                                                 const int *__restrict__ rank, int rows, int lb, int ntiles, int tc,
                                                                 const int *__restrict__ blk_off, const int *__restrict__ rem_ptr,
@@ -253,6 +253,8 @@ __global__ void __launch_bounds__(BUILD_WAVES * 64) k_core_fill(const int *__res
     volatile int *cur = fill_lds + (size_t)wave * 2 * ntiles;
     volatile int *blk = cur + ntiles;
     const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    int tile_bits = 0;
+    while ((1 << tile_bits) < ntiles) ++tile_bits;
     for (long long v = (long long)blockIdx.x * BUILD_WAVES + wave; v < rows; v += (long long)gridDim.x * BUILD_WAVES) {
         const int i = rank[v];
         const int beg = ptr[v], end = ptr[v + 1];
@@ -267,29 +269,37 @@ __global__ void __launch_bounds__(BUILD_WAVES * 64) k_core_fill(const int *__res
             blk[t] = blk_off[row_blocks + t];
         }
         const size_t lane_base = (size_t)(i % 64) * 4;
+        // the next group's neighbor ids and their ranks are fetched while the current group is placed: a long row is one
+        // wavefront's work from end to end, and without this every group would wait for two trips to memory
+        int c_next = beg + lane < end ? col[beg + lane] : 0;
+        int j_next = beg + lane < end ? rank[c_next - lb] : -1;
         for (int e0 = beg; e0 < end; e0 += 64) {
             const int e = e0 + lane;
             const bool valid = e < end;
-            const int c = valid ? col[e] : 0;
-            const int j = valid ? rank[c - lb] : -1;
+            const int c = c_next, j = j_next;
+            if (e0 + 64 < end) {
+                const int en = e + 64;
+                c_next = en < end ? col[en] : 0;
+                j_next = en < end ? rank[c_next - lb] : -1;
+            }
             const bool in_core = valid && j >= 0;
             const unsigned long long stay = __ballot(valid && !in_core);
             if (valid && !in_core) rem_col[w + __popcll(stay & below)] = c;
             w += __popcll(stay);
             if (!__any(in_core)) continue;
-            const int t = in_core ? j / tc : -1 - lane;  // lanes without a core neighbor match nobody
-            int before = 0, after = 0;
-#pragma unroll
-            for (int l = 0; l < 64; ++l) {
-                const int tl = __builtin_amdgcn_readlane(t, l);
-                before += (tl == t && l < lane) ? 1 : 0;
-                after += (tl == t && l > lane) ? 1 : 0;
+            // the lanes of this group with the same tile as this lane: one ballot per bit of the tile number
+            const int t = in_core ? j / tc : 0;
+            unsigned long long same = __ballot(in_core);
+            for (int b = 0; b < tile_bits; ++b) {
+                const bool bit = (t >> b) & 1;
+                const unsigned long long m = __ballot(bit);
+                same &= bit ? m : ~m;
             }
             if (in_core) {
-                const int k = cur[t] + before;
+                const int k = cur[t] + __popcll(same & below);
                 const size_t chunk = (size_t)blk[t] + (size_t)(k / 4);
                 idx[chunk * 256 + lane_base + (size_t)(k % 4)] = (unsigned short)(j % tc);
-                if (after == 0) cur[t] = k + 1;  // the last lane of its tile in this group
+                if ((same & ~below & ~(1ull << lane)) == 0) cur[t] = k + 1;  // the last lane of its tile in this group
             }
         }
     }
