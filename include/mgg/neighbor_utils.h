@@ -31,6 +31,7 @@ struct mgg_runtime_options {
     bool synchronize = true;             // the reference waits for the device after every call (:835)
     int col_block_rows = 0;              // column-blocked partition order: 0 = library decides, -1 = off, N = ids per block
     int core_rows = 0;                   // dense core served from LDS: 0 = library decides, -1 = off, N = rows in the core
+    bool softmax = false;                // mgg_SAG_np_div ends in the row softmax of the last layer (softmax_forward folded in)
 };
 inline mgg_runtime_options &mgg_options()
 {
@@ -123,7 +124,7 @@ inline void mgg_SAG_np_div(float *output, const float *input, const nidType *row
 {
     (void)peid;
     mggx_agg_opts o{};
-    o.flags = mgg_options().accumulate ? MGGX_AGG_ACCUMULATE : 0;
+    o.flags = (mgg_options().accumulate ? MGGX_AGG_ACCUMULATE : 0) | (mgg_options().softmax ? MGGX_AGG_SOFTMAX : 0);
     o.col_block_rows = mgg_options().col_block_rows;
     o.core_rows = mgg_options().core_rows;
     const void *remote = mgg_options().remote_table ? mgg_options().remote_table : input;

@@ -74,9 +74,12 @@ int main(int argc, char *argv[])
                        npp, a.pe, a.partSize, wpb, dist);
         dense_hidden_new_forward(dp2);
         mgg_stage_remote(d_Y2g);
+        // --fuse-softmax: the last aggregation ends in the row softmax (one call instead of two; no second pass over the logits)
+        mgg_options().softmax = a.fuse_softmax && !a.validate;
         mgg_SAG_np_div(d_buff_1, dp2->d_out, s.d_row_ptr_l, s.d_col_ind_l, s.d_row_ptr_r, s.d_col_ind_r, s.lb, s.ub, outdim,
                        npp, a.pe, a.partSize, wpb, dist);
-        if (!a.validate) softmax_new_forward(smx2);
+        mgg_options().softmax = false;
+        if (!a.validate && !a.fuse_softmax) softmax_new_forward(smx2);
     };
 
     forward();  // builds the partition plan, warms up

@@ -223,6 +223,27 @@ def test_harness_programs_with_the_search(gpu, graph_files, prog, dims):
     assert re.search(r"Validation on PE-\{0\}, status: True", r.stdout), r.stdout
 
 
+def test_harness_compact_remote_and_fused_softmax(gpu, graph_files):
+    """--compact-remote: the aggregation-only program stages one row per distinct remote id (most referenced first) and
+    still passes the all-ones validation on a 4-way share; --fuse-softmax: the 2-layer program ends its last aggregation
+    in the softmax and logs like the plain run."""
+    files, ptr, col = graph_files
+    exe = os.path.join(BIN, "mgg_np_div_kernel")
+    cmd = [exe] + files + ["4", "16", "4", "2", "16", "16", "16", "--pe", "1", "--iters", "3", "--validate", "--compact-remote"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    m = re.search(r"Compact staging: (\d+) distinct remote rows of (\d+) remote neighbors", r.stdout)
+    assert m and 0 < int(m.group(1)) < int(m.group(2)), r.stdout
+    assert re.search(r"Validation on PE-\{1\}, status: True", r.stdout), r.stdout
+    assert re.search(r"MPI time \(ms\) ([0-9.]+)", r.stdout)
+    exe = os.path.join(BIN, "mgg_np_div_mem")
+    for extra in ([], ["--fuse-softmax"]):
+        cmd = [exe] + files + ["1", "16", "4", "2", "6", "8", "4", "--iters", "3", "--validate"] + extra
+        r = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0, r.stdout + r.stderr
+        assert re.search(r"Validation on PE-\{0\}, status: True", r.stdout) and re.search(r"MPI time \(ms\) ([0-9.]+)", r.stdout), r.stdout
+
+
 def test_cpp_layer_entry_points(gpu, tmp_path):
     """mgg_api_check calls every function and class of include/mgg/*.h from C++ (loaders, split_CSR, build_part,
     mgg_SAG_np_div, mgg_GIN_np_div, SAG_host, SAG_host_fused_interleaved, sparse_*/dense_*/softmax_* layer objects, the
