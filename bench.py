@@ -47,6 +47,24 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def hbm_roofline(kernel, nbytes, ms, traffic):
+    """Roofline object of an aggregation kernel against the HBM peak.  achieved = algorithmic bytes / time.  Where hub
+    rows are served from the caches that ratio can pass the peak and bounds nothing: `frac` is then taken from the measured
+    HBM-side traffic of the same kernel (committed counter runs), and the algorithmic ratio is given under its own name."""
+    achieved = nbytes / (ms * 1e-3) / 1e9
+    r = {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+         "algorithmic_bytes": nbytes, "avg_launch_ms": round(ms, 4), **traffic}
+    ratio = achieved / HBM_PEAK_GBPS
+    if ratio <= 1.0:
+        r["frac"] = round(ratio, 4)
+    else:
+        r["algorithmic_gbps_over_hbm_peak"] = round(ratio, 4)
+        t = traffic.get("traffic")
+        r["frac"] = round(t / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4) if t else None
+        r["frac_is"] = "measured HBM-side traffic / time / peak: the algorithmic ratio exceeds 1 because hub rows are served from L2"
+    return r
+
+
 def agg_bytes(nnz, rows, dim, s_in=4, ptr_arrays=1, gin=False):
     """Algorithmic bytes of one aggregation call: per edge one index and one feature row, per row one output
     row and the row pointers; no cache credit."""
@@ -170,11 +188,12 @@ MEASURED_TRAFFIC = {
     "gcn2_agg1": (6_481_731_891, (4, 16)),
     "gcn2_agg2_blocked": (7_519_810_150, (4, 16)),   # column blocks of 49152 ids: partial rows and their reduction included
     "gcn2_agg1_blocked": (1_746_502_963, (4, 16)),
-    "gcn2_agg2_core32768_blocked": (6_186_012_569, (4, 16)),
-    "gcn2_agg1_core32768_blocked": (1_653_667_737, (4, 16)),
+    "gcn2_agg2_core32768_blocked": (6_275_730_022, (4, 16)),   # dense core of 32768 rows beside the column-blocked rest, one finish kernel (softmax inside)
+    "gcn2_agg1_core32768_blocked": (1_493_901_312, (4, 8)),
     "gcn2_agg2_core40960_blocked": (5_319_550_054, (4, 8)),   # dense core of 40960 rows from LDS beside the column-blocked rest
     "gcn2_agg1_core40960_blocked": (1_498_319_462, (4, 8)),
-    "share_agg": (1_220_807_373, (8, 1)),
+    "share_agg": (1_220_578_611, (4, 4)),
+    "share_agg_compact": (1_036_854_989, (4, 4)),   # remote rows staged compactly (one row per distinct remote id)
     "gin_agg": (25_550_513_561, (16, 1)),
     "gin_agg_core40960": (19_723_389_132, (8, 4)),   # dense core of 40960 rows from LDS beside the rest
     "big_agg": (60_511_998_361, (4, 16)),
@@ -189,7 +208,7 @@ def load_traffic(kernel_key, args, blk=-1, core=-1):
         if blk != 49152:
             return {"traffic": None}
         kernel_key += "_blocked"
-    if args.small or args.ps != 16 or (kernel_key == "share_agg" and args.share_density != 1) or \
+    if args.small or args.ps != 16 or (kernel_key.startswith("share_agg") and args.share_density != 1) or \
             (kernel_key == "big_agg" and args.big_scale != 0) or kernel_key not in MEASURED_TRAFFIC:
         return {"traffic": None}
     nbytes, (w, d) = MEASURED_TRAFFIC[kernel_key]
@@ -295,6 +314,8 @@ def bench_gcn2(args, torch, host):
     # row-major order, no dense core) and (2) the library's rules alone (no search): both timed in this run, so the
     # price of the searched setting below can be set against what it buys.
     lit = (16, 8, 1, -1, -1)
+    if args.only_headline:
+        return gcn2_headline_only(args, torch, host, forward_stages, names)
     t0 = time.perf_counter()
     for fn in forward_stages(lit, lit):
         fn()
@@ -472,6 +493,19 @@ def bench_gcn2(args, torch, host):
     }
     fail_on_parity(res, checks)
     return res
+
+
+def gcn2_headline_only(args, torch, host, forward_stages, names):
+    """--only-headline: the timed forward of the default run and nothing around it (no literal-knob / rule / search /
+    share / CPU legs), so that a profiler run sees one setting per kernel."""
+    k = (args.ps, args.wpb, args.dist, args.col_block_rows, args.core_rows)
+    stages = forward_stages(k, k)
+    r = time_steps(torch, stages, names, args.steps, args.warmup)
+    return {"metric": "gcn_2layer_fwd_ms", "value": round(r["event_median_ms"], 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(r["wall_ms"], 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "configs[1], the headline forward only; last aggregation: %s" % host.last_agg_kernel()},
+            "detail": {"stage_ms": {n: round(v, 4) for n, v in r["stage_median"].items()}}}
 
 
 def share_inputs(args, torch, host):
@@ -724,9 +758,8 @@ def bench_gin(args, torch, host):
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[2]: 5-layer GIN forward, RMAT V=%d nnz=%d, 100->64->47, 2-layer MLP per layer (%s), eps=0, "
                                "%s" % (V, nnz, "two kernels" if args.unfused_mlp else "one fused kernel", kn)},
-        "roofline": {"bound": "hbm", "kernel": "%sk_agg (GIN, dim 64)" % ("k_core_sell + " if kn.core > 0 else ""), "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("gin_agg", args, kn.blk, kn.core),
-                     "algorithmic_bytes": nbytes, "avg_launch_ms": round(agg_ms, 4)},
+        "roofline": hbm_roofline("%sk_agg (GIN, dim 64)" % ("k_core_sell + " if kn.core > 0 else ""), nbytes, agg_ms,
+                                 load_traffic("gin_agg", args, kn.blk, kn.core)),
         "cpu_baseline": cpu, "parity": parity,
         "detail": {"stage_ms": {k: round(v, 4) for k, v in avg.items()}, "mlp_total_ms": round(mlp_ms, 4)},
     }
@@ -817,9 +850,7 @@ def bench_big(args, torch, host):
         "config": {"workload": "configs[4] / 2^%d: rank-0 1/8 share of RMAT V=%d (scrambled), rows=%d nnz=%d (local %d, remote %d), "
                                "bf16 dim %d, fp32 accumulate, then %dx%d bf16 MFMA update; %s"
                                % (k, V, R, nnz, len(lc), len(rc), dim, dim, dim, kn)},
-        "roofline": {"bound": "hbm", "kernel": "k_agg (bf16 dim 128, local+remote)", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), **load_traffic("big_agg", args, kn.blk, kn.core),
-                     "algorithmic_bytes": nbytes, "avg_launch_ms": round(avg["agg"], 4)},
+        "roofline": hbm_roofline("k_agg (bf16 dim 128, local+remote)", nbytes, avg["agg"], load_traffic("big_agg", args, kn.blk, kn.core)),
         "cpu_baseline": cpu, "parity": parity,
         "detail": {"stage_ms": {k2: round(v, 4) for k2, v in avg.items()},
                    "update_tflops": round(gflop / avg["update"], 2), "update_gbps": round(gemm_bytes / (avg["update"] * 1e-3) / 1e9, 1),
@@ -965,6 +996,7 @@ def main():
     ap.add_argument("--tune", action="store_true", help="time the setting the library's search measures fastest instead of the one its rules and "
                          "cost model choose (gcn2 and share otherwise run the search afterwards, for comparison)")
     ap.add_argument("--no-search", action="store_true", help="gcn2 / share: skip the comparison run of the search")
+    ap.add_argument("--only-headline", action="store_true", help="gcn2: the headline forward only (for profiler runs)")
     ap.add_argument("--no-tune", action="store_true", help="gin / big: use the library's rules instead of its search")
     ap.add_argument("--share-density", type=int, default=1, help="multiplies the number of RMAT draws of --workload share")
     ap.add_argument("--small", action="store_true", help="tiny graph, for a quick functional run")

@@ -613,12 +613,12 @@ int core_partial_rows(CorePlan *p, int dim, const float4 **partial_out)
 //             = ALPHA x ceil(dim/4) / (BETA x 64-byte sectors of a row x (1 or HBM_FACTOR)),
 // constants fitted to sweeps of the core size on the 233 K-node width-16 / width-44 and the 2.45 M-node width-64
 // graphs (ALPHA 1.1 ps per padded 16-byte piece; BETA 9 ps per 64-byte sector of a gathered row while the table fits
-// the 256 MB last-level cache, 1.9 x that beyond).
+// the 256 MB last-level cache, 2.3 x that beyond).
 namespace mggx {
 namespace {
 
 constexpr int PROFILE_SLICES = 1024;  // 65536 ranks
-constexpr double ALPHA_PS = 1.1, BETA_PS = 9.0, HBM_FACTOR = 1.9;
+constexpr double ALPHA_PS = 1.1, BETA_PS = 9.0, HBM_FACTOR = 2.3;
 constexpr unsigned long long LAST_LEVEL_CACHE_BYTES = 256ull << 20;
 constexpr int MODEL_STEP = 4096, MODEL_MAX_CORE = 57344;
 

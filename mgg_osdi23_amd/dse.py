@@ -8,6 +8,14 @@ process on synthetic graphs of the benchmark shapes:
     python -m mgg_osdi23_amd.dse --workload whole --dim 16
 
 Prints ps x wpb (dist = 1) and dist x ps (wpb = 8) tables in ms, GB/s of algorithmic traffic, and the best setting.
+
+    python -m mgg_osdi23_amd.dse --workload whole --dim 44 --ld 48 --mode wd      # wpb x dist at ps 16, everything else by rule
+    python -m mgg_osdi23_amd.dse --workload sparse --dim 64 --gin --mode core     # dense-core size sweep, best of a few wpb x dist
+
+`--mode wd`: the wpb x dist table at ps 16 with the order and the dense core left to the library (its rules and cost
+model), and the time of the all-by-rule call beside the table's best.  `--mode core`: the aggregation time against the
+size of the dense core (no counterpart in the reference), with the entries of the built plans (useful, padded, left to
+the gather kernel) -- the data the library's cost model was fitted to -- and the size the model picks.
 """
 from __future__ import annotations
 
@@ -20,8 +28,9 @@ import numpy as np
 from . import host
 
 
-def build_workload(name: str, dim: int, small: bool):
+def build_workload(name: str, dim: int, small: bool, ld: int = 0, compact: bool = False):
     import torch
+    ld = ld or dim
     if name == "share":
         scale, V, draws, num_gpus = (22, 4_194_304, 52_000_000, 8) if not small else (16, 65_536, 800_000, 8)
         npp, lb, ub = host.range_partition(V, num_gpus, 0)
@@ -38,23 +47,33 @@ def build_workload(name: str, dim: int, small: bool):
         lp, lc = ptr, col
         rp, rc = np.zeros(V + 1, np.int32), np.zeros(0, np.int32)
         rows_tbl = V
-    x = host.fill_normal((rows_tbl, dim), seed=11)
+    x = np.zeros((rows_tbl, ld), np.float32)
+    x[:, :dim] = host.fill_normal((rows_tbl, dim), seed=11)
     dev = "cuda"
     t = lambda a: torch.from_numpy(a).to(dev) if len(a) else torch.zeros(1, dtype=torch.int32, device=dev)
-    w = dict(lb=lb, ub=ub, npp=npp, nnz=len(lc) + len(rc), rows=ub - lb, dim=dim,
+    w = dict(lb=lb, ub=ub, npp=npp, nnz=len(lc) + len(rc), rows=ub - lb, dim=dim, ld=ld,
              xr=torch.from_numpy(x).to(dev), xl=torch.from_numpy(np.ascontiguousarray(x[lb:ub])).to(dev),
              ptr_l=t(lp), col_l=t(lc), ptr_r=t(rp), col_r=t(rc))
-    w["out"] = torch.empty(ub - lb, dim, device=dev)
+    if compact and len(rc):  # the remote rows staged compactly: one row per distinct remote id, most referenced first
+        rcc, ids = host.compact_remote_device(w["col_r"], len(rc))
+        w["col_r"], w["xr"] = rcc, w["xr"][ids.long()].contiguous()
+    w["out"] = torch.empty(ub - lb, ld, device=dev)
     w["bytes"] = w["nnz"] * (4 + dim * 4) + w["rows"] * dim * 4 + (w["rows"] + 1) * 4 * (2 if len(rc) else 1)
     return w
 
 
-def time_setting(w, ps, wpb, dist, iters):
+def time_setting(w, ps, wpb, dist, iters, core_rows=-1, col_block_rows=0, gin=False):
     import torch
 
     def call():
-        host.mgg_SAG_np_div(w["out"], w["xl"], w["ptr_l"], w["col_l"], w["ptr_r"], w["col_r"], w["lb"], w["ub"], w["dim"],
-                            w["npp"], 0, ps, wpb, dist, input_remote=w["xr"])
+        if gin:
+            host.mgg_GIN_np_div(w["out"], w["xl"], w["ptr_l"], w["col_l"], w["ptr_r"], w["col_r"], w["lb"], w["ub"], w["dim"],
+                                w["npp"], 0, ps, wpb, dist, 0.0, input_remote=w["xr"], ld_in=w["ld"], ld_out=w["ld"],
+                                col_block_rows=col_block_rows, core_rows=core_rows)
+        else:
+            host.mgg_SAG_np_div(w["out"], w["xl"], w["ptr_l"], w["col_l"], w["ptr_r"], w["col_r"], w["lb"], w["ub"], w["dim"],
+                                w["npp"], 0, ps, wpb, dist, input_remote=w["xr"], ld_in=w["ld"], ld_out=w["ld"],
+                                col_block_rows=col_block_rows, core_rows=core_rows)
 
     call()
     call()
@@ -68,6 +87,47 @@ def time_setting(w, ps, wpb, dist, iters):
     return e0.elapsed_time(e1) / iters
 
 
+def sweep_wpb_dist(w, args):
+    """wpb x dist at ps 16; order and dense core by the library's rules and cost model."""
+    time_setting(w, 16, 0, 0, 4 * args.iters, core_rows=0, gin=args.gin)  # plans built, clocks up
+    rule = time_setting(w, 16, 0, 0, args.iters, core_rows=0, gin=args.gin)
+    print("everything by rule: %.4f ms   [%s]" % (rule, host.last_agg_kernel()))
+    wpbs, dists = [2, 4, 8, 16], [1, 2, 4, 8, 16]
+    print("\nms, ps = 16            " + "".join("dist=%-6d" % x for x in dists))
+    best = (1e30, None)
+    for wpb in wpbs:
+        row = [time_setting(w, 16, wpb, d, args.iters, core_rows=0, gin=args.gin) for d in dists]
+        best = min(best, min((ms, (wpb, d)) for ms, d in zip(row, dists)))
+        print("wpb=%-3d               " % wpb + "".join("%-11.4f" % x for x in row))
+        sys.stdout.flush()
+    print("\nbest: wpb=%d dist=%d  %.4f ms; by rule / best = %.3f" % (best[1][0], best[1][1], best[0], rule / best[0]))
+
+
+def sweep_core(w, args):
+    """Aggregation time against the dense-core size (best of a few wpb x dist), with the plan's entry counts."""
+    import ctypes as C
+    time_setting(w, 16, 0, 0, 4 * args.iters, core_rows=0, gin=args.gin)  # plans built, clocks up
+    rule = time_setting(w, 16, 0, 0, args.iters, core_rows=0, gin=args.gin)
+    print("everything by rule: %.4f ms   [%s]" % (rule, host.last_agg_kernel()))
+    print("\ncore rows | ms (best) | wpb dist | edges in the core | list entries with padding | edges left to the gather kernel")
+    best = (1e30, None)
+    for K in (-1, 8192, 16384, 24576, 32768, 40960, 49152, 57344, 65536, 81920, 98304):
+        if K > w["rows"] // 2:
+            continue
+        sz = [0] * 5
+        if K > 0:
+            s5 = (C.c_int64 * 5)()
+            host._check(host.lib().mggx_core_layout_device(host._dptr(w["ptr_l"]), host._dptr(w["col_l"]), w["rows"], w["lb"], K, s5, None, None,
+                                                           None, None, None, None))
+            sz = list(s5)
+        row = min((time_setting(w, 16, wpb, d, args.iters, core_rows=K, gin=args.gin), wpb, d)
+                  for wpb, d in ((4, 2), (4, 4), (4, 8), (4, 16), (8, 2), (8, 8), (16, 2)))
+        best = min(best, (row[0], K))
+        print("%9d | %9.4f | %3d %4d | %17d | %25d | %d" % (K, row[0], row[1], row[2], sz[4], sz[2], sz[3] if K > 0 else w["nnz"]))
+        sys.stdout.flush()
+    print("\nbest: %d rows, %.4f ms; by rule / best = %.3f" % (best[1], best[0], rule / best[0]))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="share", choices=["share", "whole", "sparse"])
@@ -75,13 +135,22 @@ def main():
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--small", action="store_true")
     ap.add_argument("--out", default="")
+    ap.add_argument("--mode", default="ps", choices=["ps", "wd", "core"], help="ps: the reference's ps x wpb and dist x ps tables; "
+                    "wd: wpb x dist at ps 16 with order and dense core by rule; core: dense-core size sweep")
+    ap.add_argument("--ld", type=int, default=0, help="row pitch of the tables in floats (default: dim)")
+    ap.add_argument("--gin", action="store_true", help="aggregate with the GIN self term")
+    ap.add_argument("--compact-remote", action="store_true", help="share: stage the remote rows compactly")
     args = ap.parse_args()
     import torch
     torch.cuda.set_device(0)
     host.init(0)
     host.use_torch_stream()
-    w = build_workload(args.workload, args.dim, args.small)
+    w = build_workload(args.workload, args.dim, args.small, args.ld, args.compact_remote)
     print("workload %s: rows=%d nnz=%d dim=%d algorithmic bytes=%d" % (args.workload, w["rows"], w["nnz"], args.dim, w["bytes"]))
+    if args.mode == "wd":
+        return sweep_wpb_dist(w, args)
+    if args.mode == "core":
+        return sweep_core(w, args)
     res = {"workload": args.workload, "dim": args.dim, "rows": w["rows"], "nnz": w["nnz"], "bytes": w["bytes"], "ps_wpb": {},
            "dist_ps": {}}
     best = (1e30, None)
