@@ -196,6 +196,7 @@ MEASURED_TRAFFIC = {
     "share_agg_compact": (1_036_854_989, (4, 4)),   # remote rows staged compactly (one row per distinct remote id)
     "gin_agg": (25_550_513_561, (16, 1)),
     "gin_agg_core40960": (19_723_389_132, (8, 4)),   # dense core of 40960 rows from LDS beside the rest
+    "gin_agg_core49152": (19151892377, (8, 16)),  # the size the cost model picks
     "big_agg": (60_511_998_361, (4, 16)),
 }
 
@@ -715,6 +716,7 @@ def bench_gin(args, torch, host):
             names += ["agg%d" % l, "mlp%d" % l]
     stages.append(lambda: host.softmax_forward(d_P, d_logits, V, out_dim))
     names.append("softmax")
+    kn.observe(host, stages[1])  # what the library chose where the knobs were left to it
 
     for _ in range(args.warmup):
         for fn in stages:

@@ -738,11 +738,23 @@ __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, con
         }
         if (cm.partial) {
             const int r = cm.rank[v];
-            if (r >= 0)
-                for (int seg = 0; seg < cm.nseg; ++seg) {
-                    const float4 p = cm.partial[((size_t)seg * cm.core + r) * n4 + q];
+            if (r >= 0) {
+                const float4 *src = cm.partial + (size_t)r * n4 + q;
+                const size_t seg_stride = (size_t)cm.core * n4;
+                int seg = 0;
+                for (; seg + 4 <= cm.nseg; seg += 4) {  // four segments in flight, summed in order
+                    const float4 p0 = src[(size_t)seg * seg_stride], p1 = src[(size_t)(seg + 1) * seg_stride];
+                    const float4 p2 = src[(size_t)(seg + 2) * seg_stride], p3 = src[(size_t)(seg + 3) * seg_stride];
+                    t.x += p0.x; t.y += p0.y; t.z += p0.z; t.w += p0.w;
+                    t.x += p1.x; t.y += p1.y; t.z += p1.z; t.w += p1.w;
+                    t.x += p2.x; t.y += p2.y; t.z += p2.z; t.w += p2.w;
+                    t.x += p3.x; t.y += p3.y; t.z += p3.z; t.w += p3.w;
+                }
+                for (; seg < cm.nseg; ++seg) {
+                    const float4 p = src[(size_t)seg * seg_stride];
                     t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
                 }
+            }
         }
     }
     float val[4] = {t.x, t.y, t.z, t.w};
