@@ -264,9 +264,13 @@ typedef struct mggx_agg_knobs {
  * rest of the CSR runs as usual on top.  Pays on graphs whose high-degree rows hold most edges among themselves; its
  * plan is built on the GPU on first use (milliseconds).  The core block runs on a second stream of the library's, forked from and joined to the
  * caller's stream by events inside the call (LDS-bound work beside cache-bound work).  Same result up to summation order.
- * The partition plan of (d_ptr_l, d_ptr_r, d_col_r, rows, ps) -- and d_col_l for the column-blocked order -- is built on first use and
- * cached by pointer identity: the CSR arrays must not be rewritten in place or freed
- * while cached (mggx_forget() drops what hangs on one array, mggx_release_cached() everything). */
+ * With core_rows = 0 the library picks the size itself (possibly none) from the degree histogram: it grows the core
+ * while the predicted padding of the added rows' index lists costs less than the gathers they remove.
+ * MGGX_AGG_SOFTMAX (fp32 tables): the finished rows leave as their row softmax, on every path above.
+ * The partition plan of (d_ptr_l, d_ptr_r, d_col_r, rows, ps) -- and d_col_l for the column-blocked order -- is built on
+ * first use and cached by pointer identity.  The arrays stay the caller's: what happens when they are rewritten in
+ * place or their address is reused is described at mggx_set_plan_check (mggx_forget() drops what hangs on one array,
+ * mggx_release_cached() everything). */
 int mggx_sag_np_div(float *d_out, const void *d_in_local, const void *d_in_remote,
                     const int *d_ptr_l, const int *d_col_l, const int *d_ptr_r, const int *d_col_r,
                     int lb, int ub, int dim, int nodes_per_pe,

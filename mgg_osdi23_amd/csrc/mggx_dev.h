@@ -114,7 +114,7 @@ struct Plan {
     Guard guard;               // explicit-partition plans only (the others are guarded through their GraphInfo)
 };
 
-// Dense-core plan of a local-only CSR (layout: CoreLayout in mggx_internal.h), built on the host and kept on the device.
+// Dense-core plan of a local-only CSR (layout: CoreLayout in mggx_internal.h), built on the GPU and kept there.
 struct CorePlan {
     // cache key
     const int *d_ptr_l = nullptr;
