@@ -18,6 +18,9 @@
 //   workgroups a row that crosses workgroups leaves two partial rows in a
 //              carry buffer; a small second kernel sums them in a fixed order
 // No atomics anywhere; the summation order depends only on (ps, wpb, dist, dim).
+// Index stream: a wavefront fetches the descriptors and the first ids of its next few rounds together into its own
+// piece of LDS (two HBM latencies per four rounds instead of per round, with no feature row in flight meanwhile) and
+// the rounds read them from there; the 16 lanes or so of a slot read the same words.
 #include <chrono>
 #include <cstring>
 #include <type_traits>
@@ -64,6 +67,8 @@ struct AggArgs {
     const int *nnz_l_dev;     // when set: the local edge count is read from here (a caller that may not copy it to the host)
     int lb, dim, ps, dist, cpad;
     int parts_per_wg;
+    int stage_off;            // dynamic LDS, in floats: where the wavefronts' staged descriptors and ids start
+    int stage_rounds;         // rounds staged at a time (1 .. the kernel's STAGE)
     unsigned flags;
     float eps;
     int in_is_bf16;
@@ -94,23 +99,6 @@ __device__ __forceinline__ int lane_read(int v, int src) { return __builtin_amdg
 __device__ __forceinline__ float lane_read(float v, int src)
 {
     return __int_as_float(__builtin_amdgcn_ds_bpermute(src << 2, __float_as_int(v)));
-}
-
-// Broadcast the value held by lane SRC of each slot to the whole slot.
-template <int LPR, int SRC>
-__device__ __forceinline__ int slot_bcast(int v, int slot_base)
-{
-    if constexpr (LPR == 1) {
-        return v;
-    } else if constexpr (LPR == 2) {
-        return __builtin_amdgcn_update_dpp(v, v, SRC | (SRC << 2) | ((2 + SRC) << 4) | ((2 + SRC) << 6), 0xf, 0xf, true);
-    } else if constexpr (LPR == 4) {
-        return __builtin_amdgcn_update_dpp(v, v, SRC | (SRC << 2) | (SRC << 4) | (SRC << 6), 0xf, 0xf, true);
-    } else if constexpr (LPR == 64) {
-        return __builtin_amdgcn_readlane(v, SRC);
-    } else {
-        return lane_read(v, slot_base + SRC);
-    }
 }
 
 template <int MODE>
@@ -338,6 +326,9 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     // that nobody reads again: those loads carry the streaming hint, which leaves the caches to the feature rows
     // (-5 % at width 16).  With fewer slots adjacent wavefronts share those lines and the hint costs 1-3 %.
     constexpr bool STREAM = S >= 16;
+    // rounds whose descriptors and first ids a wavefront fetches at once (1.3 - 5 KiB of LDS per wavefront; measured on
+    // the benchmark graphs: 4 rounds are as good as 8, 1 round is 5 - 10 % slower where the feature table is cache resident)
+    constexpr int STAGE = LPR >= 4 ? 4 : LPR == 2 ? 2 : 1;
     extern __shared__ float lds[];
     if (gate_closed(a.gate)) return;
 
@@ -383,13 +374,10 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     int has_first = 0;    // the open run includes its row's first partition
     bool c_open = false;  // wavefront-uniform: slot S-1 holds a row that continues in the next round
 
-    for (int j = 0; j < a.dist; ++j) {
-        const long long q0 = q_wave + (long long)j * S;
-        if (q0 >= a.num_parts) break;
-        const long long q = q0 + slot;
-        const bool pv = q < a.num_parts;
+    // A slot's descriptor, or an empty one (no row, no neighbors) past the end of the plan or of this wavefront's rounds.
+    auto load_desc = [&](long long q, bool in_range) -> int4 {
         int4 d = make_int4(0, -1, 0, 0);
-        if (pv) {
+        if (in_range && q < a.num_parts) {
             if constexpr (STREAM) {
                 typedef int v4i_a __attribute__((ext_vector_type(4)));
                 const v4i_a dv = __builtin_nontemporal_load(reinterpret_cast<const v4i_a *>(a.desc + q));
@@ -398,6 +386,116 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
                 d = a.desc[q];
             }
         }
+        return d;
+    };
+    // This lane's IPL neighbor ids of the chunk starting at neighbor k0 of the partition d describes, as row indices of
+    // that partition's table (pad_id past the end of the partition).
+    auto fetch_ids = [&](const int4 &d, int k0, int (&ids)[IPL]) {
+        const int len = (int)((unsigned)d.z & DESC_LEN_MASK);
+        const bool remote = d.x < 0;
+        const long long start = (long long)((unsigned)d.x & 0x7FFFFFFFu);
+        const int *col = remote ? a.col_r : a.col_l;
+        const int idbase = remote ? 0 : a.lb;
+        const int kk = k0 + l * IPL;
+        const long long e0 = start + kk;
+#pragma unroll
+        for (int t = 0; t < IPL; ++t) ids[t] = pad_id;
+        if (kk < len) {
+            if constexpr (IPL == 4) {
+                const int nnz_side = remote ? a.nnz_r : (a.nnz_l_dev ? *a.nnz_l_dev : a.nnz_l);
+                if (e0 + 4 <= nnz_side) {
+                    typedef int v4i_u __attribute__((ext_vector_type(4), aligned(4)));
+                    const v4i_u tv = __builtin_nontemporal_load(reinterpret_cast<const v4i_u *>(col + e0));
+                    ids[0] = tv.x; ids[1] = tv.y; ids[2] = tv.z; ids[3] = tv.w;
+                } else {
+#pragma unroll
+                    for (int t = 0; t < IPL; ++t)
+                        if (kk + t < len) ids[t] = col[e0 + t];
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < IPL; ++t)
+                    if (kk + t < len) ids[t] = col[e0 + t];
+            }
+#pragma unroll
+            for (int t = 0; t < IPL; ++t) ids[t] = (kk + t < len) ? ids[t] - idbase : pad_id;
+        }
+    };
+    // One window of gathers of a chunk of CH neighbors: get_rid(k) is the k-th neighbor's row in the slot's table.
+    auto gather_chunk = [&](int len, int k0, auto get_rid) {
+        static_for<0, CH / BATCH>([&](auto bb) {
+            constexpr int b = decltype(bb)::value;
+            if (__any(len > k0 + b * BATCH)) {
+                int rid[BATCH];
+                static_for<0, BATCH>([&](auto tt) {
+                    constexpr int t = decltype(tt)::value;
+                    rid[t] = get_rid(std::integral_constant<int, b * BATCH + t>{});
+                });
+                // lanes past the row width neither load nor sum (their sums stay zero and are never stored): a quad
+                // of idle lanes costs the address unit nothing, and no register of the batch needs clearing
+                if (lane_on) {
+                    v4u raw[BATCH];
+                    static_for<0, BATCH>([&](auto tt) {
+                        constexpr int t = decltype(tt)::value;
+                        raw[t] = g.load(rid[t]);
+                    });
+                    // keep every load of the batch in flight before the first sum waits on one
+                    __builtin_amdgcn_sched_barrier(0);
+                    static_for<0, BATCH>([&](auto tt) {
+                        constexpr int t = decltype(tt)::value;
+                        float v[NV];
+                        unpack16<MODE>(v, raw[t]);
+#pragma unroll
+                        for (int i = 0; i < NV; ++i) acc[i] += v[i];
+                    });
+                }
+            }
+        });
+    };
+
+    // The index stream comes from HBM, the feature rows (where the kernel is at its fastest) from the caches.  A
+    // wavefront that fetched descriptor, then ids, then rows in every round would wait out two HBM latencies per
+    // round with no row in flight.  Instead it fetches the descriptors and the first CH ids of each partition for
+    // STAGE rounds at a time -- all descriptor loads in flight together, then all id loads -- into its own piece of
+    // LDS, and the rounds read them from there (every lane of a slot reads the same words).
+    const int nst = a.stage_rounds < STAGE ? a.stage_rounds : STAGE;
+    int4 *st_desc = reinterpret_cast<int4 *>(lds + a.stage_off) + (size_t)wave * (nst * S);
+    int *st_ids = reinterpret_cast<int *>(lds + a.stage_off) + (size_t)wpb * (nst * S * 4) + (size_t)wave * (nst * S * CH);
+
+    for (int j0 = 0; j0 < a.dist; j0 += nst) {
+        if (q_wave + (long long)j0 * S >= a.num_parts) break;
+        {
+            int4 dd[STAGE];
+            int idv[STAGE][IPL];
+#pragma unroll
+            for (int u = 0; u < STAGE; ++u) dd[u] = load_desc(q_wave + (long long)(j0 + u) * S + slot, u < nst && j0 + u < a.dist);
+#pragma unroll
+            for (int u = 0; u < STAGE; ++u) {
+                fetch_ids(dd[u], 0, idv[u]);
+                if (u < nst && l == 0) st_desc[u * S + slot] = dd[u];
+            }
+#pragma unroll
+            for (int u = 0; u < STAGE; ++u) {
+                if (u < nst) {
+                    int *dst = st_ids + (u * S + slot) * CH + l * IPL;
+#pragma unroll
+                    for (int t = 0; t < IPL; ++t) dst[t] = idv[u][t];
+                }
+            }
+        }
+        // the lanes of this wavefront read what other lanes of it wrote
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    for (int u = 0; u < nst; ++u) {
+        const int j = j0 + u;
+        if (j >= a.dist) break;
+        const long long q0 = q_wave + (long long)j * S;
+        if (q0 >= a.num_parts) break;
+        const long long q = q0 + slot;
+        const bool pv = q < a.num_parts;
+        const int4 d = st_desc[u * S + slot];
 
         // carried partial row of the previous round: slot S-1 -> slot 0
         float cv[NV];
@@ -414,71 +512,26 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
         const int row = d.y;
         const int len = (int)((unsigned)d.z & DESC_LEN_MASK);
         const bool remote = d.x < 0;
-        const long long start = (long long)((unsigned)d.x & 0x7FFFFFFFu);
-        const int *col = remote ? a.col_r : a.col_l;
-        const int idbase = remote ? 0 : a.lb;
-        const int nnz_side = remote ? a.nnz_r : (a.nnz_l_dev ? *a.nnz_l_dev : a.nnz_l);
         if constexpr (BUF) g.cbase = (remote ? a.delta_r : a.delta_l) + cofs;
         else g.base = static_cast<const char *>(remote ? a.in_r : a.in_l) + cofs;
 
+        // neighbors [0, CH) of the partition were staged; a longer partition (ps > CH) fetches each further chunk of ids
+        // into the same words when it gets there
+        int *pid = st_ids + (u * S + slot) * CH;
         for (int k0 = 0; k0 < a.ps; k0 += CH) {
             if (!__any(len > k0)) break;
-            // this lane's IPL neighbor rows of the chunk, as row indices of the slot's table (pad_id past the end)
-            int ids[IPL];
-            {
-                const int kk = k0 + l * IPL;
-                const long long e0 = start + kk;
+            if (k0 > 0) {
+                int ids[IPL];
+                fetch_ids(d, k0, ids);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
 #pragma unroll
-                for (int t = 0; t < IPL; ++t) ids[t] = pad_id;
-                if (kk < len) {
-                    if constexpr (IPL == 4) {
-                        if (e0 + 4 <= nnz_side) {
-                            typedef int v4i_u __attribute__((ext_vector_type(4), aligned(4)));
-                            const v4i_u tv = __builtin_nontemporal_load(reinterpret_cast<const v4i_u *>(col + e0));
-                            ids[0] = tv.x; ids[1] = tv.y; ids[2] = tv.z; ids[3] = tv.w;
-                        } else {
-#pragma unroll
-                            for (int t = 0; t < IPL; ++t)
-                                if (kk + t < len) ids[t] = col[e0 + t];
-                        }
-                    } else {
-#pragma unroll
-                        for (int t = 0; t < IPL; ++t)
-                            if (kk + t < len) ids[t] = col[e0 + t];
-                    }
-#pragma unroll
-                    for (int t = 0; t < IPL; ++t) ids[t] = (kk + t < len) ? ids[t] - idbase : pad_id;
-                }
+                for (int t = 0; t < IPL; ++t) pid[l * IPL + t] = ids[t];
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             }
-            static_for<0, CH / BATCH>([&](auto bb) {
-                constexpr int b = decltype(bb)::value;
-                if (__any(len > k0 + b * BATCH)) {
-                    v4u raw[BATCH];
-                    int rid[BATCH];
-                    static_for<0, BATCH>([&](auto tt) {
-                        constexpr int t = decltype(tt)::value;
-                        constexpr int k = b * BATCH + t;
-                        rid[t] = slot_bcast<LPR, k / IPL>(ids[k % IPL], slot_base);
-                        raw[t] = (v4u){0u, 0u, 0u, 0u};
-                    });
-                    // lanes past the row width issue no load at all: a quad of idle lanes costs the address unit nothing
-                    if (lane_on) {
-                        static_for<0, BATCH>([&](auto tt) {
-                            constexpr int t = decltype(tt)::value;
-                            raw[t] = g.load(rid[t]);
-                        });
-                    }
-                    // keep every load of the batch in flight before the first sum waits on one
-                    __builtin_amdgcn_sched_barrier(0);
-                    static_for<0, BATCH>([&](auto tt) {
-                        constexpr int t = decltype(tt)::value;
-                        float v[NV];
-                        unpack16<MODE>(v, raw[t]);
-#pragma unroll
-                        for (int i = 0; i < NV; ++i) acc[i] += v[i];
-                    });
-                }
-            });
+            gather_chunk(len, k0, [&](auto kc) { return pid[decltype(kc)::value]; });
         }
 
         // ---- combine the slots of this round ----
@@ -537,6 +590,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
             }
         }
         c_open = __any(keep_open);
+    }
     }
 
     __syncthreads();
@@ -790,6 +844,8 @@ int launch_agg(int lpr, dim3 grid, dim3 block, size_t lds_bytes, hipStream_t str
     switch (lpr) {
 #define MGGX_CASE(L)                                                      \
     case L:                                                               \
+        if (lds_bytes > (48u << 10))                                      \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&k_agg<L, MODE, BUF, SMX>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes); \
         k_agg<L, MODE, BUF, SMX><<<grid, block, lds_bytes, stream>>>(a);  \
         break;
         MGGX_CASE(1)
@@ -957,7 +1013,21 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         if (blocked) {
             a.out = reinterpret_cast<float *>(static_cast<char *>(ws) + carry_bytes);
         }
-        const size_t lds_bytes = (size_t)wpb * 2 * sizeof(int2) + (size_t)wpb * 2 * cpad * sizeof(float);
+        // dynamic LDS: head/tail entries of the wavefronts, then their staged descriptors and ids (see k_agg); fewer
+        // rounds are staged at a time when many wavefronts per workgroup would take more than 40 KiB
+        const int stage_max = lpr >= 4 ? 4 : lpr == 2 ? 2 : 1;
+        const int ch = lpr > 16 ? lpr : 16;
+        const size_t round_bytes = (size_t)slots * ((size_t)ch * 4 + 16);
+        int stage = stage_max < dist ? stage_max : dist;
+        while (stage > 1 && (size_t)wpb * stage * round_bytes > (40u << 10)) stage /= 2;
+        // beside a dense core whose table does not fit the caches the gathers wait for HBM anyway, and the LDS is worth
+        // more to the core's workgroups
+        if (cm && (unsigned long long)plan->real_rows * ld_bytes > (256ull << 20)) stage = 1;
+        const size_t carry_lds = ((size_t)wpb * 2 * sizeof(int2) + (size_t)wpb * 2 * cpad * sizeof(float) + 15) & ~(size_t)15;
+        a.stage_off = (int)(carry_lds / sizeof(float));
+        a.stage_rounds = stage;
+        const size_t lds_bytes = carry_lds + (size_t)wpb * stage * round_bytes;
+        if (lds_bytes > (160u << 10)) return fail(MGGX_ELIMIT, "aggregation: %zu bytes of LDS per workgroup (wpb %d, dim %d)", lds_bytes, wpb, dim);
         const dim3 grid((unsigned)num_wg), block((unsigned)(64 * wpb));
         const bool smx = (a.flags & MGGX_AGG_SOFTMAX) != 0;  // fp32 tables only (checked above)
         if (buf) {
