@@ -794,7 +794,7 @@ __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, con
             const int r = cm.rank[v];
             if (r >= 0) {
                 const float4 *src = cm.partial + (size_t)r * n4 + q;
-                const size_t seg_stride = (size_t)cm.core * n4;
+                const size_t seg_stride = part_stride(cm.core) * n4;
                 int seg = 0;
                 for (; seg + 4 <= cm.nseg; seg += 4) {  // four segments in flight, summed in order
                     const float4 p0 = src[(size_t)seg * seg_stride], p1 = src[(size_t)(seg + 1) * seg_stride];

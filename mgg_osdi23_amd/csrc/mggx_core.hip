@@ -26,7 +26,7 @@ constexpr int CORE_TC = 256;    // core columns per LDS tile
 constexpr int CORE_WAVES = 4;   // slices (of 64 rows) per workgroup: as small as the aggregation's own workgroups, so the two
                                 // kernels of a call, running side by side, find room on a CU equally easily
 
-// tab[s * core + i] = elements 4 s .. 4 s + 3 of the feature row of the rank-i node (zero past dim)
+// tab[s * tab_stride(core) + i] = elements 4 s .. 4 s + 3 of the feature row of the rank-i node (zero past dim)
 __global__ void __launch_bounds__(256) k_core_stage(v4f *__restrict__ tab, const float *__restrict__ in, const int *__restrict__ order,
                                                     int core, int n4, int dim, long long ld_in, const Gate gate)
 {
@@ -40,27 +40,33 @@ __global__ void __launch_bounds__(256) k_core_stage(v4f *__restrict__ tab, const
     v.y = 4 * s + 1 < dim ? row[1] : 0.f;
     v.z = 4 * s + 2 < dim ? row[2] : 0.f;
     v.w = 4 * s + 3 < dim ? row[3] : 0.f;
-    tab[idx] = v;
+    tab[(size_t)s * tab_stride(core) + i] = v;
 }
 
 // One workgroup = CORE_WAVES slices x one segment of `tiles_per_seg` column tiles; lane = core row.
-// partial[(seg * core + rank) * N4 + s]
+// partial[(seg * part_stride(core) + rank) * N4 + s]
 template <int N4>
 __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *__restrict__ blk_off, const unsigned short *__restrict__ idx,
                                                                const v4f *__restrict__ tab, v4f *__restrict__ partial, int core, int ntiles,
-                                                               int tiles_per_seg, const Gate gate)
+                                                               int nseg, const Gate gate)
 {
     constexpr int TC = CORE_TC, TP = TC + 1;  // column TC of every slice row is zero: what padding entries read
     extern __shared__ v4f tile[];             // [N4][TP]
     if (gate_closed(gate)) return;
     const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
-    const int g = (int)blockIdx.x * CORE_WAVES + wave;
+    // Consecutive workgroups go to the 8 XCDs in turn and the row groups are sorted by degree: with a number of row groups
+    // that is a multiple of 8, XCD 0 would get the heaviest group of every eight in every segment.  Rotating the row
+    // groups by the segment number spreads them (measured at 32,768 rows: 6 % of the whole aggregation).
     const int seg = (int)blockIdx.y;
+    const int g = (int)(((unsigned)blockIdx.x + (unsigned)seg) % gridDim.x) * CORE_WAVES + wave;
     v4f acc[N4];
 #pragma unroll
     for (int s = 0; s < N4; ++s) acc[s] = (v4f){0.f, 0.f, 0.f, 0.f};
     if ((int)threadIdx.x < N4) tile[(int)threadIdx.x * TP + TC] = (v4f){0.f, 0.f, 0.f, 0.f};
-    const int t0 = seg * tiles_per_seg;
+    // segment `seg` takes the tiles [seg * ntiles / nseg, (seg + 1) * ntiles / nseg): any number of tiles splits into
+    // segments whose lengths differ by at most one
+    const int t0 = (int)((long long)seg * ntiles / nseg);
+    const int tiles_per_seg = (int)((long long)(seg + 1) * ntiles / nseg) - t0;
     const us4 *p = reinterpret_cast<const us4 *>(idx) + lane;
     unsigned pos = blk_off[(size_t)g * ntiles + t0];
     const unsigned end_seg = blk_off[(size_t)g * ntiles + t0 + tiles_per_seg];
@@ -71,7 +77,7 @@ __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *_
         __syncthreads();
         for (int i = (int)threadIdx.x; i < N4 * TC; i += CORE_WAVES * 64) {
             const int s = i / TC, c = i % TC;
-            tile[s * TP + c] = tab[(size_t)s * core + (size_t)t * TC + c];
+            tile[s * TP + c] = tab[(size_t)s * tab_stride(core) + (size_t)t * TC + c];
         }
         const unsigned b1 = blk_off[(size_t)g * ntiles + t + 1];
         __syncthreads();
@@ -99,7 +105,7 @@ __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *_
     }
     const int r = g * 64 + lane;
 #pragma unroll
-    for (int s = 0; s < N4; ++s) partial[((size_t)seg * core + r) * N4 + s] = acc[s];
+    for (int s = 0; s < N4; ++s) partial[((size_t)seg * part_stride(core) + r) * N4 + s] = acc[s];
 }
 
 // Adds the core block's sums to output rows that already hold the rest of the aggregation:
@@ -125,7 +131,7 @@ __global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, co
     if (lane_on) {
         v4f sum = {0.f, 0.f, 0.f, 0.f};
         if (r >= 0) {
-            for (int seg = 0; seg < nseg; ++seg) sum += partial[((size_t)seg * core + r) * n4 + q];
+            for (int seg = 0; seg < nseg; ++seg) sum += partial[((size_t)seg * part_stride(core) + r) * n4 + q];
             if (rs) sum *= rs[v];
         }
 #pragma unroll
@@ -317,7 +323,7 @@ int launch_sell(const CorePlan *p, const v4f *tab, v4f *partial, const Gate &gat
     // row groups vary fastest in the grid: workgroups that run side by side then read the same tiles, and a CU holds dense
     // and sparse row groups at once (the reverse order measured 25 % slower)
     const dim3 grid((unsigned)(p->core / (CORE_WAVES * 64)), (unsigned)p->nseg);
-    k_core_sell<N4><<<grid, dim3(CORE_WAVES * 64), lds, stream>>>(p->d_blk_off, p->d_idx, tab, partial, p->core, p->ntiles, p->ntiles / p->nseg, gate);
+    k_core_sell<N4><<<grid, dim3(CORE_WAVES * 64), lds, stream>>>(p->d_blk_off, p->d_idx, tab, partial, p->core, p->ntiles, p->nseg, gate);
     MGGX_LAUNCH_CHECK("k_core_sell");
     return MGGX_OK;
 }
@@ -454,9 +460,11 @@ static int core_plan_build_device(CorePlan *p, int tc)
     p->ntiles = ntiles;
     p->rem_nnz = rem_nnz;
     p->core_nnz = (int64_t)nnz - rem_nnz;
-    // segments: enough workgroups to fill the chip a few times over, whole tiles each
-    int nseg = 1;
-    while (nseg * 2 <= ntiles && (ntiles % (nseg * 2)) == 0 && (long long)(core / (CORE_WAVES * 64)) * nseg < 2048) nseg *= 2;
+    // segments: enough workgroups (about 2048) to fill the chip a few times over, whole tiles each
+    const int groups = core / (CORE_WAVES * 64);
+    int nseg = (2048 + groups / 2) / groups;
+    if (nseg > ntiles) nseg = ntiles;
+    if (nseg < 1) nseg = 1;
     p->nseg = nseg;
     p->bytes = ((size_t)core + 2 * (size_t)rows + 1 + (size_t)rem_nnz + (size_t)nblk + 1) * sizeof(int) + idx_elems * sizeof(unsigned short);
     return MGGX_OK;
@@ -512,8 +520,8 @@ int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int 
 static int core_scratch(const CorePlan *p, int n4, v4f **tab, v4f **partial)
 {
     State &s = state();
-    const size_t tab_bytes = ((size_t)p->core * n4 * sizeof(v4f) + 255) & ~(size_t)255;
-    const size_t part_bytes = (size_t)p->nseg * p->core * n4 * sizeof(v4f);
+    const size_t tab_bytes = (tab_stride(p->core) * n4 * sizeof(v4f) + 255) & ~(size_t)255;
+    const size_t part_bytes = (size_t)p->nseg * part_stride(p->core) * n4 * sizeof(v4f);
     if (tab_bytes + part_bytes > s.core_ws_bytes) {
         if (capturing()) return fail(MGGX_EINVAL, "core: the scratch block would have to grow inside a stream capture; run the largest call once outside it first");
         MGGX_HIP(hipDeviceSynchronize());  // both streams may still use the old block
