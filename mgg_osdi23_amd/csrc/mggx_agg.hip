@@ -388,38 +388,40 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
         }
         return d;
     };
-    // This lane's IPL neighbor ids of the chunk starting at neighbor k0 of the partition d describes, as row indices of
-    // that partition's table (pad_id past the end of the partition).
-    auto fetch_ids = [&](const int4 &d, int k0, int (&ids)[IPL]) {
+    // This lane's IPL neighbor ids of the chunk starting at neighbor k0 of the partition d describes, in two steps so that
+    // the loads of several partitions can be in flight together: issue_ids only loads (no branch around a load: a lane
+    // with nothing to fetch reads a word of the descriptor array instead, so no wait lands between two loads), and
+    // finish_ids turns what arrived into row indices of the partition's table (pad_id past the end of the partition).
+    const int *const dummy = reinterpret_cast<const int *>(a.desc);
+    auto issue_ids = [&](const int4 &d, int k0, int (&raw)[IPL]) {
         const int len = (int)((unsigned)d.z & DESC_LEN_MASK);
         const bool remote = d.x < 0;
         const long long start = (long long)((unsigned)d.x & 0x7FFFFFFFu);
         const int *col = remote ? a.col_r : a.col_l;
-        const int idbase = remote ? 0 : a.lb;
         const int kk = k0 + l * IPL;
         const long long e0 = start + kk;
-#pragma unroll
-        for (int t = 0; t < IPL; ++t) ids[t] = pad_id;
-        if (kk < len) {
-            if constexpr (IPL == 4) {
-                const int nnz_side = remote ? a.nnz_r : (a.nnz_l_dev ? *a.nnz_l_dev : a.nnz_l);
-                if (e0 + 4 <= nnz_side) {
-                    typedef int v4i_u __attribute__((ext_vector_type(4), aligned(4)));
-                    const v4i_u tv = __builtin_nontemporal_load(reinterpret_cast<const v4i_u *>(col + e0));
-                    ids[0] = tv.x; ids[1] = tv.y; ids[2] = tv.z; ids[3] = tv.w;
-                } else {
-#pragma unroll
-                    for (int t = 0; t < IPL; ++t)
-                        if (kk + t < len) ids[t] = col[e0 + t];
-                }
-            } else {
+        if constexpr (IPL == 4) {
+            const int nnz_side = remote ? a.nnz_r : (a.nnz_l_dev ? *a.nnz_l_dev : a.nnz_l);
+            const bool whole = kk < len && e0 + 4 <= nnz_side;  // the 16 bytes lie inside the array
+            typedef int v4i_u __attribute__((ext_vector_type(4), aligned(4)));
+            const v4i_u tv = __builtin_nontemporal_load(reinterpret_cast<const v4i_u *>(whole ? col + e0 : dummy));
+            raw[0] = tv.x; raw[1] = tv.y; raw[2] = tv.z; raw[3] = tv.w;
+            if (__any(kk < len && !whole)) {  // the last few ids of the array: one by one
 #pragma unroll
                 for (int t = 0; t < IPL; ++t)
-                    if (kk + t < len) ids[t] = col[e0 + t];
+                    if (kk < len && !whole && kk + t < len) raw[t] = col[e0 + t];
             }
+        } else {
 #pragma unroll
-            for (int t = 0; t < IPL; ++t) ids[t] = (kk + t < len) ? ids[t] - idbase : pad_id;
+            for (int t = 0; t < IPL; ++t) raw[t] = *(kk + t < len ? col + e0 + t : dummy);
         }
+    };
+    auto finish_ids = [&](const int4 &d, int k0, const int (&raw)[IPL], int (&ids)[IPL]) {
+        const int len = (int)((unsigned)d.z & DESC_LEN_MASK);
+        const int idbase = d.x < 0 ? 0 : a.lb;
+        const int kk = k0 + l * IPL;
+#pragma unroll
+        for (int t = 0; t < IPL; ++t) ids[t] = (kk + t < len) ? raw[t] - idbase : pad_id;
     };
     // One window of gathers of a chunk of CH neighbors: get_rid(k) is the k-th neighbor's row in the slot's table.
     auto gather_chunk = [&](int len, int k0, auto get_rid) {
@@ -471,15 +473,17 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
             for (int u = 0; u < STAGE; ++u) dd[u] = load_desc(q_wave + (long long)(j0 + u) * S + slot, u < nst && j0 + u < a.dist);
 #pragma unroll
             for (int u = 0; u < STAGE; ++u) {
-                fetch_ids(dd[u], 0, idv[u]);
+                issue_ids(dd[u], 0, idv[u]);
                 if (u < nst && l == 0) st_desc[u * S + slot] = dd[u];
             }
 #pragma unroll
             for (int u = 0; u < STAGE; ++u) {
+                int ids[IPL];
+                finish_ids(dd[u], 0, idv[u], ids);
                 if (u < nst) {
                     int *dst = st_ids + (u * S + slot) * CH + l * IPL;
 #pragma unroll
-                    for (int t = 0; t < IPL; ++t) dst[t] = idv[u][t];
+                    for (int t = 0; t < IPL; ++t) dst[t] = ids[t];
                 }
             }
         }
@@ -521,8 +525,9 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
         for (int k0 = 0; k0 < a.ps; k0 += CH) {
             if (!__any(len > k0)) break;
             if (k0 > 0) {
-                int ids[IPL];
-                fetch_ids(d, k0, ids);
+                int raw_ids[IPL], ids[IPL];
+                issue_ids(d, k0, raw_ids);
+                finish_ids(d, k0, raw_ids, ids);
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
 #pragma unroll
