@@ -188,15 +188,15 @@ MEASURED_TRAFFIC = {
     "gcn2_agg1": (6_481_731_891, (4, 16)),
     "gcn2_agg2_blocked": (7_519_810_150, (4, 16)),   # column blocks of 49152 ids: partial rows and their reduction included
     "gcn2_agg1_blocked": (1_746_502_963, (4, 16)),
-    "gcn2_agg2_core32768_blocked": (6_064_945_472, (4, 16)),   # dense core of 32768 rows beside the column-blocked rest, one finish kernel (softmax inside)
-    "gcn2_agg1_core32768_blocked": (1_470_001_792, (4, 8)),
+    "gcn2_agg2_core32768_blocked": (6_044_086_048, (4, 16)),   # dense core of 32768 rows beside the column-blocked rest, one finish kernel (softmax inside)
+    "gcn2_agg1_core32768_blocked": (1_469_388_000, (4, 8)),
     "gcn2_agg2_core40960_blocked": (5_319_550_054, (4, 8)),   # dense core of 40960 rows from LDS beside the column-blocked rest
     "gcn2_agg1_core40960_blocked": (1_498_319_462, (4, 8)),
-    "share_agg": (1_214_389_792, (4, 4)),
-    "share_agg_compact": (1_029_645_312, (4, 4)),   # remote rows staged compactly (one row per distinct remote id)
+    "share_agg": (1_213_309_056, (4, 4)),
+    "share_agg_compact": (1_028_547_520, (4, 4)),   # remote rows staged compactly (one row per distinct remote id)
     "gin_agg": (25_550_513_561, (16, 1)),
     "gin_agg_core40960": (19_723_389_132, (8, 4)),   # dense core of 40960 rows from LDS beside the rest
-    "gin_agg_core49152": (19_067_241_808, (8, 16)),  # the size the cost model picks
+    "gin_agg_core49152": (19_057_438_976, (8, 16)),  # the size the cost model picks
     "big_agg": (60_511_998_361, (4, 16)),
 }
 
