@@ -292,6 +292,32 @@ def test_dense_core_from_lds(gpu, rmat_graph, dim, core_rows, flags):
     assert np.array_equal(out.cpu().numpy()[:, :dim], np.repeat(np.diff(ptr).astype(np.float32)[:, None], dim, 1))
 
 
+@pytest.mark.parametrize("dim,core_rows", [(16, 12800), (44, 13824)])
+def test_dense_core_with_tile_segments_of_unequal_length(gpu, dim, core_rows):
+    """A core whose number of 256-column tiles (50, 54) is not a multiple of the number of tile segments its workgroups
+    split into (41, 38): segments of one and of two tiles side by side, every tile summed exactly once."""
+    import torch
+    from mgg_osdi23_amd import host
+    V = 30000
+    ptr, col = host.gen_rmat(15, V, 1_400_000, seed=23)
+    x = gpu.fill_normal((V, dim), seed=301)
+    sh = share_of(ptr, col, V, 1, 0)
+    d_ptr, d_col, d_x = to_dev(ptr), to_dev(col), to_dev(x)
+    z, zc = torch.zeros(V + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    want, mag = oracle_agg(sh, x, x, dim)
+    for blk in (-1, 0):
+        out = torch.full((V, dim), 7.5, device="cuda")
+        gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, z, zc, 0, V, dim, V, 0, 0, 0, 0, col_block_rows=blk, core_rows=core_rows)
+        gpu.sync()
+        assert "core=%d" % core_rows in gpu.last_agg_kernel()
+        assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "core of %d rows, blk=%d" % (core_rows, blk))
+    ones = torch.ones(V, dim, device="cuda")
+    out = torch.zeros(V, dim, device="cuda")
+    gpu.mgg_SAG_np_div(out, ones, d_ptr, d_col, z, zc, 0, V, dim, V, 0, 0, 0, 0, core_rows=core_rows)
+    gpu.sync()
+    assert np.array_equal(out.cpu().numpy(), np.repeat(np.diff(ptr).astype(np.float32)[:, None], dim, 1))
+
+
 def test_dense_core_on_a_share_with_unsorted_rows_and_parallel_edges(gpu, rmat_graph):
     """The local half of a share whose rows start at lb > 0, neighbor lists shuffled and some edges listed twice: the
     core's index lists carry order and multiplicity as they come, so the sums still match the oracle."""
