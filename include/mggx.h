@@ -107,7 +107,7 @@ typedef struct mggx_cache_stats_t {
     int64_t plans, plan_bytes;             /* cached partition plans (descriptors, row offsets) and their device bytes */
     int64_t core_plans, core_plan_bytes;   /* dense-core plans (ranking, index lists, remaining CSR) */
     int64_t workspace_bytes;               /* carry buffer and per-block partial rows */
-    int64_t core_scratch_bytes;            /* staged core table and per-segment partial rows */
+    int64_t core_scratch_bytes;            /* staged core table and the partial rows of the core kernel's workgroups */
     int64_t retired_bytes;                 /* outgrown blocks kept because a captured graph may point at them */
     double plan_build_ms, core_plan_build_ms, search_ms;  /* search_ms excludes the plan builds inside the search */
 } mggx_cache_stats_t;

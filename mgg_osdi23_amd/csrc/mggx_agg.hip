@@ -746,9 +746,9 @@ __global__ void __launch_bounds__(256) k_agg_tail(const AggArgs a, int num_wg, i
 // plan's row offsets, so no fix-up pass, no zero fill and no separate reduction run.  G lanes per row (a power of two
 // >= dim/4), lane q holds columns 4 q .. 4 q + 3; the epilogue is the caller's (row scale, accumulate, ReLU, softmax).
 struct CoreMergeArgs {
-    const float4 *partial;  // [nseg][core][n4] or NULL
+    const float4 *partial;  // [slot][CORE_GROUP_ROWS][n4] or NULL
     const int *rank;        // [rows]: rank in the core or -1
-    int core, nseg;
+    const int *wg_base;     // [core / CORE_GROUP_ROWS + 1]: the slots of row group g are wg_base[g] .. wg_base[g + 1] - 1
 };
 
 __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp, int G,
@@ -798,19 +798,21 @@ __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, con
         if (cm.partial) {
             const int r = cm.rank[v];
             if (r >= 0) {
-                const float4 *src = cm.partial + (size_t)r * n4 + q;
-                const size_t seg_stride = part_stride(cm.core) * n4;
-                int seg = 0;
-                for (; seg + 4 <= cm.nseg; seg += 4) {  // four segments in flight, summed in order
-                    const float4 p0 = src[(size_t)seg * seg_stride], p1 = src[(size_t)(seg + 1) * seg_stride];
-                    const float4 p2 = src[(size_t)(seg + 2) * seg_stride], p3 = src[(size_t)(seg + 3) * seg_stride];
+                const int grp = r / CORE_GROUP_ROWS;
+                int slot = cm.wg_base[grp];
+                const int slot_end = cm.wg_base[grp + 1];
+                const size_t stride = (size_t)CORE_GROUP_ROWS * n4;
+                const float4 *src = cm.partial + (size_t)(r % CORE_GROUP_ROWS) * n4 + q;
+                for (; slot + 4 <= slot_end; slot += 4) {  // four partial rows in flight, summed in order
+                    const float4 p0 = src[(size_t)slot * stride], p1 = src[(size_t)(slot + 1) * stride];
+                    const float4 p2 = src[(size_t)(slot + 2) * stride], p3 = src[(size_t)(slot + 3) * stride];
                     t.x += p0.x; t.y += p0.y; t.z += p0.z; t.w += p0.w;
                     t.x += p1.x; t.y += p1.y; t.z += p1.z; t.w += p1.w;
                     t.x += p2.x; t.y += p2.y; t.z += p2.z; t.w += p2.w;
                     t.x += p3.x; t.y += p3.y; t.z += p3.z; t.w += p3.w;
                 }
-                for (; seg < cm.nseg; ++seg) {
-                    const float4 p = src[(size_t)seg * seg_stride];
+                for (; slot < slot_end; ++slot) {
+                    const float4 p = src[(size_t)slot * stride];
                     t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
                 }
             }
@@ -882,7 +884,7 @@ struct FixedScratch {
 struct CoreMerge {
     const float4 *partial;
     const int *rank;
-    int core, nseg;
+    const int *wg_base;
     hipEvent_t join;
     bool merged;
 };
@@ -1060,10 +1062,10 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         r.ld_out = ld_out;
         r.rs_out = o.d_row_scale_out;
         r.flags = o.flags;
-        CoreMergeArgs cma{nullptr, nullptr, 0, 0};
+        CoreMergeArgs cma{nullptr, nullptr, nullptr};
         if (cm) {
             MGGX_HIP(hipStreamWaitEvent(st.stream, cm->join, 0));
-            cma = CoreMergeArgs{cm->partial, cm->rank, cm->core, cm->nseg};
+            cma = CoreMergeArgs{cm->partial, cm->rank, cm->wg_base};
             cm->merged = true;
         }
         const int G = pow2_ceil((dim + 3) / 4);
@@ -1179,7 +1181,7 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
             const hipError_t er = hipEventRecord(join, side);
             int rc2 = MGGX_OK;
             GraphInfo *gr = nullptr;
-            CoreMerge cm{nullptr, cp->d_rank, cp->core, cp->nseg, join, false};
+            CoreMerge cm{nullptr, cp->d_rank, cp->d_wg_base, join, false};
             if (!rc) rc2 = core_partial_rows(cp, dim, &cm.partial);
             if (!rc && !rc2) rc2 = graph_info(cp->d_rem_ptr, nullptr, cp->d_rem_col, nullptr, ub - lb, true, &gr);
             if (!rc && !rc2 && er == hipSuccess) {

@@ -4,9 +4,9 @@
 // block does not need one gather per edge from the caches: the feature rows of 256 core columns at a time are staged
 // in LDS with whole-line reads, and every lane owns one core row and adds the LDS rows its index list names
 // (sliced-ELL lists over degree-ranked rows, so the 64 lanes of a wavefront have lists of similar length).  The
-// block's sums go to partial rows per column segment.  This kernel is bound by the LDS, the ordinary aggregation of
-// the rest of the CSR by the caches, so the caller runs the two side by side on two streams; k_core_finish then adds
-// the partial rows to the output the aggregation wrote.
+// block's sums go to partial rows, one per row and run of column tiles a workgroup takes.  This kernel is bound by the
+// LDS, the ordinary aggregation of the rest of the CSR by the caches, so the caller runs the two side by side on two
+// streams; k_core_finish then adds the partial rows to the output the aggregation wrote.
 #include <algorithm>
 #include <chrono>
 #include <cmath>
@@ -23,8 +23,10 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned short us4 __attribute__((ext_vector_type(4)));
 
 constexpr int CORE_TC = 256;    // core columns per LDS tile
-constexpr int CORE_WAVES = 4;   // slices (of 64 rows) per workgroup: as small as the aggregation's own workgroups, so the two
-                                // kernels of a call, running side by side, find room on a CU equally easily
+constexpr int CORE_TARGET_WGS = 2048;  // workgroups the LDS kernel's work is cut into (about)
+constexpr int CORE_WAVES = CORE_GROUP_ROWS / 64;  // slices (of 64 rows) per workgroup: as small as the aggregation's own
+                                                  // workgroups, so the two kernels of a call, running side by side, find
+                                                  // room on a CU equally easily
 
 // tab[s * tab_stride(core) + i] = elements 4 s .. 4 s + 3 of the feature row of the rank-i node (zero past dim)
 __global__ void __launch_bounds__(256) k_core_stage(v4f *__restrict__ tab, const float *__restrict__ in, const int *__restrict__ order,
@@ -43,37 +45,33 @@ __global__ void __launch_bounds__(256) k_core_stage(v4f *__restrict__ tab, const
     tab[(size_t)s * tab_stride(core) + i] = v;
 }
 
-// One workgroup = CORE_WAVES slices x one segment of `tiles_per_seg` column tiles; lane = core row.
-// partial[(seg * part_stride(core) + rank) * N4 + s]
+// One workgroup = CORE_WAVES slices (a row group) x a run of column tiles; lane = core row.  Row groups and tiles are both
+// sorted by degree, so the work of a (row group, tile) cell spans two orders of magnitude: the plan cuts every row
+// group's tiles into runs of about equal list length (wgs[i] = {row group, first tile, end tile, slot}), so all
+// workgroups take about the same time and the launch has no tail of a few heavy ones.
+// partial[(slot * CORE_WAVES * 64 + row in the group) * N4 + s]
 template <int N4>
 __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *__restrict__ blk_off, const unsigned short *__restrict__ idx,
-                                                               const v4f *__restrict__ tab, v4f *__restrict__ partial, int core, int ntiles,
-                                                               int nseg, const Gate gate)
+                                                               const v4f *__restrict__ tab, v4f *__restrict__ partial,
+                                                               const int4 *__restrict__ wgs, int core, int ntiles, const Gate gate)
 {
     constexpr int TC = CORE_TC, TP = TC + 1;  // column TC of every slice row is zero: what padding entries read
     extern __shared__ v4f tile[];             // [N4][TP]
     if (gate_closed(gate)) return;
     const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
-    // Consecutive workgroups go to the 8 XCDs in turn and the row groups are sorted by degree: with a number of row groups
-    // that is a multiple of 8, XCD 0 would get the heaviest group of every eight in every segment.  Rotating the row
-    // groups by the segment number spreads them (measured at 32,768 rows: 6 % of the whole aggregation).
-    const int seg = (int)blockIdx.y;
-    const int g = (int)(((unsigned)blockIdx.x + (unsigned)seg) % gridDim.x) * CORE_WAVES + wave;
+    const int4 wg = wgs[blockIdx.x];
+    const int g = wg.x * CORE_WAVES + wave;
+    const int t0 = wg.y, t1 = wg.z;
     v4f acc[N4];
 #pragma unroll
     for (int s = 0; s < N4; ++s) acc[s] = (v4f){0.f, 0.f, 0.f, 0.f};
     if ((int)threadIdx.x < N4) tile[(int)threadIdx.x * TP + TC] = (v4f){0.f, 0.f, 0.f, 0.f};
-    // segment `seg` takes the tiles [seg * ntiles / nseg, (seg + 1) * ntiles / nseg): any number of tiles splits into
-    // segments whose lengths differ by at most one
-    const int t0 = (int)((long long)seg * ntiles / nseg);
-    const int tiles_per_seg = (int)((long long)(seg + 1) * ntiles / nseg) - t0;
     const us4 *p = reinterpret_cast<const us4 *>(idx) + lane;
     unsigned pos = blk_off[(size_t)g * ntiles + t0];
-    const unsigned end_seg = blk_off[(size_t)g * ntiles + t0 + tiles_per_seg];
+    const unsigned end_run = blk_off[(size_t)g * ntiles + t1];
     const us4 pad = (us4){0xFFFF, 0xFFFF, 0xFFFF, 0xFFFF};
-    us4 cur = pos < end_seg ? p[(size_t)pos * 64] : pad;  // the lists of a slice's tiles follow one another: read one chunk ahead
-    for (int tt = 0; tt < tiles_per_seg; ++tt) {
-        const int t = t0 + tt;
+    us4 cur = pos < end_run ? p[(size_t)pos * 64] : pad;  // the lists of a slice's tiles follow one another: read one chunk ahead
+    for (int t = t0; t < t1; ++t) {
         __syncthreads();
         for (int i = (int)threadIdx.x; i < N4 * TC; i += CORE_WAVES * 64) {
             const int s = i / TC, c = i % TC;
@@ -82,7 +80,7 @@ __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *_
         const unsigned b1 = blk_off[(size_t)g * ntiles + t + 1];
         __syncthreads();
         while (pos < b1) {
-            const us4 nxt = pos + 1 < end_seg ? p[(size_t)(pos + 1) * 64] : pad;
+            const us4 nxt = pos + 1 < end_run ? p[(size_t)(pos + 1) * 64] : pad;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int c = cur[j];
@@ -103,18 +101,20 @@ __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *_
             ++pos;
         }
     }
-    const int r = g * 64 + lane;
+    const size_t r = (size_t)wg.w * (CORE_WAVES * 64) + (size_t)(wave * 64 + lane);
 #pragma unroll
-    for (int s = 0; s < N4; ++s) partial[((size_t)seg * part_stride(core) + r) * N4 + s] = acc[s];
+    for (int s = 0; s < N4; ++s) partial[r * N4 + s] = acc[s];
 }
 
 // Adds the core block's sums to output rows that already hold the rest of the aggregation:
-// out[v] = post(out[v] + scale[v] * sum over segments of the partial rows of v), post = ReLU and / or row softmax.
+// out[v] = post(out[v] + scale[v] * sum over the workgroups of v's row group of their partial rows of v), post = ReLU
+// and / or row softmax.
 // G lanes per row (a power of two >= ceil(dim/4)), lane q holds columns 4 q .. 4 q + 3.  all_rows = 0: the core rows only
 // (index -> rank -> row); all_rows = 1: every row (needed when there is a post-operation).
 __global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, const v4f *__restrict__ partial, const int *__restrict__ rank,
                                                      const int *__restrict__ order, const float *__restrict__ rs, int rows, int dim,
-                                                     long long ld_out, int core, int nseg, int G, int relu, int softmax, int all_rows, const Gate gate)
+                                                     long long ld_out, int core, const int *__restrict__ wg_base, int G, int relu, int softmax,
+                                                     int all_rows, const Gate gate)
 {
     if (gate_closed(gate)) return;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -131,7 +131,9 @@ __global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, co
     if (lane_on) {
         v4f sum = {0.f, 0.f, 0.f, 0.f};
         if (r >= 0) {
-            for (int seg = 0; seg < nseg; ++seg) sum += partial[((size_t)seg * part_stride(core) + r) * n4 + q];
+            const int grp = r / (CORE_WAVES * 64), in_grp = r % (CORE_WAVES * 64);
+            const int s1 = wg_base[grp + 1];
+            for (int slot = wg_base[grp]; slot < s1; ++slot) sum += partial[((size_t)slot * (CORE_WAVES * 64) + in_grp) * n4 + q];
             if (rs) sum *= rs[v];
         }
 #pragma unroll
@@ -245,6 +247,17 @@ __global__ void __launch_bounds__(256) k_core_widths(const unsigned short *__res
     chunks[idx] = (w + 3) / 4;
 }
 
+// work[g * ntiles + t] = list chunks of the CORE_WAVES slices of row group g in tile t
+__global__ void __launch_bounds__(256) k_core_group_work(const int *__restrict__ chunks, int groups, int ntiles, int *__restrict__ work)
+{
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long long)groups * ntiles) return;
+    const int g = (int)(idx / ntiles), t = (int)(idx % ntiles);
+    int w = 0;
+    for (int k = 0; k < CORE_WAVES; ++k) w += chunks[(size_t)(g * CORE_WAVES + k) * ntiles + t];
+    work[idx] = w;
+}
+
 // Pass 2, one wavefront per row, 64 neighbors at a time in edge order: neighbors that stay go to the remaining CSR (order
 // kept); a core row's core neighbors go to the list of their tile, the k-th of a tile (in edge order) to list position k.
 // Inside a group of 64 every lane finds the lanes with the same tile by one ballot per bit of the tile number; the counts
@@ -320,10 +333,7 @@ int launch_sell(const CorePlan *p, const v4f *tab, v4f *partial, const Gate &gat
         MGGX_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_core_sell<N4>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         raised = true;
     }
-    // row groups vary fastest in the grid: workgroups that run side by side then read the same tiles, and a CU holds dense
-    // and sparse row groups at once (the reverse order measured 25 % slower)
-    const dim3 grid((unsigned)(p->core / (CORE_WAVES * 64)), (unsigned)p->nseg);
-    k_core_sell<N4><<<grid, dim3(CORE_WAVES * 64), lds, stream>>>(p->d_blk_off, p->d_idx, tab, partial, p->core, p->ntiles, p->nseg, gate);
+    k_core_sell<N4><<<dim3((unsigned)p->nwg), dim3(CORE_WAVES * 64), lds, stream>>>(p->d_blk_off, p->d_idx, tab, partial, p->d_wgs, p->core, p->ntiles, gate);
     MGGX_LAUNCH_CHECK("k_core_sell");
     return MGGX_OK;
 }
@@ -336,6 +346,8 @@ void core_plan_free_arrays(CorePlan *p)
     if (p->d_idx) (void)hipFree(p->d_idx);
     if (p->d_rem_ptr) (void)hipFree(p->d_rem_ptr);
     if (p->d_rem_col) (void)hipFree(p->d_rem_col);
+    if (p->d_wgs) (void)hipFree(p->d_wgs);
+    if (p->d_wg_base) (void)hipFree(p->d_wg_base);
 }
 
 }  // namespace
@@ -409,12 +421,13 @@ static int core_plan_build_device(CorePlan *p, int tc)
     const int ntiles = core / tc, nslices = core / 64;
     if (ntiles > 2048) return fail(MGGX_ELIMIT, "core plan: %d core rows", core);
     Scratch tmp;
-    int *deg = nullptr, *deg_sorted = nullptr, *ids = nullptr, *sorted = nullptr, *keep = nullptr, *chunks = nullptr, *flag = nullptr, *blk = nullptr;
+    int *deg = nullptr, *deg_sorted = nullptr, *ids = nullptr, *sorted = nullptr, *keep = nullptr, *chunks = nullptr, *flag = nullptr, *blk = nullptr, *work = nullptr;
     unsigned short *cnt = nullptr;
     int rc;
     if ((rc = tmp.get(&deg, (size_t)rows)) || (rc = tmp.get(&deg_sorted, (size_t)rows)) || (rc = tmp.get(&ids, (size_t)rows)) ||
         (rc = tmp.get(&sorted, (size_t)rows)) || (rc = tmp.get(&keep, (size_t)rows)) || (rc = tmp.get(&chunks, (size_t)nslices * ntiles)) ||
-        (rc = tmp.get(&flag, 1)) || (rc = tmp.get(&cnt, (size_t)core * ntiles)) || (rc = tmp.get(&blk, (size_t)nslices * ntiles + 1)))
+        (rc = tmp.get(&flag, 1)) || (rc = tmp.get(&cnt, (size_t)core * ntiles)) || (rc = tmp.get(&blk, (size_t)nslices * ntiles + 1)) ||
+        (rc = tmp.get(&work, (size_t)(nslices / CORE_WAVES) * ntiles)))
         return rc;
     if ((rc = device_array(&p->d_order, (size_t)core)) || (rc = device_array(&p->d_rank, (size_t)rows)) ||
         (rc = device_array(&p->d_blk_off, (size_t)nslices * ntiles + 1)) || (rc = device_array(&p->d_rem_ptr, (size_t)rows + 1)))
@@ -460,13 +473,48 @@ static int core_plan_build_device(CorePlan *p, int tc)
     p->ntiles = ntiles;
     p->rem_nnz = rem_nnz;
     p->core_nnz = (int64_t)nnz - rem_nnz;
-    // segments: enough workgroups (about 2048) to fill the chip a few times over, whole tiles each
-    const int groups = core / (CORE_WAVES * 64);
-    int nseg = (2048 + groups / 2) / groups;
-    if (nseg > ntiles) nseg = ntiles;
-    if (nseg < 1) nseg = 1;
-    p->nseg = nseg;
-    p->bytes = ((size_t)core + 2 * (size_t)rows + 1 + (size_t)rem_nnz + (size_t)nblk + 1) * sizeof(int) + idx_elems * sizeof(unsigned short);
+    // Workgroups of the LDS kernel: every row group's tiles cut into runs of about total / 2048 list chunks (a run ends
+    // where half of the next tile would overshoot that), enough workgroups to fill the chip a few times over and none
+    // much longer than the others.  Launch order: the first run of every row group, then the second of those that have
+    // one, ... -- neighbors in the launch, which share a CU, then read different rows' lists and mostly the same tiles.
+    // The cut needs one number per (row group, tile), reduced on the GPU: 64 KB for a core of 32,768 rows.
+    const int groups = core / CORE_GROUP_ROWS;
+    k_core_group_work<<<(unsigned)(((long long)groups * ntiles + 255) / 256), 256, 0, s.stream>>>(chunks, groups, ntiles, work);
+    MGGX_LAUNCH_CHECK("k_core_group_work");
+    std::vector<int> h_work((size_t)groups * ntiles);
+    MGGX_HIP(hipMemcpyAsync(h_work.data(), work, h_work.size() * sizeof(int), hipMemcpyDeviceToHost, s.stream));
+    MGGX_HIP(hipStreamSynchronize(s.stream));
+    const long long target = std::max<long long>((total_chunks + CORE_TARGET_WGS - 1) / CORE_TARGET_WGS, 1);
+    std::vector<int4> runs;                      // row-group-major: slot order
+    std::vector<int> wg_base((size_t)groups + 1, 0);
+    int longest = 0;
+    for (int g = 0; g < groups; ++g) {
+        long long acc = 0;
+        int first = 0;
+        for (int t = 0; t < ntiles; ++t) {
+            const int w = h_work[(size_t)g * ntiles + t];
+            if (t > first && acc + w / 2 > target) {
+                runs.push_back(make_int4(g, first, t, (int)runs.size()));
+                first = t;
+                acc = 0;
+            }
+            acc += w;
+        }
+        runs.push_back(make_int4(g, first, ntiles, (int)runs.size()));
+        wg_base[(size_t)g + 1] = (int)runs.size();
+        longest = std::max(longest, wg_base[(size_t)g + 1] - wg_base[(size_t)g]);
+    }
+    std::vector<int4> launch;
+    launch.reserve(runs.size());
+    for (int k = 0; k < longest; ++k)
+        for (int g = 0; g < groups; ++g)
+            if (wg_base[(size_t)g] + k < wg_base[(size_t)g + 1]) launch.push_back(runs[(size_t)wg_base[(size_t)g] + k]);
+    p->nwg = (int)launch.size();
+    if ((rc = device_array(&p->d_wgs, launch.size())) || (rc = device_array(&p->d_wg_base, wg_base.size()))) return rc;
+    MGGX_HIP(hipMemcpy(p->d_wgs, launch.data(), launch.size() * sizeof(int4), hipMemcpyHostToDevice));
+    MGGX_HIP(hipMemcpy(p->d_wg_base, wg_base.data(), wg_base.size() * sizeof(int), hipMemcpyHostToDevice));
+    p->bytes = ((size_t)core + 2 * (size_t)rows + 1 + (size_t)rem_nnz + (size_t)nblk + 1 + wg_base.size()) * sizeof(int) + idx_elems * sizeof(unsigned short) +
+               launch.size() * sizeof(int4);
     return MGGX_OK;
 }
 
@@ -516,12 +564,12 @@ int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int 
     return MGGX_OK;
 }
 
-// Scratch of the dense-core path: the staged core table, then one partial row per core row and segment.
+// Scratch of the dense-core path: the staged core table, then one partial row per workgroup of the LDS kernel and row of its group.
 static int core_scratch(const CorePlan *p, int n4, v4f **tab, v4f **partial)
 {
     State &s = state();
     const size_t tab_bytes = (tab_stride(p->core) * n4 * sizeof(v4f) + 255) & ~(size_t)255;
-    const size_t part_bytes = (size_t)p->nseg * part_stride(p->core) * n4 * sizeof(v4f);
+    const size_t part_bytes = (size_t)p->nwg * CORE_GROUP_ROWS * n4 * sizeof(v4f);
     if (tab_bytes + part_bytes > s.core_ws_bytes) {
         if (capturing()) return fail(MGGX_EINVAL, "core: the scratch block would have to grow inside a stream capture; run the largest call once outside it first");
         MGGX_HIP(hipDeviceSynchronize());  // both streams may still use the old block
@@ -591,7 +639,7 @@ int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const 
     while (G < n4) G <<= 1;
     const long long n = (long long)(all_rows ? p->rows : p->core) * G;
     k_core_finish<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(d_out, partial, p->d_rank, p->d_order, d_row_scale, p->rows, dim, ld_out,
-                                                                                p->core, p->nseg, G, relu, softmax, all_rows, gate);
+                                                                                p->core, p->d_wg_base, G, relu, softmax, all_rows, gate);
     MGGX_LAUNCH_CHECK("k_core_finish");
     return MGGX_OK;
 }
@@ -618,17 +666,18 @@ int core_partial_rows(CorePlan *p, int dim, const float4 **partial_out)
 // useful and the padded entries of any core size from the degree histogram alone (within 3 % of the built plans on the
 // benchmark graphs).  Growing the core by a band of rows pays while the band's useful entries per padded entry stay
 // above theta = (cost of one padded entry in the LDS kernel) / (cost of one edge in the gather kernel)
-//             = ALPHA x ceil(dim/4) / (BETA x 64-byte sectors of a row x (1 or HBM_FACTOR)),
+//             = ALPHA x ceil(dim/4) / (BETA x (1 + 64-byte sectors of a row) x (1 or HBM_FACTOR)),
 // constants fitted to sweeps of the core size on the 233 K-node width-16 / width-44 and the 2.45 M-node width-64
-// graphs (ALPHA 1.1 ps per padded 16-byte piece; BETA 9 ps per 64-byte sector of a gathered row while the table fits
-// the 256 MB last-level cache, 2.3 x that beyond).
+// graphs (ALPHA 1.42 ps per padded 16-byte piece; BETA 9 ps per gathered row plus as much per 64-byte sector of it while
+// the table fits the 256 MB last-level cache, 3.2 x that beyond).  The staging of the tiles (core^2 / 65536 tiles of
+// 256 x ceil(dim/4) x 16 bytes per row group) is not in the model; it shows beyond 80,000 rows, where the model stops.
 namespace mggx {
 namespace {
 
-constexpr int PROFILE_SLICES = 1024;  // 65536 ranks
-constexpr double ALPHA_PS = 1.1, BETA_PS = 9.0, HBM_FACTOR = 2.3;
+constexpr int PROFILE_SLICES = 2048;  // 131072 ranks
+constexpr double ALPHA_PS = 1.42, BETA_PS = 9.0, HBM_FACTOR = 3.2;
 constexpr unsigned long long LAST_LEVEL_CACHE_BYTES = 256ull << 20;
-constexpr int MODEL_STEP = 4096, MODEL_MAX_CORE = 57344;
+constexpr int MODEL_STEP = 4096, MODEL_MAX_CORE = 81920;
 
 __global__ void __launch_bounds__(256) k_degrees(const int *__restrict__ ptr, int rows, int *__restrict__ deg)
 {
@@ -725,7 +774,7 @@ int predict_core_rows(GraphInfo &g, int dim, unsigned long long table_bytes, int
     if (rc) return rc;
     const int n4 = (dim + 3) / 4;
     const int sectors = (dim * 4 + 63) / 64;
-    const double theta = ALPHA_PS * n4 / (BETA_PS * sectors * (beyond_cache ? HBM_FACTOR : 1.0));
+    const double theta = ALPHA_PS * n4 / (BETA_PS * (1 + sectors) * (beyond_cache ? HBM_FACTOR : 1.0));
     const double nnz = (double)g.nnz_l;
     const int max_core = std::min({MODEL_MAX_CORE, g.rows / 2 / MODEL_STEP * MODEL_STEP, (int)g.slice_deg.size() * 64 / MODEL_STEP * MODEL_STEP});
     // useful and padded entries of the block (slices [s0, s1) x tiles [t0, t1))

@@ -114,13 +114,13 @@ struct Plan {
     Guard guard;               // explicit-partition plans only (the others are guarded through their GraphInfo)
 };
 
-// Scratch layout of the dense core.  Staged table: slice s of the rank-i node's row at tab[s * tab_stride(core) + i];
-// partial rows: segment seg of rank r at partial[(seg * part_stride(core) + r) * n4 + piece].  Both strides carry a few
-// rows more than the core size: with a power-of-two core the slices of a tile, and the segments of one row that the
-// finishing kernel reads together, would otherwise all start in the same memory channel (measured at 32,768 rows: 6 %
-// of the whole aggregation).
+// Scratch layout of the dense core.  Staged table: slice s of the rank-i node's row at tab[s * tab_stride(core) + i]; the
+// stride carries a few rows more than the core size: with a power-of-two core the slices of a tile would otherwise all
+// start in the same memory channel.  Partial rows: one per workgroup of the LDS kernel and row of its row group, at
+// partial[(slot * CORE_GROUP_ROWS + rank % CORE_GROUP_ROWS) * n4 + piece]; the slots of row group g are
+// wg_base[g] .. wg_base[g + 1] - 1.
 __host__ __device__ inline size_t tab_stride(int core) { return (size_t)core + 16; }
-__host__ __device__ inline size_t part_stride(int core) { return (size_t)core + 24; }
+constexpr int CORE_GROUP_ROWS = 256;  // core rows per workgroup of the LDS kernel (4 wavefronts, one row per lane)
 
 // Dense-core plan of a local-only CSR (layout: CoreLayout in mggx_internal.h), built on the GPU and kept there.
 struct CorePlan {
@@ -129,12 +129,15 @@ struct CorePlan {
     const int *d_col_l = nullptr;
     int rows = 0, lb = 0, asked = 0;
     // contents
-    int core = 0, ntiles = 0, nseg = 1;
+    int core = 0, ntiles = 0;
+    int nwg = 0;              // workgroups of the LDS kernel: runs of column tiles of about equal work per row group
     int64_t core_nnz = 0, rem_nnz = 0;
     int *d_order = nullptr, *d_rank = nullptr;
     unsigned *d_blk_off = nullptr;
     unsigned short *d_idx = nullptr;
     int *d_rem_ptr = nullptr, *d_rem_col = nullptr;
+    int4 *d_wgs = nullptr;    // [nwg] {row group, first tile, end tile, slot of the partial rows}, in launch order
+    int *d_wg_base = nullptr; // [core / CORE_GROUP_ROWS + 1] first slot of every row group
     bool unsuitable = false;  // no core of whole units fits, or the ids do not allow it
     bool pinned = false;      // used inside a stream capture: never evicted
     size_t bytes = 0;         // device memory held
@@ -147,7 +150,7 @@ struct GraphInfo {
     const int *d_col_l = nullptr;
     const int *d_col_r = nullptr;
     int rows = 0;
-    // degree profile for the dense-core cost model: sum of the degrees of ranks [64 s, 64 s + 64) for the 1024 highest-degree
+    // degree profile for the dense-core cost model: sum of the degrees of ranks [64 s, 64 s + 64) for the 2048 highest-degree
     // slices (rows ranked by falling degree), fetched once per record
     std::vector<float> slice_deg;
     bool have_profile = false;
@@ -228,7 +231,7 @@ int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, con
 int run_core_sums(CorePlan *p, int dim, const Gate &gate, hipStream_t stream);
 int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, int softmax, const Gate &gate,
                     hipStream_t stream);
-// Where run_core_sums leaves the core block's sums: [segment][rank][ceil(dim/4)] float4.
+// Where run_core_sums leaves the core block's sums: [slot][row in its group][ceil(dim/4)] float4 (CorePlan::d_wg_base).
 int core_partial_rows(CorePlan *p, int dim, const float4 **partial);
 // Second stream of the dense-core path (created on first use, default priority) and the two events that fork and join it.
 int core_side_stream(hipStream_t *stream, hipEvent_t *fork, hipEvent_t *join);

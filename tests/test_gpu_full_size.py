@@ -57,7 +57,7 @@ def test_full_size_gin_graph_layer(gpu):
         gpu.sync()
         if core_rows == 0:
             m = re.search(r"core=(\d+)", gpu.last_agg_kernel())
-            assert m and 28672 <= int(m.group(1)) <= 57344, gpu.last_agg_kernel()  # the swept optimum lies between 32 and 56 Ki rows
+            assert m and 57344 <= int(m.group(1)) <= 86016, gpu.last_agg_kernel()  # the swept optimum is flat between 72 and 84 Ki rows
         else:
             assert ("core=40960" in gpu.last_agg_kernel()) == (core_rows > 0)
         h = H.cpu().numpy()
@@ -180,7 +180,7 @@ def test_full_size_gcn_forward_end_to_end(gpu, core_rows):
                        ld_out=pitch)
     gpu.softmax_forward(P, H2, V, out_dim, ld_in=pitch)
     gpu.sync()
-    if core_rows == 0:  # the cost model's choice: the swept optimum is flat between 32 and 48 Ki rows
+    if core_rows == 0:  # the cost model's choice: the swept optimum lies at 36 Ki rows, within 5 % from 32 to 48 Ki
         m = re.search(r"core=(\d+)", gpu.last_agg_kernel())
         assert m and 28672 <= int(m.group(1)) <= 49152, gpu.last_agg_kernel()
     else:
