@@ -1181,8 +1181,8 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
             const hipError_t er = hipEventRecord(join, side);
             int rc2 = MGGX_OK;
             GraphInfo *gr = nullptr;
-            CoreMerge cm{nullptr, cp->d_rank, cp->d_wg_base, join, false};
-            if (!rc) rc2 = core_partial_rows(cp, dim, &cm.partial);
+            CoreMerge cm{nullptr, cp->d_rank, nullptr, join, false};
+            if (!rc) rc2 = core_partial_rows(cp, dim, &cm.partial, &cm.wg_base);
             if (!rc && !rc2) rc2 = graph_info(cp->d_rem_ptr, nullptr, cp->d_rem_col, nullptr, ub - lb, true, &gr);
             if (!rc && !rc2 && er == hipSuccess) {
                 Knobs k2 = k;

@@ -23,7 +23,6 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned short us4 __attribute__((ext_vector_type(4)));
 
 constexpr int CORE_TC = 256;    // core columns per LDS tile
-constexpr int CORE_TARGET_WGS = 2048;  // workgroups the LDS kernel's work is cut into (about)
 constexpr int CORE_WAVES = CORE_GROUP_ROWS / 64;  // slices (of 64 rows) per workgroup: as small as the aggregation's own
                                                   // workgroups, so the two kernels of a call, running side by side, find
                                                   // room on a CU equally easily
@@ -325,7 +324,7 @@ __global__ void __launch_bounds__(BUILD_WAVES * 64) k_core_fill(const int *__res
 }
 
 template <int N4>
-int launch_sell(const CorePlan *p, const v4f *tab, v4f *partial, const Gate &gate, hipStream_t stream)
+int launch_sell(const CorePlan *p, const CorePlan::Cut &cut, const v4f *tab, v4f *partial, const Gate &gate, hipStream_t stream)
 {
     const size_t lds = (size_t)N4 * (CORE_TC + 1) * sizeof(v4f);
     static bool raised = false;  // per instantiation
@@ -333,7 +332,7 @@ int launch_sell(const CorePlan *p, const v4f *tab, v4f *partial, const Gate &gat
         MGGX_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_core_sell<N4>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         raised = true;
     }
-    k_core_sell<N4><<<dim3((unsigned)p->nwg), dim3(CORE_WAVES * 64), lds, stream>>>(p->d_blk_off, p->d_idx, tab, partial, p->d_wgs, p->core, p->ntiles, gate);
+    k_core_sell<N4><<<dim3((unsigned)cut.nwg), dim3(CORE_WAVES * 64), lds, stream>>>(p->d_blk_off, p->d_idx, tab, partial, cut.d_wgs, p->core, p->ntiles, gate);
     MGGX_LAUNCH_CHECK("k_core_sell");
     return MGGX_OK;
 }
@@ -346,8 +345,11 @@ void core_plan_free_arrays(CorePlan *p)
     if (p->d_idx) (void)hipFree(p->d_idx);
     if (p->d_rem_ptr) (void)hipFree(p->d_rem_ptr);
     if (p->d_rem_col) (void)hipFree(p->d_rem_col);
-    if (p->d_wgs) (void)hipFree(p->d_wgs);
-    if (p->d_wg_base) (void)hipFree(p->d_wg_base);
+    for (CorePlan::Cut &c : p->cuts) {
+        if (c.d_wgs) (void)hipFree(c.d_wgs);
+        if (c.d_wg_base) (void)hipFree(c.d_wg_base);
+    }
+    p->cuts.clear();
 }
 
 }  // namespace
@@ -473,48 +475,16 @@ static int core_plan_build_device(CorePlan *p, int tc)
     p->ntiles = ntiles;
     p->rem_nnz = rem_nnz;
     p->core_nnz = (int64_t)nnz - rem_nnz;
-    // Workgroups of the LDS kernel: every row group's tiles cut into runs of about total / 2048 list chunks (a run ends
-    // where half of the next tile would overshoot that), enough workgroups to fill the chip a few times over and none
-    // much longer than the others.  Launch order: the first run of every row group, then the second of those that have
-    // one, ... -- neighbors in the launch, which share a CU, then read different rows' lists and mostly the same tiles.
-    // The cut needs one number per (row group, tile), reduced on the GPU: 64 KB for a core of 32,768 rows.
+    // What cutting the LDS kernel's work into workgroups needs later: one number per (row group, tile), reduced on the GPU
+    // (64 KB for a core of 32,768 rows)
     const int groups = core / CORE_GROUP_ROWS;
     k_core_group_work<<<(unsigned)(((long long)groups * ntiles + 255) / 256), 256, 0, s.stream>>>(chunks, groups, ntiles, work);
     MGGX_LAUNCH_CHECK("k_core_group_work");
-    std::vector<int> h_work((size_t)groups * ntiles);
-    MGGX_HIP(hipMemcpyAsync(h_work.data(), work, h_work.size() * sizeof(int), hipMemcpyDeviceToHost, s.stream));
+    p->work.resize((size_t)groups * ntiles);
+    MGGX_HIP(hipMemcpyAsync(p->work.data(), work, p->work.size() * sizeof(int), hipMemcpyDeviceToHost, s.stream));
     MGGX_HIP(hipStreamSynchronize(s.stream));
-    const long long target = std::max<long long>((total_chunks + CORE_TARGET_WGS - 1) / CORE_TARGET_WGS, 1);
-    std::vector<int4> runs;                      // row-group-major: slot order
-    std::vector<int> wg_base((size_t)groups + 1, 0);
-    int longest = 0;
-    for (int g = 0; g < groups; ++g) {
-        long long acc = 0;
-        int first = 0;
-        for (int t = 0; t < ntiles; ++t) {
-            const int w = h_work[(size_t)g * ntiles + t];
-            if (t > first && acc + w / 2 > target) {
-                runs.push_back(make_int4(g, first, t, (int)runs.size()));
-                first = t;
-                acc = 0;
-            }
-            acc += w;
-        }
-        runs.push_back(make_int4(g, first, ntiles, (int)runs.size()));
-        wg_base[(size_t)g + 1] = (int)runs.size();
-        longest = std::max(longest, wg_base[(size_t)g + 1] - wg_base[(size_t)g]);
-    }
-    std::vector<int4> launch;
-    launch.reserve(runs.size());
-    for (int k = 0; k < longest; ++k)
-        for (int g = 0; g < groups; ++g)
-            if (wg_base[(size_t)g] + k < wg_base[(size_t)g + 1]) launch.push_back(runs[(size_t)wg_base[(size_t)g] + k]);
-    p->nwg = (int)launch.size();
-    if ((rc = device_array(&p->d_wgs, launch.size())) || (rc = device_array(&p->d_wg_base, wg_base.size()))) return rc;
-    MGGX_HIP(hipMemcpy(p->d_wgs, launch.data(), launch.size() * sizeof(int4), hipMemcpyHostToDevice));
-    MGGX_HIP(hipMemcpy(p->d_wg_base, wg_base.data(), wg_base.size() * sizeof(int), hipMemcpyHostToDevice));
-    p->bytes = ((size_t)core + 2 * (size_t)rows + 1 + (size_t)rem_nnz + (size_t)nblk + 1 + wg_base.size()) * sizeof(int) + idx_elems * sizeof(unsigned short) +
-               launch.size() * sizeof(int4);
+    p->total_chunks = total_chunks;
+    p->bytes = ((size_t)core + 2 * (size_t)rows + 1 + (size_t)rem_nnz + (size_t)nblk + 1) * sizeof(int) + idx_elems * sizeof(unsigned short);
     return MGGX_OK;
 }
 
@@ -564,12 +534,78 @@ int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int 
     return MGGX_OK;
 }
 
+// The workgroups of the LDS kernel for rows of n4 16-byte pieces: every row group's tiles cut into runs of about
+// total / target list chunks (a run ends where half of the next tile would overshoot that), so no workgroup runs much
+// longer than the others -- row groups and tiles are both sorted by degree, and equal numbers of tiles would differ in
+// work a hundredfold.  Narrow rows: about 3072 workgroups (short ones; the kernel's own tail matters most); wide rows:
+// about 1280 (every workgroup costs 256 partial rows that the finishing kernel reads back).  Measured on the 233 K-node
+// graph at widths 16 / 44 and the 2.45 M-node graph at width 64: 1024 / 1536 / 2048 / 3072 workgroups give
+// 0.72 / 0.62 / 0.59 / 0.57, 1.41 / 1.42 / 1.43 / 1.53 and 3.02 / 2.98 / 3.01 / 3.03 ms per aggregation.
+// Launch order: the first run of every row group, then the second of those that have one, ... -- neighbors in the
+// launch, which share a CU, then read different rows' lists and mostly the same tiles.
+static int core_cut(CorePlan *p, int n4, const CorePlan::Cut **out)
+{
+    const int want = n4 <= 6 ? 3072 : 1280;
+    for (const CorePlan::Cut &c : p->cuts)
+        if (c.target == want) {
+            *out = &c;
+            return MGGX_OK;
+        }
+    if (capturing()) return fail(MGGX_EINVAL, "core: first use of this core with rows of this width inside a stream capture; call once outside the capture first");
+    const int groups = p->core / CORE_GROUP_ROWS, ntiles = p->ntiles;
+    const long long target = std::max<long long>((p->total_chunks + want - 1) / want, 1);
+    std::vector<int4> runs;  // row-group-major: slot order
+    std::vector<int> wg_base((size_t)groups + 1, 0);
+    int longest = 0;
+    for (int g = 0; g < groups; ++g) {
+        long long acc = 0;
+        int first = 0;
+        for (int t = 0; t < ntiles; ++t) {
+            const int w = p->work[(size_t)g * ntiles + t];
+            if (t > first && acc + w / 2 > target) {
+                runs.push_back(make_int4(g, first, t, (int)runs.size()));
+                first = t;
+                acc = 0;
+            }
+            acc += w;
+        }
+        runs.push_back(make_int4(g, first, ntiles, (int)runs.size()));
+        wg_base[(size_t)g + 1] = (int)runs.size();
+        longest = std::max(longest, wg_base[(size_t)g + 1] - wg_base[(size_t)g]);
+    }
+    std::vector<int4> launch;
+    launch.reserve(runs.size());
+    for (int k = 0; k < longest; ++k)
+        for (int g = 0; g < groups; ++g)
+            if (wg_base[(size_t)g] + k < wg_base[(size_t)g + 1]) launch.push_back(runs[(size_t)wg_base[(size_t)g] + k]);
+    CorePlan::Cut c;
+    c.target = want;
+    c.nwg = (int)launch.size();
+    int rc;
+    if ((rc = device_array(&c.d_wgs, launch.size()))) return rc;
+    if ((rc = device_array(&c.d_wg_base, wg_base.size()))) {
+        (void)hipFree(c.d_wgs);
+        return rc;
+    }
+    p->cuts.reserve(4);  // pointers into the vector are handed out: two targets exist
+    p->cuts.push_back(c);
+    MGGX_HIP(hipMemcpy(c.d_wgs, launch.data(), launch.size() * sizeof(int4), hipMemcpyHostToDevice));
+    MGGX_HIP(hipMemcpy(c.d_wg_base, wg_base.data(), wg_base.size() * sizeof(int), hipMemcpyHostToDevice));
+    p->bytes += launch.size() * sizeof(int4) + wg_base.size() * sizeof(int);
+    *out = &p->cuts.back();
+    return MGGX_OK;
+}
+
 // Scratch of the dense-core path: the staged core table, then one partial row per workgroup of the LDS kernel and row of its group.
-static int core_scratch(const CorePlan *p, int n4, v4f **tab, v4f **partial)
+static int core_scratch(CorePlan *p, int n4, v4f **tab, v4f **partial, const CorePlan::Cut **cut_out = nullptr)
 {
     State &s = state();
+    const CorePlan::Cut *cut = nullptr;
+    const int rc_cut = core_cut(p, n4, &cut);
+    if (rc_cut) return rc_cut;
+    if (cut_out) *cut_out = cut;
     const size_t tab_bytes = (tab_stride(p->core) * n4 * sizeof(v4f) + 255) & ~(size_t)255;
-    const size_t part_bytes = (size_t)p->nwg * CORE_GROUP_ROWS * n4 * sizeof(v4f);
+    const size_t part_bytes = (size_t)cut->nwg * CORE_GROUP_ROWS * n4 * sizeof(v4f);
     if (tab_bytes + part_bytes > s.core_ws_bytes) {
         if (capturing()) return fail(MGGX_EINVAL, "core: the scratch block would have to grow inside a stream capture; run the largest call once outside it first");
         MGGX_HIP(hipDeviceSynchronize());  // both streams may still use the old block
@@ -614,10 +650,11 @@ int run_core_sums(CorePlan *p, int dim, const Gate &gate, hipStream_t stream)
     const int n4 = (dim + 3) / 4;
     if (n4 < 1 || n4 > 16) return fail(MGGX_ELIMIT, "core: dim %d outside 1..64", dim);
     v4f *tab = nullptr, *partial = nullptr;
-    int rc = core_scratch(p, n4, &tab, &partial);
+    const CorePlan::Cut *cut = nullptr;
+    int rc = core_scratch(p, n4, &tab, &partial, &cut);
     if (rc) return rc;
     switch (n4) {
-#define MGGX_CASE(N) case N: rc = launch_sell<N>(p, tab, partial, gate, stream); break;
+#define MGGX_CASE(N) case N: rc = launch_sell<N>(p, *cut, tab, partial, gate, stream); break;
         MGGX_CASE(1) MGGX_CASE(2) MGGX_CASE(3) MGGX_CASE(4) MGGX_CASE(5) MGGX_CASE(6) MGGX_CASE(7) MGGX_CASE(8)
         MGGX_CASE(9) MGGX_CASE(10) MGGX_CASE(11) MGGX_CASE(12) MGGX_CASE(13) MGGX_CASE(14) MGGX_CASE(15) MGGX_CASE(16)
 #undef MGGX_CASE
@@ -632,24 +669,27 @@ int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const 
 {
     const int n4 = (dim + 3) / 4;
     v4f *tab = nullptr, *partial = nullptr;
-    int rc = core_scratch(p, n4, &tab, &partial);  // sized by run_core_sums already: only hands the pointers out
+    const CorePlan::Cut *cut = nullptr;
+    int rc = core_scratch(p, n4, &tab, &partial, &cut);  // sized by run_core_sums already: only hands the pointers out
     if (rc) return rc;
     const int all_rows = (relu || softmax) ? 1 : 0;
     int G = 1;
     while (G < n4) G <<= 1;
     const long long n = (long long)(all_rows ? p->rows : p->core) * G;
     k_core_finish<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(d_out, partial, p->d_rank, p->d_order, d_row_scale, p->rows, dim, ld_out,
-                                                                                p->core, p->d_wg_base, G, relu, softmax, all_rows, gate);
+                                                                                p->core, cut->d_wg_base, G, relu, softmax, all_rows, gate);
     MGGX_LAUNCH_CHECK("k_core_finish");
     return MGGX_OK;
 }
 
-int core_partial_rows(CorePlan *p, int dim, const float4 **partial_out)
+int core_partial_rows(CorePlan *p, int dim, const float4 **partial_out, const int **wg_base)
 {
     const int n4 = (dim + 3) / 4;
     v4f *tab = nullptr, *partial = nullptr;
-    const int rc = core_scratch(p, n4, &tab, &partial);
+    const CorePlan::Cut *cut = nullptr;
+    const int rc = core_scratch(p, n4, &tab, &partial, &cut);
     if (rc) return rc;
+    *wg_base = cut->d_wg_base;
     *partial_out = reinterpret_cast<const float4 *>(partial);
     return MGGX_OK;
 }

@@ -130,14 +130,23 @@ struct CorePlan {
     int rows = 0, lb = 0, asked = 0;
     // contents
     int core = 0, ntiles = 0;
-    int nwg = 0;              // workgroups of the LDS kernel: runs of column tiles of about equal work per row group
     int64_t core_nnz = 0, rem_nnz = 0;
     int *d_order = nullptr, *d_rank = nullptr;
     unsigned *d_blk_off = nullptr;
     unsigned short *d_idx = nullptr;
     int *d_rem_ptr = nullptr, *d_rem_col = nullptr;
-    int4 *d_wgs = nullptr;    // [nwg] {row group, first tile, end tile, slot of the partial rows}, in launch order
-    int *d_wg_base = nullptr; // [core / CORE_GROUP_ROWS + 1] first slot of every row group
+    // Workgroups of the LDS kernel: every row group's tiles cut into runs of about equal work.  How many runs pays depends
+    // on the row width (narrow rows: many short ones; wide rows: fewer, their partial rows are dearer), so a plan holds
+    // one table per number asked for, made from `work` when first needed.
+    struct Cut {
+        int target = 0;            // workgroups asked for
+        int nwg = 0;               // workgroups made
+        int4 *d_wgs = nullptr;     // [nwg] {row group, first tile, end tile, slot of the partial rows}, in launch order
+        int *d_wg_base = nullptr;  // [core / CORE_GROUP_ROWS + 1] first slot of every row group
+    };
+    std::vector<Cut> cuts;
+    std::vector<int> work;    // [core / CORE_GROUP_ROWS][ntiles] list chunks of a row group in a tile (host copy)
+    long long total_chunks = 0;
     bool unsuitable = false;  // no core of whole units fits, or the ids do not allow it
     bool pinned = false;      // used inside a stream capture: never evicted
     size_t bytes = 0;         // device memory held
@@ -231,8 +240,9 @@ int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, con
 int run_core_sums(CorePlan *p, int dim, const Gate &gate, hipStream_t stream);
 int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, int softmax, const Gate &gate,
                     hipStream_t stream);
-// Where run_core_sums leaves the core block's sums: [slot][row in its group][ceil(dim/4)] float4 (CorePlan::d_wg_base).
-int core_partial_rows(CorePlan *p, int dim, const float4 **partial);
+// Where run_core_sums leaves the core block's sums: [slot][row in its group][ceil(dim/4)] float4, and the first slot of
+// every row group (CorePlan::Cut::d_wg_base of the cut used for this width).
+int core_partial_rows(CorePlan *p, int dim, const float4 **partial, const int **wg_base);
 // Second stream of the dense-core path (created on first use, default priority) and the two events that fork and join it.
 int core_side_stream(hipStream_t *stream, hipEvent_t *fork, hipEvent_t *join);
 
