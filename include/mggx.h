@@ -279,10 +279,11 @@ int mggx_sag_np_div(float *d_out, const void *d_in_local, const void *d_in_remot
 /* The design-space search of bench_MGG_DSE_dist_ps.py:12-42 / bench_MGG_DSE_dist_wpb.py (one process launch per
  * setting there) as one call: runs the aggregation of mggx_sag_np_div over ps (as given, or {16, 32} when 0) x plain /
  * column-blocked order (where the rows are long enough, unless opts fixes it) x without a dense core / with one of
- * 32, 40, 48 or 64 Ki rows (where eligible, unless opts fixes it) x wpb in {4, 8, 16} x dist in
+ * 32, 40, 48, 64 or 80 Ki rows (where eligible, unless opts fixes it) x wpb in {4, 8, 16} x dist in
  * {1, 2, 4, 8, 16} -- one untimed and two timed calls back to back per setting; the four fastest settings and the setting
- * the library's own rules and cost model would pick then meet again over eight calls each -- returns the fastest setting
- * and its time (ms per call in that last round), and
+ * the library's own rules and cost model would pick then meet again, twice over eight calls each, the faster of the two
+ * counting (a plan built a moment ago runs slower for its first calls) -- returns the fastest setting and its time (ms
+ * per call in that last round), and
  * remembers it, so later mggx_sag_np_div calls on the same CSR arrays with the same dim and in_dtype that leave
  * wpb = dist = col_block_rows = core_rows = 0 (and ps = 0 or the winning ps) use it.  d_out holds a valid result afterwards.
  * Synchronises; not for stream capture.  MGGX_AGG_ACCUMULATE is rejected (the repeated runs would add up).

@@ -1290,11 +1290,11 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
     int blks[2] = {-1, 0}, n_blk = 1;
     if (o.col_block_rows > 0) blks[0] = o.col_block_rows;
     else if (o.col_block_rows == 0 && mggx::blocking_eligible(*g, mggx::DEFAULT_BLOCK_ROWS)) { blks[1] = mggx::DEFAULT_BLOCK_ROWS; n_blk = 2; }
-    int cores[5] = {-1, 0, 0, 0, 0}, n_core = 1;  // without a dense core and, where it may pay, with one of four sizes
+    int cores[6] = {-1, 0, 0, 0, 0, 0}, n_core = 1;  // without a dense core and, where it may pay, with one of five sizes
     if (o.core_rows > 0) {
         cores[0] = o.core_rows;
     } else if (o.core_rows == 0) {
-        static const int sizes[] = {32 * 1024, 40 * 1024, 48 * 1024, 64 * 1024};
+        static const int sizes[] = {32 * 1024, 40 * 1024, 48 * 1024, 64 * 1024, 80 * 1024};
         for (int c : sizes)
             if (mggx::core_eligible(*g, dim, o.in_dtype, c)) cores[n_core++] = c;
     }
@@ -1317,8 +1317,8 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
         return r;
     };
     // The grid is measured coarsely (one untimed call, two timed ones back to back); the four fastest settings and the
-    // one the library's rules and cost model pick then meet again over eight calls each, so that a setting cannot win on
-    // one lucky measurement, and the result is never slower than leaving the knobs at 0 by more than the noise.
+    // one the library's rules and cost model pick then meet again, twice over eight calls each, so that a setting cannot
+    // win on one lucky measurement, and the result is never slower than leaving the knobs at 0 by more than the noise.
     constexpr int FINALISTS = 4;
     mggx::Knobs top[FINALISTS + 1];
     float top_ms[FINALISTS + 1];
@@ -1362,12 +1362,18 @@ MGGX_EXPORT int mggx_sag_np_div_tune(float *d_out, const void *d_in_local, const
             ++n_top;
         }
     }
+    // Two passes, the faster one counts: a plan built a moment ago (the rule's core size, if the grid did not hold it) runs
+    // 5 - 10 % slower for its first dozen calls, which the first pass absorbs.
     float best = -1.f;
-    for (int i = 0; i < n_top && !rc; ++i) {
-        float ms = 0.f;
-        rc = measure(top[i], 2, 8, &ms);
-        if (!rc && (best < 0.f || ms < best)) { best = ms; bk = top[i]; }
-    }
+    float final_ms[FINALISTS + 1];
+    for (int pass = 0; pass < 2 && !rc; ++pass)
+        for (int i = 0; i < n_top && !rc; ++i) {
+            float ms = 0.f;
+            rc = measure(top[i], 2, 8, &ms);
+            if (!rc && (pass == 0 || ms < final_ms[i])) final_ms[i] = ms;
+        }
+    for (int i = 0; i < n_top && !rc; ++i)
+        if (best < 0.f || final_ms[i] < best) { best = final_ms[i]; bk = top[i]; }
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     if (rc) return rc;

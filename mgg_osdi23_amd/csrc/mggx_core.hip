@@ -520,7 +520,8 @@ int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int 
         delete p;
         return rc;
     }
-    if (s.cores.size() >= 4)  // these plans are large (about 3 bytes per edge): keep the four most recently used, and any a captured graph holds
+    if (s.cores.size() >= 8)  // these plans are large (about 3 bytes per edge): keep the eight most recently used (the search compares
+                              // up to six core sizes and must not rebuild one between its rounds), and any a captured graph holds
         for (size_t i = 0; i < s.cores.size(); ++i)
             if (!s.cores[i]->pinned) {
                 CorePlan *old = s.cores[i];

@@ -398,7 +398,7 @@ __global__ void __launch_bounds__(256) k_lds_probe(float *__restrict__ sink, int
 }
 
 template <int N4>
-int launch_lds_probe(float *sink, int iters, unsigned seed, hipStream_t stream)
+int launch_lds_probe(float *sink, int blocks, int iters, unsigned seed, hipStream_t stream)
 {
     const size_t lds = (size_t)N4 * 257 * sizeof(probe_v4f);
     static bool raised = false;
@@ -406,9 +406,24 @@ int launch_lds_probe(float *sink, int iters, unsigned seed, hipStream_t stream)
         MGGX_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_lds_probe<N4>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         raised = true;
     }
-    k_lds_probe<N4><<<dim3(PROBE_BLOCKS), dim3(256), lds, stream>>>(sink, iters, seed);
+    k_lds_probe<N4><<<dim3((unsigned)blocks), dim3(256), lds, stream>>>(sink, iters, seed);
     MGGX_LAUNCH_CHECK("k_lds_probe");
     return MGGX_OK;
+}
+
+// Workgroups of the LDS yardstick: as many as are resident at once (160 KB of LDS and 8 workgroups of 4 wavefronts per
+// CU), so the launch is one full wave of workgroups and no second, partly filled one dilutes the rate.
+int lds_probe_blocks(size_t lds_bytes)
+{
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return PROBE_BLOCKS;
+        cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    }
+    const long long fit = std::min<long long>(8, (160 * 1024) / (long long)lds_bytes);
+    return (int)std::min<long long>(PROBE_BLOCKS, std::max<long long>(1, fit) * cus);
 }
 
 }  // namespace
@@ -417,12 +432,13 @@ MGGX_EXPORT int mggx_lds_probe(float *d_sink, size_t row_bytes, int64_t n_reads,
 {
     if (!d_sink || row_bytes < 16 || row_bytes > 256 || (row_bytes % 16) || n_reads < 1)
         return fail(MGGX_EINVAL, "lds_probe: NULL sink, or rows not 16..256 bytes in 16-byte pieces");
-    const long long per_iter = (long long)PROBE_BLOCKS * 256 * 4;
+    const int blocks = lds_probe_blocks(row_bytes / 16 * 257 * sizeof(probe_v4f));
+    const long long per_iter = (long long)blocks * 256 * 4;
     const long long iters = (n_reads + per_iter - 1) / per_iter;
     if (iters > 0x7fffffffLL) return fail(MGGX_ELIMIT, "lds_probe: too many reads");
     int rc;
     switch ((int)(row_bytes / 16)) {
-#define MGGX_CASE(N) case N: rc = launch_lds_probe<N>(d_sink, (int)iters, seed, state().stream); break;
+#define MGGX_CASE(N) case N: rc = launch_lds_probe<N>(d_sink, blocks, (int)iters, seed, state().stream); break;
         MGGX_CASE(1) MGGX_CASE(2) MGGX_CASE(3) MGGX_CASE(4) MGGX_CASE(5) MGGX_CASE(6) MGGX_CASE(7) MGGX_CASE(8)
         MGGX_CASE(9) MGGX_CASE(10) MGGX_CASE(11) MGGX_CASE(12) MGGX_CASE(13) MGGX_CASE(14) MGGX_CASE(15) MGGX_CASE(16)
 #undef MGGX_CASE

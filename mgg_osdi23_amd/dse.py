@@ -111,7 +111,7 @@ def sweep_core(w, args):
     print("everything by rule: %.4f ms   [%s]" % (rule, host.last_agg_kernel()))
     print("\ncore rows | ms (best) | wpb dist | edges in the core | list entries with padding | edges left to the gather kernel")
     best = (1e30, None)
-    for K in (-1, 8192, 16384, 24576, 32768, 40960, 49152, 57344, 65536, 81920, 98304):
+    for K in (-1, 8192, 16384, 24576, 32768, 36864, 40960, 49152, 57344, 61440, 65536, 73728, 81920, 98304):
         if K > w["rows"] // 2:
             continue
         sz = [0] * 5
