@@ -199,13 +199,15 @@ constexpr int BUILD_WAVES = 4;  // rows per workgroup of the two passes below (o
 // 16-bit count per core row and tile), and how many neighbors every row keeps in the remaining CSR.  flag |= 1 on a
 // neighbor id outside [lb, lb + rows) or a list longer than 65534.
 __global__ void __launch_bounds__(BUILD_WAVES * 64) k_core_count(const int *__restrict__ ptr, const int *__restrict__ col,
-                                                                 const int *__restrict__ rank, int rows, int lb, int ntiles, int tc,
-                                                                 unsigned short *__restrict__ cnt, int *__restrict__ keep, int *__restrict__ flag)
+                                                                 const int *__restrict__ rank, const int *__restrict__ sorted, int rows, int lb,
+                                                                 int ntiles, int tc, unsigned short *__restrict__ cnt, int *__restrict__ keep,
+                                                                 int *__restrict__ flag)
 {
     extern __shared__ int hist_all[];  // [BUILD_WAVES][ntiles]
     const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
     int *hist = hist_all + (size_t)wave * ntiles;
-    for (long long v = (long long)blockIdx.x * BUILD_WAVES + wave; v < rows; v += (long long)gridDim.x * BUILD_WAVES) {
+    for (long long at = (long long)blockIdx.x * BUILD_WAVES + wave; at < rows; at += (long long)gridDim.x * BUILD_WAVES) {
+        const int v = sorted[at];  // rows in rank order: the longest first
         const int i = rank[v];
         const int beg = ptr[v], end = ptr[v + 1];
         if (i >= 0)
@@ -262,9 +264,10 @@ __global__ void __launch_bounds__(256) k_core_group_work(const int *__restrict__
 // Inside a group of 64 every lane finds the lanes with the same tile by one ballot per bit of the tile number; the counts
 // so far per tile and the row's block offsets sit in LDS, and the next group's ids and ranks are fetched ahead.
 __global__ void __launch_bounds__(BUILD_WAVES * 64) k_core_fill(const int *__restrict__ ptr, const int *__restrict__ col,
-                                                                const int *__restrict__ rank, int rows, int lb, int ntiles, int tc,
-                                                                const int *__restrict__ blk_off, const int *__restrict__ rem_ptr,
-                                                                unsigned short *__restrict__ idx, int *__restrict__ rem_col)
+                                                                const int *__restrict__ rank, const int *__restrict__ sorted, int rows, int lb,
+                                                                int ntiles, int tc, const int *__restrict__ blk_off,
+                                                                const int *__restrict__ rem_ptr, unsigned short *__restrict__ idx,
+                                                                int *__restrict__ rem_col)
 {
     extern __shared__ int fill_lds[];  // [BUILD_WAVES][2][ntiles]: entries already in each tile's list; the row's block offsets
     const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
@@ -273,7 +276,11 @@ __global__ void __launch_bounds__(BUILD_WAVES * 64) k_core_fill(const int *__res
     const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
     int tile_bits = 0;
     while ((1 << tile_bits) < ntiles) ++tile_bits;
-    for (long long v = (long long)blockIdx.x * BUILD_WAVES + wave; v < rows; v += (long long)gridDim.x * BUILD_WAVES) {
+    // Rows in rank order: the 64 rows of a slice are then filled by neighbouring wavefronts at about the same time, and
+    // their 8-byte pieces of the same 512-byte list chunks meet in the L2 instead of each going to memory as a partial
+    // line; the longest rows also start first.
+    for (long long at = (long long)blockIdx.x * BUILD_WAVES + wave; at < rows; at += (long long)gridDim.x * BUILD_WAVES) {
+        const int v = sorted[at];
         const int i = rank[v];
         const int beg = ptr[v], end = ptr[v + 1];
         int w = rem_ptr[v];
@@ -445,7 +452,7 @@ static int core_plan_build_device(CorePlan *p, int tc)
     k_core_rank<<<row_blocks, 256, 0, s.stream>>>(sorted, rows, core, p->d_order, p->d_rank);
     const unsigned wave_blocks = (unsigned)std::min<long long>(((long long)rows + BUILD_WAVES - 1) / BUILD_WAVES, 256 * 64);
     const size_t lds = (size_t)BUILD_WAVES * ntiles * sizeof(int);
-    k_core_count<<<wave_blocks, BUILD_WAVES * 64, lds, s.stream>>>(p->d_ptr_l, p->d_col_l, p->d_rank, rows, lb, ntiles, tc, cnt, keep, flag);
+    k_core_count<<<wave_blocks, BUILD_WAVES * 64, lds, s.stream>>>(p->d_ptr_l, p->d_col_l, p->d_rank, sorted, rows, lb, ntiles, tc, cnt, keep, flag);
     MGGX_LAUNCH_CHECK("k_core_count");
     long long rem_nnz = 0, total_chunks = 0;
     rc = exclusive_scan_i32(keep, p->d_rem_ptr, rows, &rem_nnz);
@@ -467,7 +474,7 @@ static int core_plan_build_device(CorePlan *p, int tc)
     const size_t idx_elems = std::max<size_t>((size_t)total_chunks * 256, 256);
     if ((rc = device_array(&p->d_idx, idx_elems)) || (rc = device_array(&p->d_rem_col, (size_t)rem_nnz))) return rc;
     MGGX_HIP(hipMemsetAsync(p->d_idx, 0xFF, idx_elems * sizeof(unsigned short), s.stream));
-    k_core_fill<<<wave_blocks, BUILD_WAVES * 64, 2 * lds, s.stream>>>(p->d_ptr_l, p->d_col_l, p->d_rank, rows, lb, ntiles, tc, blk, p->d_rem_ptr, p->d_idx,
+    k_core_fill<<<wave_blocks, BUILD_WAVES * 64, 2 * lds, s.stream>>>(p->d_ptr_l, p->d_col_l, p->d_rank, sorted, rows, lb, ntiles, tc, blk, p->d_rem_ptr, p->d_idx,
                                                                   p->d_rem_col);
     MGGX_LAUNCH_CHECK("k_core_fill");
     MGGX_HIP(hipStreamSynchronize(s.stream));
