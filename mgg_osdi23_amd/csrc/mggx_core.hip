@@ -595,10 +595,15 @@ static int core_cut(CorePlan *p, int n4, const CorePlan::Cut **out)
         (void)hipFree(c.d_wgs);
         return rc;
     }
+    hipError_t e = hipMemcpy(c.d_wgs, launch.data(), launch.size() * sizeof(int4), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(c.d_wg_base, wg_base.data(), wg_base.size() * sizeof(int), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {  // a cut that is kept must be complete: later calls find it by its target alone
+        (void)hipFree(c.d_wgs);
+        (void)hipFree(c.d_wg_base);
+        return fail(MGGX_EHIP, "core: uploading the workgroup table: %s", hipGetErrorString(e));
+    }
     p->cuts.reserve(4);  // pointers into the vector are handed out: two targets exist
     p->cuts.push_back(c);
-    MGGX_HIP(hipMemcpy(c.d_wgs, launch.data(), launch.size() * sizeof(int4), hipMemcpyHostToDevice));
-    MGGX_HIP(hipMemcpy(c.d_wg_base, wg_base.data(), wg_base.size() * sizeof(int), hipMemcpyHostToDevice));
     p->bytes += launch.size() * sizeof(int4) + wg_base.size() * sizeof(int);
     *out = &p->cuts.back();
     return MGGX_OK;
