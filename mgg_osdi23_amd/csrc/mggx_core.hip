@@ -44,27 +44,20 @@ __global__ void __launch_bounds__(256) k_core_stage(v4f *__restrict__ tab, const
     tab[(size_t)s * tab_stride(core) + i] = v;
 }
 
-// One workgroup = CORE_WAVES slices (a row group) x a run of column tiles; lane = core row.  Row groups and tiles are both
-// sorted by degree, so the work of a (row group, tile) cell spans two orders of magnitude: the plan cuts every row
-// group's tiles into runs of about equal list length (wgs[i] = {row group, first tile, end tile, slot}), so all
-// workgroups take about the same time and the launch has no tail of a few heavy ones.
-// partial[(slot * CORE_WAVES * 64 + row in the group) * N4 + s]
-template <int N4>
-__global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *__restrict__ blk_off, const unsigned short *__restrict__ idx,
-                                                               const v4f *__restrict__ tab, v4f *__restrict__ partial,
-                                                               const int4 *__restrict__ wgs, int core, int ntiles, const Gate gate)
+// The body for the 16-byte pieces [S0, S0 + NS) of rows of N4 pieces.
+template <int N4, int S0, int NS>
+__device__ __forceinline__ void core_sell_body(const unsigned *__restrict__ blk_off, const unsigned short *__restrict__ idx,
+                                               const v4f *__restrict__ tab, v4f *__restrict__ partial, const int4 wg, int core, int ntiles,
+                                               v4f *tile)
 {
-    constexpr int TC = CORE_TC, TP = TC + 1;  // column TC of every slice row is zero: what padding entries read
-    extern __shared__ v4f tile[];             // [N4][TP]
-    if (gate_closed(gate)) return;
+    constexpr int TC = CORE_TC, TP = TC + 1;  // column TC of every slice row is zero: what padding entries read; tile[NS][TP]
     const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
-    const int4 wg = wgs[blockIdx.x];
     const int g = wg.x * CORE_WAVES + wave;
     const int t0 = wg.y, t1 = wg.z;
-    v4f acc[N4];
+    v4f acc[NS];
 #pragma unroll
-    for (int s = 0; s < N4; ++s) acc[s] = (v4f){0.f, 0.f, 0.f, 0.f};
-    if ((int)threadIdx.x < N4) tile[(int)threadIdx.x * TP + TC] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < NS; ++s) acc[s] = (v4f){0.f, 0.f, 0.f, 0.f};
+    if ((int)threadIdx.x < NS) tile[(int)threadIdx.x * TP + TC] = (v4f){0.f, 0.f, 0.f, 0.f};
     const us4 *p = reinterpret_cast<const us4 *>(idx) + lane;
     unsigned pos = blk_off[(size_t)g * ntiles + t0];
     const unsigned end_run = blk_off[(size_t)g * ntiles + t1];
@@ -72,9 +65,9 @@ __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *_
     us4 cur = pos < end_run ? p[(size_t)pos * 64] : pad;  // the lists of a slice's tiles follow one another: read one chunk ahead
     for (int t = t0; t < t1; ++t) {
         __syncthreads();
-        for (int i = (int)threadIdx.x; i < N4 * TC; i += CORE_WAVES * 64) {
+        for (int i = (int)threadIdx.x; i < NS * TC; i += CORE_WAVES * 64) {
             const int s = i / TC, c = i % TC;
-            tile[s * TP + c] = tab[(size_t)s * tab_stride(core) + (size_t)t * TC + c];
+            tile[s * TP + c] = tab[(size_t)(S0 + s) * tab_stride(core) + (size_t)t * TC + c];
         }
         const unsigned b1 = blk_off[(size_t)g * ntiles + t + 1];
         __syncthreads();
@@ -86,13 +79,13 @@ __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *_
                 const v4f *q = tile + (c < TC ? c : TC);
                 // at most eight LDS reads in flight per entry: wide rows otherwise cost a wavefront a hundred registers, and
                 // this kernel shares each SIMD's register file with the aggregation running beside it
-                constexpr int H = N4 > 8 ? (N4 + 1) / 2 : N4;
+                constexpr int H = NS > 8 ? (NS + 1) / 2 : NS;
 #pragma unroll
                 for (int s = 0; s < H; ++s) acc[s] += q[s * TP];
-                if constexpr (H < N4) {
+                if constexpr (H < NS) {
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int s = H; s < N4; ++s) acc[s] += q[s * TP];
+                    for (int s = H; s < NS; ++s) acc[s] += q[s * TP];
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -102,7 +95,30 @@ __global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *_
     }
     const size_t r = (size_t)wg.w * (CORE_WAVES * 64) + (size_t)(wave * 64 + lane);
 #pragma unroll
-    for (int s = 0; s < N4; ++s) partial[r * N4 + s] = acc[s];
+    for (int s = 0; s < NS; ++s) partial[r * N4 + S0 + s] = acc[s];
+}
+
+// One workgroup = CORE_WAVES slices (a row group) x a run of column tiles [x all pieces of the rows, or one half of
+// them when SPLIT: blockIdx.y]; lane = core row.  Row groups and tiles are both sorted by degree, so the work of a
+// (row group, tile) cell spans two orders of magnitude: the plan cuts every row group's tiles into runs of about equal
+// list length (wgs[i] = {row group, first tile, end tile, slot}), so all workgroups take about the same time and the
+// launch has no tail of a few heavy ones.
+// partial[(slot * CORE_WAVES * 64 + row in the group) * N4 + s]
+template <int N4, bool SPLIT>
+__global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *__restrict__ blk_off, const unsigned short *__restrict__ idx,
+                                                               const v4f *__restrict__ tab, v4f *__restrict__ partial,
+                                                               const int4 *__restrict__ wgs, int core, int ntiles, const Gate gate)
+{
+    extern __shared__ v4f tile[];
+    if (gate_closed(gate)) return;
+    const int4 wg = wgs[blockIdx.x];
+    if constexpr (!SPLIT) {
+        core_sell_body<N4, 0, N4>(blk_off, idx, tab, partial, wg, core, ntiles, tile);
+    } else {
+        constexpr int A = (N4 + 1) / 2;
+        if (blockIdx.y == 0) core_sell_body<N4, 0, A>(blk_off, idx, tab, partial, wg, core, ntiles, tile);
+        else core_sell_body<N4, A, N4 - A>(blk_off, idx, tab, partial, wg, core, ntiles, tile);
+    }
 }
 
 // Adds the core block's sums to output rows that already hold the rest of the aggregation:
@@ -330,16 +346,25 @@ __global__ void __launch_bounds__(BUILD_WAVES * 64) k_core_fill(const int *__res
     }
 }
 
+// Rows of more than 192 bytes are summed in two halves by two workgroups (blockIdx.y): half the accumulators per lane
+// (81 instead of 119 registers at 256 bytes), at the price of walking the index lists twice.  Three such workgroups per
+// CU, which a request of a little over a quarter of the LDS enforces, leave the aggregation beside them the room it had
+// (measured on the 2.45 M-node graph at width 64: 3.01 ms whole, 2.92 ms in halves with three per CU; 3.21 with four,
+// 2.97 with two; at width 44 halves gain nothing: 1.42 against 1.40 ms).
 template <int N4>
 int launch_sell(const CorePlan *p, const CorePlan::Cut &cut, const v4f *tab, v4f *partial, const Gate &gate, hipStream_t stream)
 {
-    const size_t lds = (size_t)N4 * (CORE_TC + 1) * sizeof(v4f);
+    constexpr bool SPLIT = N4 > 12;
+    constexpr int NS = SPLIT ? (N4 + 1) / 2 : N4;
+    size_t lds = (size_t)NS * (CORE_TC + 1) * sizeof(v4f);
+    if (SPLIT) lds = std::max<size_t>(lds, (160u << 10) / 4 + 256);
     static bool raised = false;  // per instantiation
     if (lds > 48 * 1024 && !raised) {
-        MGGX_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_core_sell<N4>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        MGGX_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_core_sell<N4, SPLIT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         raised = true;
     }
-    k_core_sell<N4><<<dim3((unsigned)cut.nwg), dim3(CORE_WAVES * 64), lds, stream>>>(p->d_blk_off, p->d_idx, tab, partial, cut.d_wgs, p->core, p->ntiles, gate);
+    k_core_sell<N4, SPLIT><<<dim3((unsigned)cut.nwg, SPLIT ? 2u : 1u), dim3(CORE_WAVES * 64), lds, stream>>>(p->d_blk_off, p->d_idx, tab, partial, cut.d_wgs,
+                                                                                                          p->core, p->ntiles, gate);
     MGGX_LAUNCH_CHECK("k_core_sell");
     return MGGX_OK;
 }
