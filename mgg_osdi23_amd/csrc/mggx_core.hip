@@ -748,14 +748,14 @@ int core_partial_rows(CorePlan *p, int dim, const float4 **partial_out, const in
 // constants fitted to sweeps of the core size on the 233 K-node width-16 / width-44 and the 2.45 M-node width-64
 // graphs (ALPHA 1.42 ps per padded 16-byte piece; BETA 9 ps per gathered row plus as much per 64-byte sector of it while
 // the table fits the 256 MB last-level cache, 3.2 x that beyond).  The staging of the tiles (core^2 / 65536 tiles of
-// 256 x ceil(dim/4) x 16 bytes per row group) is not in the model; it shows beyond 80,000 rows, where the model stops.
+// 256 x ceil(dim/4) x 16 bytes per row group) is not in the model; it shows beyond 100,000 rows, where the model stops.
 namespace mggx {
 namespace {
 
 constexpr int PROFILE_SLICES = 2048;  // 131072 ranks
 constexpr double ALPHA_PS = 1.42, BETA_PS = 9.0, HBM_FACTOR = 3.2;
 constexpr unsigned long long LAST_LEVEL_CACHE_BYTES = 256ull << 20;
-constexpr int MODEL_STEP = 4096, MODEL_MAX_CORE = 81920;
+constexpr int MODEL_STEP = 4096, MODEL_MAX_CORE = 98304;
 
 __global__ void __launch_bounds__(256) k_degrees(const int *__restrict__ ptr, int rows, int *__restrict__ deg)
 {
@@ -852,7 +852,8 @@ int predict_core_rows(GraphInfo &g, int dim, unsigned long long table_bytes, int
     if (rc) return rc;
     const int n4 = (dim + 3) / 4;
     const int sectors = (dim * 4 + 63) / 64;
-    const double theta = ALPHA_PS * n4 / (BETA_PS * (1 + sectors) * (beyond_cache ? HBM_FACTOR : 1.0));
+    // rows summed in two halves (more than 12 pieces) leave the gather kernel beside them more room: measured 0.75 of the cost
+    const double theta = ALPHA_PS * (n4 > 12 ? 0.75 : 1.0) * n4 / (BETA_PS * (1 + sectors) * (beyond_cache ? HBM_FACTOR : 1.0));
     const double nnz = (double)g.nnz_l;
     const int max_core = std::min({MODEL_MAX_CORE, g.rows / 2 / MODEL_STEP * MODEL_STEP, (int)g.slice_deg.size() * 64 / MODEL_STEP * MODEL_STEP});
     // useful and padded entries of the block (slices [s0, s1) x tiles [t0, t1))
