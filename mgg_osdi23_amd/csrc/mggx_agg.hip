@@ -930,12 +930,13 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     // 0 = let the library choose (from sweeps of wpb x dist on the benchmark graphs; each choice within 5 % of the best
     // setting of its sweep).  Few slots per wavefront (wide rows): 8 wavefronts and 16 rounds, so a workgroup still covers
     // a few thousand neighbors -- 4 wavefronts where the kernel shares the chip with the dense core's 4-wavefront
-    // workgroups (column-blocked plans, and whatever a core leaves), and then 4 rounds in row-major order.  Many slots
+    // workgroups (column-blocked plans, and whatever a core leaves), and then 4 rounds in row-major order; 4 wavefronts
+    // also where rows are short (under 3 partitions per row: -3 % on the 13.9 M-row bf16 share).  Many slots
     // (narrow rows): 4 wavefronts, 4 rounds; 8 rounds where a column-blocked plan is left with short rows (under 8
     // partitions per row and block).
     const double per_row = (double)plan->num_parts / (double)(plan->rows > 0 ? plan->rows : 1);
     const bool beside_core = cm != nullptr;
-    if (wpb == 0) wpb = (blocked || beside_core || slots > 4) ? 4 : 8;
+    if (wpb == 0) wpb = (blocked || beside_core || slots > 4 || per_row < 3.0) ? 4 : 8;
     if (dist == 0) {
         if (slots <= 4) dist = (beside_core && !blocked) ? 4 : 16;
         else if (blocked && per_row < 8.0) dist = 8;
