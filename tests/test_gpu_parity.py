@@ -293,9 +293,10 @@ def test_dense_core_from_lds(gpu, rmat_graph, dim, core_rows, flags):
 
 
 @pytest.mark.parametrize("dim,core_rows", [(16, 12800), (44, 13824)])
-def test_dense_core_with_tile_segments_of_unequal_length(gpu, dim, core_rows):
-    """A core whose number of 256-column tiles (50, 54) is not a multiple of the number of tile segments its workgroups
-    split into (41, 38): segments of one and of two tiles side by side, every tile summed exactly once."""
+def test_dense_core_with_tile_runs_of_unequal_length(gpu, dim, core_rows):
+    """A core of 50 / 54 row groups and as many 256-column tiles, large enough for its workgroups to be cut into runs of
+    tiles of unequal length (one tile for the heaviest row groups, many for the lightest): every (row group, tile) cell
+    summed exactly once, at both row-width classes of the cut."""
     import torch
     from mgg_osdi23_amd import host
     V = 30000
