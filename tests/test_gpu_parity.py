@@ -236,11 +236,12 @@ def test_column_blocked_order(gpu, rmat_graph, dim, block_rows, flags):
 
 
 @pytest.mark.parametrize("dim,core_rows,flags", [(16, 1024, "plain"), (44, 512, "scale"), (41, 2048, "gin"), (8, 1500, "acc_relu"),
-                                                 (64, 1024, "plain"), (5, 512, "scale")])
+                                                 (64, 1024, "plain"), (5, 512, "scale"), (52, 1024, "scale"), (57, 512, "gin")])
 def test_dense_core_from_lds(gpu, rmat_graph, dim, core_rows, flags):
     """The dense-core path (core x core block summed from LDS tiles, the rest of the CSR on top): same sums as the
     ordinary path and the oracle with every epilogue, with padded row strides, and together with the column-blocked
-    order of what is left."""
+    order of what is left.  Widths 52, 57 and 64 are rows of 13, 15 and 16 pieces, which the LDS kernel sums in two
+    halves (7 + 6, 8 + 7, 8 + 8)."""
     import torch
     V, ptr, col = rmat_graph
     x = gpu.fill_normal((V, dim), seed=191)
