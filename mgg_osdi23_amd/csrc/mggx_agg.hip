@@ -322,6 +322,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     constexpr int CH = LPR > 16 ? LPR : 16;  // neighbor ids fetched per slot per chunk
     constexpr int IPL = CH / LPR;            // ids fetched per lane
     constexpr int BATCH = MGGX_BATCH;        // gathers issued back to back
+    static_assert(CH % BATCH == 0, "the gathers of a chunk of ids are issued in whole batches");
     // With 16 slots a wavefront reads its ids 1 KiB at a time and its descriptors 256 B at a time -- whole cache lines
     // that nobody reads again: those loads carry the streaming hint, which leaves the caches to the feature rows
     // (-5 % at width 16).  With fewer slots adjacent wavefronts share those lines and the hint costs 1-3 %.
