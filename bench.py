@@ -985,7 +985,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=20,
+                    help="untimed steps before the timed ones (default 20: a dense-core plan built a moment ago runs up to 10 %% slower "
+                         "for its first twenty calls)")
     ap.add_argument("--workload", default="gcn2", choices=["gcn2", "share", "gin", "big", "copy", "gather", "vendor"])
     ap.add_argument("--ps", type=int, default=16, help="partSize; 0 = let the library choose (the search then tries 16 and 32)")
     ap.add_argument("--col-block-rows", type=int, default=0, help="column-blocked partition order: 0 = library decides, -1 = off, "
