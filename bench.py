@@ -41,6 +41,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+COLD_COPIES = 6           # disjoint copies of the share's working set the cold-cache leg rotates over
 
 
 def log(*a):
@@ -453,9 +454,14 @@ def bench_gcn2(args, torch, host):
     share = share_record(args, torch, host, with_cpu=not args.no_cpu)
     extra["share"] = share
 
+    checks = list(share.pop("_checks"))
+    if not args.small and not args.no_extra:
+        more, more_checks = other_configs(args, torch, host)
+        extra.update(more)
+        checks += more_checks
+
     cpu = None
     parity = None
-    checks = list(share.pop("_checks"))
     if not args.no_cpu:
         from oracle import orc
         th = orc.max_threads()
@@ -494,6 +500,44 @@ def bench_gcn2(args, torch, host):
     }
     fail_on_parity(res, checks)
     return res
+
+
+def other_configs(args, torch, host):
+    """configs[4] (large bf16 share: aggregation + 128x128 update) and configs[2] (5-layer GIN forward) at their full sizes, in
+    the same process as the default run, knobs by the library's rules, fewer timed steps; each with its parity figure from the
+    same run (the large share on sampled rows as a sub-problem of their own, the GIN forward whole).  -> ({"big": ..., "gin":
+    ...}, parity checks)"""
+    import copy
+    out, checks = {}, []
+    a = copy.copy(args)
+    a.no_tune, a.no_compact, a.big_scale = True, True, 0
+    a.steps, a.warmup = max(3, min(args.steps, 10)), 3
+    host.release_cached()
+    t0 = time.perf_counter()
+    r = bench_big(a, torch, host)
+    rf = r["roofline"]
+    out["big"] = {"workload": r["config"]["workload"], "ms": r["detail"]["stage_ms"]["agg"], "update_ms": r["detail"]["stage_ms"]["update"],
+                  "algorithmic_bytes": rf["algorithmic_bytes"], "achieved": rf["achieved"], "frac": rf["frac"], "traffic": rf.get("traffic"),
+                  "traffic_measured_at": rf.get("traffic_measured_at"), "update_gbps": r["detail"]["update_gbps"],
+                  "update_tflops": r["detail"]["update_tflops"], "steps": a.steps, "parity": r["parity"], "cpu_baseline": r["cpu_baseline"],
+                  "leg_wall_s": round(time.perf_counter() - t0, 1)}
+    checks += r["_checks"]
+    host.release_cached()
+    torch.cuda.empty_cache()
+    a.warmup = 10
+    t0 = time.perf_counter()
+    r = bench_gin(a, torch, host)
+    rf = r["roofline"]
+    agg_ms = rf["avg_launch_ms"]
+    out["gin"] = {"workload": r["config"]["workload"], "fwd_ms": r["value"], "agg_ms": agg_ms, "mlp_total_ms": r["detail"]["mlp_total_ms"],
+                  "algorithmic_bytes": rf["algorithmic_bytes"], "algorithmic_gbps_over_hbm_peak": rf.get("algorithmic_gbps_over_hbm_peak"),
+                  "traffic": rf.get("traffic"), "traffic_measured_at": rf.get("traffic_measured_at"),
+                  "frac_traffic": round(rf["traffic"] / (agg_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4) if rf.get("traffic") else None,
+                  "steps": a.steps, "parity": r["parity"], "cpu_baseline": r["cpu_baseline"], "leg_wall_s": round(time.perf_counter() - t0, 1)}
+    checks += r["_checks"]
+    host.release_cached()
+    torch.cuda.empty_cache()
+    return out, checks
 
 
 def gcn2_headline_only(args, torch, host, forward_stages, names):
@@ -539,6 +583,52 @@ def share_record(args, torch, host, with_cpu):
     lb, ub, dim, npp, R, nnz = sh["lb"], sh["ub"], sh["dim"], sh["npp"], sh["R"], sh["nnz"]
     nbytes = agg_bytes(nnz, R, dim, ptr_arrays=2)
 
+    def cold_leg(kn, col_r, table, want):
+        """The same call with nothing of it left in the caches: each launch goes to the next of COLD_COPIES disjoint
+        copies of everything the call touches (row pointers, column ids, both feature tables, the output, and -- a plan
+        is keyed by its CSR's addresses -- its own descriptors and row offsets), so between two uses of a copy the others
+        move several times the 256 MB of the last-level cache.  HIP events around each launch only; the mean over all."""
+        n = COLD_COPIES
+        sets = []
+        for _ in range(n):
+            c = [t.clone() for t in (d[0], d[1], d[2], col_r, d_xl, table)]
+            c.append(torch.empty_like(d_out))
+            sets.append(c)
+        calls = [lambda c=c: host.mgg_SAG_np_div(c[6], c[4], c[0], c[1], c[2], c[3], lb, ub, dim, npp, 0, kn.ps, kn.wpb, kn.dist,
+                                                 input_remote=c[5], col_block_rows=kn.blk, core_rows=kn.core) for c in sets]
+        mark = host.cache_stats()["plan_bytes"]
+        calls[0]()
+        plan_bytes = host.cache_stats()["plan_bytes"] - mark
+        for fn in calls:   # plans built, code loaded
+            fn()
+            fn()
+        torch.cuda.synchronize()
+        ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)] for _ in range(args.steps)]
+        for step in ev:
+            for (e0, e1), fn in zip(step, calls):
+                e0.record()
+                fn()
+                e1.record()
+        torch.cuda.synchronize()
+        ms = [e0.elapsed_time(e1) for step in ev for e0, e1 in step]
+        slowest = sorted(range(len(ms)), key=lambda i: -ms[i])[:4]
+        same = all(bool((c[6] == sets[0][6]).all()) for c in sets) and bool(np.array_equal(sets[0][6].cpu().numpy(), want))
+        per_copy = sum(t.numel() * t.element_size() for t in sets[0]) + plan_bytes
+        # the median launch: with events around single launches a stall of the launching thread (the stream runs empty
+        # between the first event and the kernel) lands inside one interval; the mean is given beside it
+        mean, med = float(np.mean(ms)), float(np.median(ms))
+        out = {"copies": n, "launches": len(ms), "avg_launch_ms": round(mean, 4), "median_launch_ms": round(med, 4),
+               "achieved": round(nbytes / (med * 1e-3) / 1e9, 1), "frac": round(nbytes / (med * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+               "frac_by_mean_launch": round(nbytes / (mean * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+               "bytes_allocated_per_copy": int(per_copy), "bytes_of_other_copies_between_two_uses": int(per_copy * (n - 1)),
+               "results_identical_to_the_warm_call": same,
+               "slowest_launches": [{"step": i // n, "copy": i % n, "ms": round(ms[i], 4)} for i in slowest]}
+        for c in sets:
+            for t in c[:4]:
+                host.forget(t)
+        del sets, calls
+        return out
+
     def measure(col_r, table, key):
         search = lambda ps, blk, core: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], col_r, lb, ub, dim, npp, ps, input_remote=table,
                                                         col_block_rows=blk, core_rows=core)
@@ -559,6 +649,8 @@ def share_record(args, torch, host, with_cpu):
         call()
         torch.cuda.synchronize()
         result = d_out.cpu().numpy()
+        rec["cold"] = cold_leg(kn, col_r, table, result)
+        rec["frac_cold"] = rec["cold"]["frac"]
         if not args.tune and not args.no_search:
             t0 = time.perf_counter()
             ks = Knobs(args, search)
@@ -605,12 +697,18 @@ def share_record(args, torch, host, with_cpu):
         cpu = {"value": round(cpu_s * 1e3, 1), "unit": "ms", "cores": th, "kind": "port", "sample": "the same aggregation call, whole share (fp32, OpenMP over rows)",
                "max_abs_diff_vs_gpu": float(np.abs(out_glob - ref).max())}
         checks = [("share, global-id table", e1, 1e-5), ("share, compact staging", e2, 1e-5)]
+    for rec_, name in ((glob, "global-id table"), (comp, "compact staging")):
+        checks.append(("share, %s: cold-cache copies differ from the warm call" % name, 0.0 if rec_["cold"]["results_identical_to_the_warm_call"] else 1.0, 0.5))
     workload = ("configs[3]: rank-0 1/8 share of RMAT V=%d (ids scrambled), rows=%d nnz=%d (local %d, remote %d), fp32 dim %d, remote rows "
                 "pre-staged in a second HBM table" % (sh["V"], R, nnz, len(sh["lc"]), len(sh["rc"]), dim))
     roofline = {"bound": "hbm", "kernel": "%s on %s, remote rows staged compactly (%s)" % (comp["kernel"], "configs[3]", comp["knobs"]),
                 "achieved": comp["achieved"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": comp["frac"], "traffic": comp.get("traffic"),
                 "algorithmic_bytes": nbytes, "avg_launch_ms": comp["avg_launch_ms"],
-                "frac_global_id_table": glob["frac"], "achieved_global_id_table": glob["achieved"], "traffic_global_id_table": glob.get("traffic")}
+                "frac_cold": comp["frac_cold"], "median_launch_ms_cold": comp["cold"]["median_launch_ms"], "avg_launch_ms_cold": comp["cold"]["avg_launch_ms"],
+                "cold_is": "every launch on the next of %d disjoint copies of all arrays of the call (%.0f MB of other copies between two uses of "
+                           "one; the last-level cache holds 256 MB)" % (COLD_COPIES, comp["cold"]["bytes_of_other_copies_between_two_uses"] / 1e6),
+                "frac_global_id_table": glob["frac"], "frac_cold_global_id_table": glob["frac_cold"],
+                "achieved_global_id_table": glob["achieved"], "traffic_global_id_table": glob.get("traffic")}
     if comp.get("traffic_measured_at"):
         roofline["traffic_measured_at"] = comp["traffic_measured_at"]
     return {"workload": workload, "ms": comp["avg_launch_ms"], "algorithmic_bytes": nbytes, "frac": comp["frac"], "traffic": comp.get("traffic"),
@@ -764,6 +862,8 @@ def bench_gin(args, torch, host):
                                  load_traffic("gin_agg", args, kn.blk, kn.core)),
         "cpu_baseline": cpu, "parity": parity,
         "detail": {"stage_ms": {k: round(v, 4) for k, v in avg.items()}, "mlp_total_ms": round(mlp_ms, 4)},
+        "_checks": [("configs[2] logits, relative", parity["logits_max_rel_err"], 1e-5),
+                    ("configs[2] softmax", parity["softmax_max_abs_err"], 1e-5)] if parity else [],
     }
 
 
@@ -844,7 +944,7 @@ def bench_big(args, torch, host):
                "sample": "%d sampled rows (%d neighbors) of the same share, double accumulation" % (len(rows), edges),
                "gpu_same_unit": round(nnz / (avg["agg"] * 1e-3) / 1e6, 1)}
         log("parity %s; cpu %s" % (parity, cpu))
-    compact = compact_variant(args, torch, host, d_out, d_xl, d_xr, d, rc, lb, ub, dim, npp, nbytes, 2)
+    compact = None if getattr(args, "no_compact", False) else compact_variant(args, torch, host, d_out, d_xl, d_xr, d, rc, lb, ub, dim, npp, nbytes, 2)
     return {
         "metric": "np_aggregation_plus_update_ms", "value": round(wall_ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": False, "scaling": "weak",
@@ -857,6 +957,7 @@ def bench_big(args, torch, host):
         "detail": {"stage_ms": {k2: round(v, 4) for k2, v in avg.items()},
                    "update_tflops": round(gflop / avg["update"], 2), "update_gbps": round(gemm_bytes / (avg["update"] * 1e-3) / 1e9, 1),
                    "compact_remote_staging": compact},
+        "_checks": [("configs[4] sampled rows", parity["agg_max_err_over_abs_sum"], 1e-5)] if parity else [],
     }
 
 
@@ -1000,6 +1101,7 @@ def main():
     ap.add_argument("--tune", action="store_true", help="time the setting the library's search measures fastest instead of the one its rules and "
                          "cost model choose (gcn2 and share otherwise run the search afterwards, for comparison)")
     ap.add_argument("--no-search", action="store_true", help="gcn2 / share: skip the comparison run of the search")
+    ap.add_argument("--no-extra", action="store_true", help="gcn2: skip the legs on configs[4] and configs[2] (large bf16 share, GIN forward)")
     ap.add_argument("--only-headline", action="store_true", help="gcn2: the headline forward only (for profiler runs)")
     ap.add_argument("--no-tune", action="store_true", help="gin / big: use the library's rules instead of its search")
     ap.add_argument("--share-density", type=int, default=1, help="multiplies the number of RMAT draws of --workload share")
@@ -1028,6 +1130,9 @@ def main():
     log("device:", host.device_name())
     res = {"gcn2": bench_gcn2, "share": bench_share, "gin": bench_gin, "big": bench_big, "copy": bench_copy,
            "gather": bench_gather, "vendor": bench_vendor}[args.workload](args, torch, host)
+    checks = res.pop("_checks", None)
+    if checks:
+        fail_on_parity(res, checks)
     print(json.dumps(res), flush=True)
 
 

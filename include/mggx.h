@@ -311,8 +311,14 @@ int mggx_sag_parts(float *d_out, const float *d_in, const int *d_row_ptr, const 
  * on the first call there).  A call whose 16 bytes per partition + 4 bytes per row + carry buffer (two partial rows per
  * workgroup) do not fit returns MGGX_ELIMIT.  The call only launches kernels on the library's stream -- no allocation,
  * no memset, no copy to the host, no synchronisation.  Every call on a GPU uses that GPU's one array: calls that may
- * overlap on one GPU (two streams, two host threads) race; issue them on one stream. */
+ * overlap on one GPU (two streams, two host threads) race; issue them on one stream.
+ * Cost: the array is part of the library's code object, so every process that loads the library holds it on every GPU it
+ * touches (64 MiB per process and GPU by default), whether or not this entry point is ever called; a build for many
+ * processes per GPU can shrink it with -DMGGX_STATIC_SCRATCH_BYTES=<bytes> (the limit a call meets is the built library's).
+ * If the array's address cannot be looked up, mggx_init still succeeds and only this entry point returns the error. */
+#ifndef MGGX_STATIC_SCRATCH_BYTES
 #define MGGX_STATIC_SCRATCH_BYTES (64u << 20)
+#endif
 int mggx_sag_parts_static(float *d_out, const float *d_in, const int *d_row_ptr, const int *d_col,
                           const int *d_part_ptr, const int *d_part2node,
                           int lowbound, int num_nodes, int num_parts, int ps, int dim, int wpb, int dist);

@@ -1162,7 +1162,7 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
     if (k.core_rows > 0 && ub - lb >= 1024 && g.nnz_r == 0 && g.nnz_l > 0 && d_col_l && o.in_dtype == MGGX_F32 && dim >= 1 && dim <= 64 && d_out &&
         d_in_local) {
         CorePlan *cp = nullptr;
-        rc = core_plan_get(d_ptr_l, d_col_l, ub - lb, lb, k.core_rows, &cp);
+        rc = core_plan_get(d_ptr_l, d_col_l, ub - lb, lb, k.core_rows, g.serial, &cp);
         if (rc) return rc;
         if (!cp->unsuitable) {
             // The core block is bound by the LDS, the rest of the CSR by the caches: they run side by side.  The core's sums
@@ -1212,12 +1212,12 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
         }
     }
     if (k.block_rows > 0 && g.nnz_r == 0 && d_col_l && ub - lb >= 2 * (long long)k.block_rows) {
-        rc = plan_get_blocked(d_ptr_l, d_col_l, ub - lb, lb, k.ps, k.block_rows, &plan);
+        rc = plan_get_blocked(d_ptr_l, d_col_l, ub - lb, lb, k.ps, k.block_rows, g.serial, &plan);
         if (rc) return rc;
         if (plan->unsuitable) plan = nullptr;
     }
     if (!plan) {
-        rc = plan_get(d_ptr_l, d_ptr_r, d_col_r, ub - lb, k.ps, &plan);
+        rc = plan_get(d_ptr_l, d_ptr_r, d_col_r, ub - lb, k.ps, g.serial, &plan);
         if (rc) return rc;
     }
     return run_agg(plan, d_out, d_in_local, d_in_remote, d_col_l, d_col_r, lb, dim, k.wpb, k.dist, o, gate, nullptr, cm);

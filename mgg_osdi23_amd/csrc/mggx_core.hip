@@ -369,18 +369,34 @@ int launch_sell(const CorePlan *p, const CorePlan::Cut &cut, const v4f *tab, v4f
     return MGGX_OK;
 }
 
+// A plan that was used inside a stream capture: a captured graph still holds the addresses of its arrays, so they are
+// retired (freed by mggx_release_cached) instead of freed.
 void core_plan_free_arrays(CorePlan *p)
 {
-    if (p->d_order) (void)hipFree(p->d_order);
-    if (p->d_rank) (void)hipFree(p->d_rank);
-    if (p->d_blk_off) (void)hipFree(p->d_blk_off);
-    if (p->d_idx) (void)hipFree(p->d_idx);
-    if (p->d_rem_ptr) (void)hipFree(p->d_rem_ptr);
-    if (p->d_rem_col) (void)hipFree(p->d_rem_col);
+    const bool keep = p->pinned;
+    size_t left = keep ? p->bytes : 0;  // the plan's bytes, accounted to the first retired block
+    const auto drop = [&](void *q) {
+        if (!q) return;
+        if (keep) {
+            retire_block(q, left);
+            left = 0;
+        } else {
+            (void)hipFree(q);
+        }
+    };
+    drop(p->d_order);
+    drop(p->d_rank);
+    drop(p->d_blk_off);
+    drop(p->d_idx);
+    drop(p->d_rem_ptr);
+    drop(p->d_rem_col);
     for (CorePlan::Cut &c : p->cuts) {
-        if (c.d_wgs) (void)hipFree(c.d_wgs);
-        if (c.d_wg_base) (void)hipFree(c.d_wg_base);
+        drop(c.d_wgs);
+        drop(c.d_wg_base);
     }
+    p->d_order = p->d_rank = p->d_rem_ptr = p->d_rem_col = nullptr;
+    p->d_blk_off = nullptr;
+    p->d_idx = nullptr;
     p->cuts.clear();
 }
 
@@ -520,12 +536,14 @@ static int core_plan_build_device(CorePlan *p, int tc)
     return MGGX_OK;
 }
 
-int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, CorePlan **out)
+int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, int graph_serial, CorePlan **out)
 {
     State &s = state();
     for (size_t i = 0; i < s.cores.size(); ++i) {
         CorePlan *p = s.cores[i];
-        if (p->d_ptr_l == d_ptr_l && p->d_col_l == d_col_l && p->rows == rows && p->lb == lb && p->asked == core) {
+        // a plan belongs to the graph record it was built under (see drop_plans_of_record): it carries its own copy of that
+        // graph's remaining CSR and index lists, and a later record of the same addresses may stand for another graph
+        if (p->d_ptr_l == d_ptr_l && p->d_col_l == d_col_l && p->rows == rows && p->lb == lb && p->asked == core && p->graph_serial == graph_serial) {
             if (i + 1 != s.cores.size()) {  // most recently used last
                 s.cores.erase(s.cores.begin() + (long)i);
                 s.cores.push_back(p);
@@ -546,6 +564,7 @@ int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int 
     p->rows = rows;
     p->lb = lb;
     p->asked = core;
+    p->graph_serial = graph_serial;
     int rc = core_plan_build_device(p, CORE_TC);
     if (rc) {
         core_plan_free_arrays(p);
@@ -892,8 +911,11 @@ MGGX_EXPORT int mggx_core_layout_device(const int *d_ptr, const int *d_col, int 
     int rc = mggx::ensure_init();
     if (rc) return rc;
     if (!sizes) return fail(MGGX_EINVAL, "core_layout_device: NULL sizes");
+    mggx::GraphInfo *g = nullptr;
+    rc = mggx::graph_info(d_ptr, nullptr, d_col, nullptr, rows, false, &g);
+    if (rc) return rc;
     mggx::CorePlan *p = nullptr;
-    rc = mggx::core_plan_get(d_ptr, d_col, rows, lb, core_rows, &p);
+    rc = mggx::core_plan_get(d_ptr, d_col, rows, lb, core_rows, g->serial, &p);
     if (rc) return rc;
     if (p->unsuitable) return fail(MGGX_EINVAL, "core layout: no core of whole 512-row units in %d rows, or a neighbor id outside [lb, lb + rows)", rows);
     const int64_t nblk = (int64_t)(p->core / 64) * p->ntiles + 1;

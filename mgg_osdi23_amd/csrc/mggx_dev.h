@@ -109,7 +109,10 @@ struct Plan {
     int block_lb = 0;          // id of the first row of block 0 (part of the cache key)
     int blocks = 1;
     bool unsuitable = false;   // blocked plan asked for, but the rows are not sorted by neighbor id
-    bool pinned = false;       // used inside a stream capture: a captured graph holds its device addresses, never evicted
+    bool pinned = false;       // used inside a stream capture: a captured graph holds its device addresses, so its device
+                               // blocks are never freed before mggx_release_cached (dropped from the cache, they are retired)
+    int graph_serial = 0;      // the graph record (GraphInfo::serial) this plan was built under; a call under another record
+                               // of the same addresses -- the arrays may hold another graph now -- rebuilds it
     size_t bytes = 0;          // device memory held
     Guard guard;               // explicit-partition plans only (the others are guarded through their GraphInfo)
 };
@@ -148,7 +151,8 @@ struct CorePlan {
     std::vector<int> work;    // [core / CORE_GROUP_ROWS][ntiles] list chunks of a row group in a tile (host copy)
     long long total_chunks = 0;
     bool unsuitable = false;  // no core of whole units fits, or the ids do not allow it
-    bool pinned = false;      // used inside a stream capture: never evicted
+    bool pinned = false;      // used inside a stream capture: its device blocks outlive the cache entry (retired, not freed)
+    int graph_serial = 0;     // as Plan::graph_serial
     size_t bytes = 0;         // device memory held
 };
 
@@ -167,6 +171,7 @@ struct GraphInfo {
     std::vector<Predicted> predicted;  // what the cost model said for a row width (evaluated once, a millisecond of host time)
     bool internal = false;  // arrays owned by the library (the remainder CSR of a dense-core plan): no content check
     bool pinned = false;    // used inside a stream capture: never evicted
+    int serial = 0;         // unique per record: plans remember the record they were built under
     Guard guard;
     int64_t nnz_l = 0, nnz_r = 0;
     // knobs measured best by mggx_sag_np_div_tune for a row width and element type; used where a call passes 0
@@ -192,6 +197,7 @@ struct State {
     int plan_check = 1;            // 0: checks off (the caller vouches for its arrays), 1: live edge counts, 2: + fingerprint kernel
     volatile int *h_stale = nullptr;  // pinned host word the check kernel writes a record id to on a mismatch
     int next_guard_id = 1;
+    int next_graph_serial = 1;
     // blocks a captured graph may still point at: kept until mggx_release_cached instead of being freed on growth
     bool ws_captured = false, core_ws_captured = false;
     std::vector<void *> retired;
@@ -216,11 +222,16 @@ bool capturing();
 // found (MGGX_EINVAL, after dropping the records) -- called on entry of every compute call and by mggx_sync.
 int guard_arm(Guard &g);
 int guard_check(Guard &g, Gate *gate);
-void guard_free(Guard &g);
+// `retire`: a captured graph may still launch the check kernel that writes this record's verdict word -- the word is kept
+// until mggx_release_cached instead of being freed.
+void guard_free(Guard &g, bool retire = false);
+// Hands a device block a captured graph may still point at to the list mggx_release_cached frees.
+void retire_block(void *p, size_t bytes);
 int stale_poll();
-int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int rows, int ps, Plan **out);
+// graph_serial: GraphInfo::serial of the call's graph record; a cached plan built under another record is rebuilt.
+int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int rows, int ps, int graph_serial, Plan **out);
 // Column-blocked plan of a local-only CSR; (*out)->unsuitable is set when the rows are not sorted by neighbor id.
-int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int ps, int block_rows, Plan **out);
+int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int ps, int block_rows, int graph_serial, Plan **out);
 int graph_info(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_l, const int *d_col_r, int rows, bool internal, GraphInfo **out);
 int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows,
                       int num_parts, int ps, Plan **out);
@@ -230,7 +241,7 @@ int explicit_desc_fill(const int *d_row_ptr, const int *d_part_ptr, const int *d
 int static_scratch_ptr(unsigned char **out);
 void plan_free(Plan *p);
 int forget_pointer(const void *d_ptr);
-int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, CorePlan **out);
+int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, int graph_serial, CorePlan **out);
 // Cost model of the dense core (degree histogram x row width): the core size that is predicted to pay for this CSR, a
 // multiple of 4096, or -1 for none.  table_bytes = rows x row pitch of the feature table.  Fetches the record's degree
 // profile on first use (one sort of the degrees on the device, 4 KiB to the host; synchronises).

@@ -443,9 +443,20 @@ int guard_check(Guard &g, Gate *gate)
     return MGGX_OK;
 }
 
-void guard_free(Guard &g)
+void retire_block(void *p, size_t bytes)
 {
-    if (g.d_fp) (void)hipFree(g.d_fp);
+    if (!p) return;
+    State &s = state();
+    s.retired.push_back(p);
+    s.retired_bytes += bytes;
+}
+
+void guard_free(Guard &g, bool retire)
+{
+    if (g.d_fp) {
+        if (retire) retire_block(g.d_fp, 16);
+        else (void)hipFree(g.d_fp);
+    }
     g.d_fp = nullptr;
     g.armed = false;
 }
@@ -498,13 +509,21 @@ int exclusive_scan_i32(const int *d_in, int *d_out, int n, long long *total_host
     return MGGX_OK;
 }
 
+// A plan that was used inside a stream capture leaves the cache like any other, but a captured graph still holds the
+// addresses of its device arrays: those are retired (freed by mggx_release_cached), not freed.
 void plan_free(Plan *p)
 {
     if (!p) return;
-    if (p->d_desc) (void)hipFree(p->d_desc);
-    if (p->d_off) (void)hipFree(p->d_off);
-    if (p->d_empty_rows) (void)hipFree(p->d_empty_rows);
-    guard_free(p->guard);
+    if (p->pinned) {
+        retire_block(p->d_desc, sizeof(int4) * (size_t)std::max(p->num_parts, 1));
+        retire_block(p->d_off, sizeof(int) * ((size_t)p->rows + 1));
+        retire_block(p->d_empty_rows, sizeof(int) * (size_t)std::max(p->rows, 1));
+    } else {
+        if (p->d_desc) (void)hipFree(p->d_desc);
+        if (p->d_off) (void)hipFree(p->d_off);
+        if (p->d_empty_rows) (void)hipFree(p->d_empty_rows);
+    }
+    guard_free(p->guard, p->pinned);
     delete p;
 }
 
@@ -564,13 +583,48 @@ struct BuildClock {  // adds the host-clock time of a plan build to the library'
 };
 static const char *const CAPTURE_MSG = "plan: first use of this CSR and partition size inside a stream capture; call once outside the capture first";
 
-int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int rows, int ps, Plan **out)
+// Plans belong to the graph record (GraphInfo) they were built under: the record vouches for what the arrays hold (its
+// edge counts, its fingerprint), so a plan is found by its addresses AND that record's serial, and it goes when the record
+// goes.  A later record of the same addresses -- the arrays may hold another graph by then -- builds its own.
+static void drop_plans_of_record(int serial)
+{
+    State &s = state();
+    if (serial == 0) return;
+    bool synced = false;
+    const auto sync_once = [&]() {
+        if (!synced && s.device >= 0) (void)hipDeviceSynchronize();  // kernels in flight on either stream may still read them
+        synced = true;
+    };
+    for (size_t i = 0; i < s.plans.size();) {
+        if (s.plans[i]->graph_serial == serial) {
+            sync_once();
+            Plan *p = s.plans[i];
+            s.plans.erase(s.plans.begin() + (long)i);
+            plan_free(p);
+        } else {
+            ++i;
+        }
+    }
+    std::vector<CorePlan *> gone;
+    for (size_t i = 0; i < s.cores.size();) {
+        if (s.cores[i]->graph_serial == serial) {
+            gone.push_back(s.cores[i]);
+            s.cores.erase(s.cores.begin() + (long)i);
+        } else {
+            ++i;
+        }
+    }
+    if (!gone.empty()) sync_once();
+    for (CorePlan *c : gone) core_plan_free(c);  // forgets the records (and so the plans) of its remainder CSR in turn
+}
+
+int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int rows, int ps, int graph_serial, Plan **out)
 {
     State &s = state();
     for (size_t i = 0; i < s.plans.size(); ++i) {
         const Plan *p = s.plans[i];
         if (p->d_ptr_l == d_ptr_l && p->d_ptr_r == d_ptr_r && p->d_col_r == d_col_r && p->rows == rows && p->ps == ps &&
-            !p->d_part_ptr && p->blocks == 1 && !p->unsuitable) {
+            !p->d_part_ptr && p->blocks == 1 && !p->unsuitable && p->graph_serial == graph_serial) {
             *out = cache_hit(i);
             return MGGX_OK;
         }
@@ -578,6 +632,7 @@ int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int row
     if (capturing()) return fail(MGGX_EINVAL, "%s", CAPTURE_MSG);
     BuildClock clock;
     Plan *p = new Plan;
+    p->graph_serial = graph_serial;
     p->d_ptr_l = d_ptr_l;
     p->d_ptr_r = d_ptr_r;
     p->d_col_r = d_col_r;  // the plan holds the largest remote id
@@ -727,13 +782,13 @@ int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_
     return MGGX_OK;
 }
 
-int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int ps, int block_rows, Plan **out)
+int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int ps, int block_rows, int graph_serial, Plan **out)
 {
     State &s = state();
     for (size_t i = 0; i < s.plans.size(); ++i) {
         const Plan *p = s.plans[i];
         if (p->d_ptr_l == d_ptr_l && p->d_col_l == d_col_l && p->real_rows == rows && p->ps == ps && p->block_rows == block_rows && p->block_lb == lb &&
-            (p->blocks > 1 || p->unsuitable)) {
+            (p->blocks > 1 || p->unsuitable) && p->graph_serial == graph_serial) {
             *out = cache_hit(i);
             return MGGX_OK;
         }
@@ -745,6 +800,7 @@ int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, i
     const long long vrows = blocks * rows;
     if (blocks < 2 || vrows + rows > 0x7fffffffLL) return fail(MGGX_ELIMIT, "plan: %lld column blocks over %d rows", blocks, rows);
     Plan *p = new Plan;
+    p->graph_serial = graph_serial;
     p->d_ptr_l = d_ptr_l;
     p->d_col_l = d_col_l;
     p->real_rows = rows;
@@ -837,6 +893,8 @@ int graph_info(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_l, const
     g.d_col_r = d_col_r;
     g.rows = rows;
     g.internal = internal;
+    g.serial = s.next_graph_serial++;
+    if (s.next_graph_serial > 0x3fffffff) s.next_graph_serial = 1;
     int ends[2] = {0, 0};
     if (rows > 0) {
         MGGX_HIP(hipStreamSynchronize(s.stream));
@@ -849,8 +907,10 @@ int graph_info(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_l, const
         for (auto it = s.graphs.begin(); it != s.graphs.end(); ++it)
             if (!it->pinned) {
                 (void)hipStreamSynchronize(s.stream);  // a check kernel in flight may still write the record's verdict word
+                const int serial = it->serial;
                 guard_free(it->guard);
                 s.graphs.erase(it);
+                drop_plans_of_record(serial);  // may erase further records (the remainder CSRs of its dense-core plans)
                 break;
             }
     s.graphs.push_back(g);
@@ -879,12 +939,15 @@ int graph_info(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_l, const
     return MGGX_OK;
 }
 
-// Drops every cached plan and graph record keyed by this device address (an array about to be freed or rewritten).
+// Drops every cached plan and graph record keyed by this device address (an array about to be freed or rewritten).  What a
+// captured graph may still point at (records used inside a stream capture) leaves the lookup tables all the same, but its
+// device blocks are retired, not freed: a replay then reads the old plan, never freed memory.
 int forget_pointer(const void *d_ptr)
 {
     if (!d_ptr) return MGGX_OK;  // NULL is what absent arrays are keyed by: nothing hangs on it
     State &s = state();
     bool synced = false;
+    std::vector<int> orphaned;  // serials of the graph records dropped below
     for (size_t i = 0; i < s.plans.size();) {
         Plan *p = s.plans[i];
         if (p->d_ptr_l == d_ptr || p->d_ptr_r == d_ptr || p->d_col_l == d_ptr || p->d_col_r == d_ptr || p->d_part_ptr == d_ptr ||
@@ -905,7 +968,8 @@ int forget_pointer(const void *d_ptr)
                 MGGX_HIP(hipStreamSynchronize(s.stream));
                 synced = true;
             }
-            guard_free(it->guard);
+            guard_free(it->guard, it->pinned);
+            orphaned.push_back(it->serial);
             it = s.graphs.erase(it);
         } else {
             ++it;
@@ -923,6 +987,7 @@ int forget_pointer(const void *d_ptr)
     }
     if (!gone.empty() && !synced && s.device >= 0) MGGX_HIP(hipStreamSynchronize(s.stream));
     for (CorePlan *c : gone) core_plan_free(c);
+    for (int serial : orphaned) drop_plans_of_record(serial);  // plans of a dropped record keyed by its other arrays only
     return MGGX_OK;
 }
 

@@ -75,8 +75,11 @@ MGGX_EXPORT int mggx_init(int device)
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(MGGX_EHIP, "init: device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
     state().device = device;
-    unsigned char *scratch_addr = nullptr;  // set-up of the allocation-free entry point: look its array up on this device now
-    return mggx::static_scratch_ptr(&scratch_addr);
+    // Set-up of the allocation-free entry point: its array's address on this device is looked up now.  Should the lookup
+    // fail, only that entry point is unavailable (mggx_sag_parts_static asks again and reports the error itself).
+    unsigned char *scratch_addr = nullptr;
+    (void)mggx::static_scratch_ptr(&scratch_addr);
+    return MGGX_OK;
 }
 
 MGGX_EXPORT int mggx_device_name(char *buf, size_t len)

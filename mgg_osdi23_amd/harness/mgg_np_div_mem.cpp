@@ -8,6 +8,8 @@
 // keep their own buffer (the reference lets the second aggregation overwrite them).
 // With nGPU > 1 the rows of the other ranks are produced once, before the timed
 // loop, by a whole-graph pass on this GPU and staged as the remote tables.
+#include <cmath>
+
 #include "harness_common.h"
 
 int main(int argc, char *argv[])
@@ -96,6 +98,26 @@ int main(int argc, char *argv[])
         bool ok = check_equal(ref.data(), h.data(), rows * outdim, outdim);
         printf("Validation on PE-{%d}, status: %s\n", a.pe, ok ? "True" : "False");
         a.validate = false;
+    }
+
+    if (a.fuse_softmax) {
+        // what the timed iterations below run -- the softmax inside the last aggregation -- against the same forward
+        // followed by softmax_new_forward: the two must give the same class probabilities
+        std::vector<float> fused((size_t)rows * outdim), plain((size_t)rows * outdim);
+        forward();
+        MGG_CHECK(mggx_memcpy_d2h(fused.data(), d_buff_1, fused.size() * sizeof(float)));
+        a.fuse_softmax = false;
+        forward();
+        MGG_CHECK(mggx_memcpy_d2h(plain.data(), d_buff_1, plain.size() * sizeof(float)));
+        a.fuse_softmax = true;
+        float worst = 0.f;
+        double total = 0.0;
+        for (size_t i = 0; i < fused.size(); ++i) {
+            worst = std::max(worst, std::fabs(fused[i] - plain[i]));
+            total += fused[i];
+        }
+        const bool ok = worst <= 1e-6f && std::fabs(total - (double)rows) <= 1e-4 * (double)rows;  // every row sums to one
+        printf("Fused softmax on PE-{%d}, status: %s (max abs diff %.3g against aggregation + softmax_forward)\n", a.pe, ok ? "True" : "False", worst);
     }
 
     std::clock_t c_start = std::clock();

@@ -272,20 +272,29 @@ def sync() -> None:
 
 
 _pinned = {}  # CSR tensors of cached plans, by address: keeps the addresses from being reused while cached
+_captured = set()  # keys of _pinned that were used while a stream capture was recording: a captured graph reads those arrays
 _PIN_MAX_SETS, _PIN_MAX_BYTES = 64, 8 << 30
 
 
 def _pin(*tensors) -> None:
     """Holds a reference to the CSR tensors of a call so that torch's allocator does not hand their addresses to other
     data while the library has plans cached for them; bounded by count and bytes, oldest first, and the library forgets
-    a set before it is let go."""
+    a set before it is let go.  Sets used inside a stream capture are never let go here (a replay of the captured graph
+    reads them); forget() and release_cached() are the ways to drop those."""
+    import torch
     key = tuple(t.data_ptr() if t is not None else 0 for t in tensors)
+    if torch.cuda.is_current_stream_capturing():
+        _captured.add(key)
     if key in _pinned:
         return
     _pinned[key] = tensors
     size = lambda ts: sum(t.numel() * t.element_size() for t in ts if t is not None)
-    while len(_pinned) > _PIN_MAX_SETS or (len(_pinned) > 1 and sum(size(ts) for ts in _pinned.values()) > _PIN_MAX_BYTES):
-        old = _pinned.pop(next(iter(_pinned)))
+    while True:
+        loose = [k for k in _pinned if k not in _captured and k != key]
+        over = len(_pinned) > _PIN_MAX_SETS or sum(size(ts) for ts in _pinned.values()) > _PIN_MAX_BYTES
+        if not over or not loose:
+            break
+        old = _pinned.pop(loose[0])
         for t in old:
             if t is not None:
                 _check(lib().mggx_forget(C.c_void_p(t.data_ptr())))
@@ -296,11 +305,13 @@ def forget(tensor) -> None:
     _check(lib().mggx_forget(C.c_void_p(tensor.data_ptr())))
     for key in [k for k in _pinned if tensor.data_ptr() in k]:
         _pinned.pop(key)
+        _captured.discard(key)
 
 
 def release_cached() -> None:
     _check(lib().mggx_release_cached())
     _pinned.clear()
+    _captured.clear()
 
 
 def set_plan_check(level: int) -> None:

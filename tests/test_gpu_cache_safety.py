@@ -192,6 +192,131 @@ def test_captured_graph_survives_workspace_growth_and_cache_pressure(gpu):
         gpu.release_cached()
 
 
+@pytest.mark.parametrize("core_rows", [-1, 1024])
+def test_captured_graph_survives_forget(gpu, core_rows):
+    """mggx_forget on a CSR array whose plans a captured graph still launches: the records leave the lookup tables, but
+    their device blocks (descriptors, row offsets, the dense-core lists, the fingerprint word) are retired, not freed -- a
+    replay reads the old plan, never freed memory."""
+    import torch
+    V, dim = 6000, 16
+    ptr, col = gpu.gen_rmat(13, V, 200_000, seed=21)
+    x = gpu.fill_normal((V, dim), seed=1)
+    d_ptr, d_col, d_x = to_dev(ptr), to_dev(col), to_dev(x)
+    zp, zc = torch.zeros(V + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    out = torch.empty(V, dim, device="cuda")
+    call = lambda: gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, zp, zc, 0, V, dim, V, 0, 16, 4, 2, core_rows=core_rows)
+    gpu.release_cached()
+    gpu.set_plan_check(2)  # the fingerprint kernel is captured too and writes the record's verdict word on every replay
+    side = torch.cuda.Stream()
+    try:
+        with torch.cuda.stream(side):
+            gpu.use_torch_stream()
+            call()
+            side.synchronize()
+            want = out.clone()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                gpu.use_torch_stream()
+                call()
+            gpu.use_torch_stream()
+            before = gpu.cache_stats()
+            assert before["plans"] >= 1 and before["retired_bytes"] == 0
+            gpu.forget(d_ptr)
+            after = gpu.cache_stats()
+            assert after["plans"] == 0 and after["core_plans"] == 0
+            assert after["retired_bytes"] >= before["plan_bytes"] + before["core_plan_bytes"] > 0
+            # memory handed out now must not be what the graph reads
+            junk = [torch.full((1 << 20,), -1, dtype=torch.int32, device="cuda") for _ in range(8)]
+            for i in range(2):
+                out.fill_(-1.0)
+                graph.replay()
+                side.synchronize()
+                assert torch.equal(out, want), "replay %d after mggx_forget differs" % i
+            del junk
+            # an eager call afterwards builds fresh records and gives the same sums
+            out.fill_(-1.0)
+            call()
+            side.synchronize()
+            assert torch.equal(out, want)
+    finally:
+        torch.cuda.synchronize()
+        gpu.use_torch_stream()
+        gpu.set_plan_check(1)
+        gpu.release_cached()
+    assert gpu.cache_stats()["retired_bytes"] == 0
+
+
+def test_plans_go_with_their_graph_record(gpu):
+    """The content check lives with the graph record (32 cached).  A dense-core plan must not outlive the record it was
+    built under: after 33 other CSR sets have passed through, the first set's arrays are rewritten in place with another
+    graph of another size; the next call makes a fresh record from what is there now -- and must not find the old graph's
+    dense-core plan (which holds its own copy of the old remaining CSR) by address."""
+    import torch
+    V, dim = 6000, 16
+    ptr_a, col_a = gpu.gen_rmat(13, V, 200_000, seed=31)
+    ptr_b, col_b = gpu.gen_rmat(13, V, 120_000, seed=32)
+    assert len(col_b) < len(col_a)
+    x = gpu.fill_normal((V, dim), seed=3)
+    d_x, d_ptr, d_col = to_dev(x), to_dev(ptr_a), to_dev(col_a)
+    zp, zc = torch.zeros(V + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    out = torch.empty(V, dim, device="cuda")
+    call = lambda: gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_col, zp, zc, 0, V, dim, V, 0, 16, 4, 2, core_rows=1024)
+    gpu.release_cached()
+    call()
+    gpu.sync()
+    assert "core=1024" in gpu.last_agg_kernel() and gpu.cache_stats()["core_plans"] == 1
+    want, mag = _want(x, ptr_a, col_a, V, dim)
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "graph A")
+    # 33 other CSR sets (no dense core: core plans are only displaced by other core plans)
+    n = 300
+    sp, sc = gpu.gen_rmat(9, n, 3000, seed=33)
+    others = [(to_dev(sp), to_dev(sc)) for _ in range(33)]
+    szp, sx, so = torch.zeros(n + 1, dtype=torch.int32, device="cuda"), to_dev(gpu.fill_normal((n, dim), seed=4)), torch.empty(n, dim, device="cuda")
+    for p_, c_ in others:
+        gpu.mgg_SAG_np_div(so, sx, p_, c_, szp, zc, 0, n, dim, n, 0, 16, 4, 2, core_rows=-1)
+    gpu.sync()
+    assert gpu.cache_stats()["core_plans"] == 0, "the dense-core plan outlived its graph record"
+    d_ptr.copy_(torch.from_numpy(ptr_b))
+    d_col[: len(col_b)].copy_(torch.from_numpy(col_b))
+    torch.cuda.synchronize()
+    out.fill_(-7.0)
+    call()
+    gpu.sync()
+    want, mag = _want(x, ptr_b, col_b, V, dim)
+    assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "graph B in the arrays of graph A, new record")
+    for p_, _c in others:
+        gpu.forget(p_)
+    gpu.forget(d_ptr)
+
+
+def test_two_records_over_one_row_pointer_array_keep_their_own_plans(gpu):
+    """Two CSRs that share the row-pointer array but not the column array are two graph records, each with its own plan:
+    alternating between them rebuilds nothing."""
+    import torch
+    V, dim = 4000, 16
+    ptr, col = gpu.gen_rmat(12, V, 60_000, seed=41)
+    rng = np.random.default_rng(0)
+    col2 = rng.integers(0, V, len(col)).astype(np.int32)
+    x = gpu.fill_normal((V, dim), seed=5)
+    d_x, d_ptr, d_c1, d_c2 = to_dev(x), to_dev(ptr), to_dev(col), to_dev(col2)
+    zp, zc = torch.zeros(V + 1, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    out = torch.empty(V, dim, device="cuda")
+    gpu.release_cached()
+    for d_c in (d_c1, d_c2):
+        gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_c, zp, zc, 0, V, dim, V, 0, 16, 4, 2, core_rows=-1, col_block_rows=-1)
+    gpu.sync()
+    built = gpu.cache_stats()
+    assert built["plans"] == 2
+    for d_c, c in ((d_c1, col), (d_c2, col2), (d_c1, col)):
+        gpu.mgg_SAG_np_div(out, d_x, d_ptr, d_c, zp, zc, 0, V, dim, V, 0, 16, 4, 2, core_rows=-1, col_block_rows=-1)
+        gpu.sync()
+        want, mag = _want(x, ptr, c, V, dim)
+        assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "shared row pointers")
+    now = gpu.cache_stats()
+    assert now["plans"] == 2 and now["plan_build_ms"] == built["plan_build_ms"]
+    gpu.forget(d_ptr)
+
+
 # --------------------------------------------------------------------------- dense-core plan built on the GPU
 @pytest.mark.parametrize("shape", ["rmat", "ragged", "unsorted_parallel"])
 def test_core_plan_built_on_the_gpu_is_the_host_layout(gpu, shape):

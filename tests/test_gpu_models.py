@@ -226,7 +226,7 @@ def test_harness_programs_with_the_search(gpu, graph_files, prog, dims):
 def test_harness_compact_remote_and_fused_softmax(gpu, graph_files):
     """--compact-remote: the aggregation-only program stages one row per distinct remote id (most referenced first) and
     still passes the all-ones validation on a 4-way share; --fuse-softmax: the 2-layer program ends its last aggregation
-    in the softmax and logs like the plain run."""
+    in the softmax, checks that forward against aggregation + softmax_forward, and logs like the plain run."""
     files, ptr, col = graph_files
     exe = os.path.join(BIN, "mgg_np_div_kernel")
     cmd = [exe] + files + ["4", "16", "4", "2", "16", "16", "16", "--pe", "1", "--iters", "3", "--validate", "--compact-remote"]
@@ -242,6 +242,8 @@ def test_harness_compact_remote_and_fused_softmax(gpu, graph_files):
         r = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
         assert r.returncode == 0, r.stdout + r.stderr
         assert re.search(r"Validation on PE-\{0\}, status: True", r.stdout) and re.search(r"MPI time \(ms\) ([0-9.]+)", r.stdout), r.stdout
+        if extra:  # the forward the timed iterations run (softmax inside the aggregation) against aggregation + softmax_forward
+            assert re.search(r"Fused softmax on PE-\{0\}, status: True", r.stdout), r.stdout
 
 
 def test_cpp_layer_entry_points(gpu, tmp_path):

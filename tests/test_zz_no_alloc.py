@@ -43,6 +43,51 @@ def test_static_entry_point_matches_sag_parts_twice(gpu):
     _case(gpu, 500, 9, 3_000, 9, 64, 3, 2, 3)
 
 
+def test_static_entry_point_runs_under_capture_and_allocates_nothing(gpu):
+    """What the entry point exists for: a call launches kernels and nothing else.  It is recorded into a HIP graph on a
+    stream in global capture mode -- an allocation, a copy to the host or a synchronisation inside the call would fail the
+    capture -- the replays are compared with the eager result, and neither the library's caches nor the device's free
+    memory move across an eager call."""
+    import torch
+    V, dim, ps = 30_000, 16, 16
+    ptr, col = gpu.gen_rmat(15, V, 700_000, seed=13)
+    x = gpu.fill_normal((V, dim), seed=14)
+    pp, p2n, _ = orc.build_part(ptr, V, ps)
+    d_x, d_ptr, d_col, d_pp, d_p2n = to_dev(x), to_dev(ptr), to_dev(col), to_dev(pp), to_dev(p2n)
+    args = (d_x, d_ptr, d_col, d_pp, d_p2n, 0, V, len(p2n), ps, dim, 32, 4, 2)
+    out = torch.zeros(V, dim, device="cuda")
+    gpu.SAG_host_static(out, *args)  # code loaded, the array's address looked up
+    gpu.sync()
+    want = out.clone()
+    stats0, free0 = gpu.cache_stats(), torch.cuda.mem_get_info()[0]
+    out.zero_()
+    gpu.SAG_host_static(out, *args)
+    gpu.sync()
+    assert torch.equal(out, want)
+    assert gpu.cache_stats() == stats0, "the static entry point touched the library's caches"
+    assert torch.cuda.mem_get_info()[0] == free0, "device memory was allocated or freed across the call"
+    side = torch.cuda.Stream()
+    try:
+        with torch.cuda.stream(side):
+            gpu.use_torch_stream()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side, capture_error_mode="global"):
+                gpu.use_torch_stream()
+                gpu.SAG_host_static(out, *args)
+            for i in range(3):
+                out.zero_()  # the call accumulates into its output
+                graph.replay()
+                side.synchronize()
+                assert torch.equal(out, want), "replay %d differs from the eager call" % i
+                gpu.use_torch_stream()
+                gpu.SAG_host_static(out, *args)  # eager work between the replays shares the array
+                side.synchronize()
+    finally:
+        torch.cuda.synchronize()
+        gpu.use_torch_stream()
+    assert gpu.cache_stats() == stats0
+
+
 def test_static_entry_point_rejects_what_does_not_fit(gpu):
     import torch
     z = torch.zeros(4, dtype=torch.int32, device="cuda")
