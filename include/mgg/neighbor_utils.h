@@ -49,11 +49,12 @@ std::vector<std::vector<T>> split_CSR(std::vector<T> &origin_ptr, std::vector<T>
     std::vector<T> local_ptr(rows + 1, 0), remote_ptr(rows + 1, 0), local_col, remote_col;
     if constexpr (std::is_same<T, int>::value) {
         int64_t nl = 0, nr = 0;
-        MGG_CHECK(mggx_split_csr(origin_ptr.data(), origin_col_idx.data(), lb, ub, nullptr, nullptr, nullptr, nullptr, &nl, &nr));
+        int dummy = 0;  // non-null arrays even when a side, or the whole graph, has no edge
+        const int *col = origin_col_idx.empty() ? &dummy : origin_col_idx.data();
+        MGG_CHECK(mggx_split_csr(origin_ptr.data(), col, lb, ub, nullptr, nullptr, nullptr, nullptr, &nl, &nr));
         local_col.resize((size_t)nl);
         remote_col.resize((size_t)nr);
-        int dummy = 0;  // non-null targets even when a side is empty
-        MGG_CHECK(mggx_split_csr(origin_ptr.data(), origin_col_idx.data(), lb, ub, local_ptr.data(), remote_ptr.data(),
+        MGG_CHECK(mggx_split_csr(origin_ptr.data(), col, lb, ub, local_ptr.data(), remote_ptr.data(),
                                  nl ? local_col.data() : &dummy, nr ? remote_col.data() : &dummy, &nl, &nr));
     } else {
         for (T i = lb; i < ub; ++i) {

@@ -31,6 +31,7 @@ sed -n '71p'  "$UT" | grep -q 'SAG_ref'    || { echo "build_ref: SAG_ref not at 
 {
     cat <<'EOF'
 #include <limits>
+#include <sstream>
 #include <vector>
 #include <string>
 #include <cstdio>
@@ -79,6 +80,52 @@ void ref_graph_load(const char* beg, const char* csr, const char* weight,
     if (beg_pos) memcpy(beg_pos, g.beg_pos, sizeof(int) * ((size_t)g.vert_count + 1));
     if (csr_out) memcpy(csr_out, g.csr, sizeof(int) * (size_t)g.edge_count);
     if (weight_out) memcpy(weight_out, g.weight, sizeof(int) * (size_t)g.edge_count);
+}
+// split_CSR<long> / build_part<long>: the same templates for 64-bit ids, sizes as above
+void ref_split_csr_long(const long* ptr, int64_t n_ptr, const long* col, int64_t n_col, long lb, long ub,
+                        long* lp, long* rp, long* lc, long* rc, int64_t* n) {
+    std::vector<long> p(ptr, ptr + n_ptr), c(col, col + n_col);
+    auto r = split_CSR<long>(p, c, lb, ub);
+    for (int i = 0; i < 4; i++) n[i] = (int64_t)r[i].size();
+    if (lp) memcpy(lp, r[0].data(), r[0].size() * sizeof(long));
+    if (rp) memcpy(rp, r[1].data(), r[1].size() * sizeof(long));
+    if (lc) memcpy(lc, r[2].data(), r[2].size() * sizeof(long));
+    if (rc) memcpy(rc, r[3].data(), r[3].size() * sizeof(long));
+}
+void ref_build_part_long(const long* indptr, int64_t n_ptr, long num_nodes, long part_size,
+                         long* part_ptr, long* part2node, long* node2part, int64_t* n) {
+    std::vector<long> p(indptr, indptr + n_ptr);
+    auto r = build_part<long>(std::string("ref"), p, num_nodes, part_size);
+    for (int i = 0; i < 3; i++) n[i] = (int64_t)r[i].size();
+    if (part_ptr) memcpy(part_ptr, r[0].data(), r[0].size() * sizeof(long));
+    if (part2node) memcpy(part2node, r[1].data(), r[1].size() * sizeof(long));
+    if (node2part) memcpy(node2part, r[2].data(), r[2].size() * sizeof(long));
+}
+// assemble_csr_matrix (which = 0) / assemble_simetric_csr_matrix (which = 1): n[3] = {|row_ptr|, |col_ind|, |val|};
+// getBandwidth of the result in *bandwidth; printMatrix's output for the result with row_ptr[0] set to 1 into text (at most
+// text_cap - 1 characters) when non-NULL
+void ref_mtx_load_other(int which, const char* path, int* row_ptr, int* col_ind, double* val, int64_t* n, int* bandwidth,
+                        char* text, int64_t text_cap) {
+    CSR m = which ? assemble_simetric_csr_matrix(std::string(path)) : assemble_csr_matrix(std::string(path));
+    n[0] = (int64_t)m.row_ptr.size();
+    n[1] = (int64_t)m.col_ind.size();
+    n[2] = (int64_t)m.val.size();
+    if (row_ptr) memcpy(row_ptr, m.row_ptr.data(), m.row_ptr.size() * sizeof(int));
+    if (col_ind) memcpy(col_ind, m.col_ind.data(), m.col_ind.size() * sizeof(int));
+    if (val) memcpy(val, m.val.data(), m.val.size() * sizeof(double));
+    if (bandwidth) *bandwidth = getBandwidth(m);
+    if (text && text_cap > 0) {
+        std::ostringstream os;
+        std::streambuf* old = std::cout.rdbuf(os.rdbuf());
+        CSR one_based = m;  // printMatrix reads col_ind[row_ptr[i-1] - 1 ...): with row_ptr[0] = 0 it would start before the array
+        one_based.row_ptr[0] = 1;
+        printMatrix(one_based);
+        std::cout.rdbuf(old);
+        const std::string t = os.str();
+        const size_t k = std::min<size_t>(t.size(), (size_t)text_cap - 1);
+        memcpy(text, t.data(), k);
+        text[k] = 0;
+    }
 }
 // assemble_csr_matrix_new: n[2] = {|row_ptr|, |col_ind|}
 void ref_mtx_load(const char* path, int* row_ptr, int* col_ind, int64_t* n) {

@@ -297,3 +297,40 @@ def ref_mtx_load(path):
     ci = np.zeros(n[1], np.int32)
     ref().ref_mtx_load(path.encode(), _i(rp), _i(ci), n)
     return rp, ci
+
+
+def _l(a):
+    return a.ctypes.data_as(C.POINTER(C.c_long))
+
+
+def ref_split_csr_long(ptr, col, lb, ub):
+    """split_CSR<long> of the reference -> the four arrays as int64."""
+    ptr, col = np.ascontiguousarray(ptr, np.int64), np.ascontiguousarray(col, np.int64)
+    n = (C.c_int64 * 4)()
+    ref().ref_split_csr_long(_l(ptr), C.c_int64(len(ptr)), _l(col), C.c_int64(len(col)), C.c_long(lb), C.c_long(ub), None, None, None, None, n)
+    outs = [np.zeros(n[i], np.int64) for i in range(4)]
+    ref().ref_split_csr_long(_l(ptr), C.c_int64(len(ptr)), _l(col), C.c_int64(len(col)), C.c_long(lb), C.c_long(ub), _l(outs[0]), _l(outs[1]),
+                             _l(outs[2]), _l(outs[3]), n)
+    return tuple(outs)
+
+
+def ref_build_part_long(indptr, num_nodes, ps):
+    indptr = np.ascontiguousarray(indptr, np.int64)
+    n = (C.c_int64 * 3)()
+    ref().ref_build_part_long(_l(indptr), C.c_int64(len(indptr)), C.c_long(num_nodes), C.c_long(ps), None, None, None, n)
+    outs = [np.zeros(n[i], np.int64) for i in range(3)]
+    ref().ref_build_part_long(_l(indptr), C.c_int64(len(indptr)), C.c_long(num_nodes), C.c_long(ps), _l(outs[0]), _l(outs[1]), _l(outs[2]), n)
+    return tuple(outs)
+
+
+def ref_mtx_load_other(path, symmetric):
+    """assemble_csr_matrix / assemble_simetric_csr_matrix of the reference -> dict(row_ptr, col_ind, val, bandwidth, text):
+    getBandwidth of the result and what printMatrix prints for it (with row_ptr[0] = 1, see build_ref.sh)."""
+    n = (C.c_int64 * 3)()
+    ref().ref_mtx_load_other(int(symmetric), path.encode(), None, None, None, n, None, None, C.c_int64(0))
+    rp, ci, val = np.zeros(n[0], np.int32), np.zeros(n[1], np.int32), np.zeros(n[2], np.float64)
+    bw = C.c_int()
+    text = C.create_string_buffer(1 << 20)
+    ref().ref_mtx_load_other(int(symmetric), path.encode(), _i(rp), _i(ci), val.ctypes.data_as(C.POINTER(C.c_double)), n, C.byref(bw),
+                             text, C.c_int64(len(text)))
+    return {"row_ptr": rp, "col_ind": ci, "val": val, "bandwidth": bw.value, "text": text.value.decode()}

@@ -42,6 +42,36 @@ def random_csr(rng, n, avg_deg, empty_frac=0.0, hub=0):
     return ptr, col
 
 
+def mtx_other():
+    """tests/golden/mtx_other.json: assemble_csr_matrix, assemble_simetric_csr_matrix, getBandwidth and printMatrix of the
+    reference's csr_formatter.h on small hand-written and seeded files (the file text is stored with the outputs)."""
+    import tempfile
+    files = [
+        ("hand_sorted", "%%MatrixMarket matrix coordinate real general\n% a comment\n4 4 7\n1 1 1.5\n1 3 2\n2 2 3\n3 1 4\n3 4 5.25\n4 2 6\n4 4 7\n"),
+        ("hand_gap_rows", "5 5 6\n1 2 1\n1 5 2\n3 1 3\n3 3 4\n5 4 5\n5 5 6\n"),
+        ("hand_lower_triangle", "%%MatrixMarket matrix coordinate real symmetric\n4 4 6\n1 1 10\n2 1 20\n3 2 30\n4 1 40\n4 3 50\n4 4 60\n"),
+    ]
+    rng = np.random.default_rng(99)
+    n = 9
+    ent = sorted({(int(r), int(c)) for r, c in zip(rng.integers(1, n + 1, 30), rng.integers(1, n + 1, 30))})
+    files.append(("seeded_9", "%d %d %d\n" % (n, n, len(ent)) + "".join("%d %d %g\n" % (r, c, 0.5 * (i + 1)) for i, (r, c) in enumerate(ent))))
+    cases = []
+    with tempfile.TemporaryDirectory() as d:
+        for name, text in files:
+            path = os.path.join(d, name + ".mtx")
+            with open(path, "w") as f:
+                f.write(text)
+            rec = {"name": name, "file": text}
+            for tag, sym in (("old", 0), ("sym", 1)):
+                r = orc.ref_mtx_load_other(path, sym)
+                rec[tag] = {"row_ptr": r["row_ptr"].tolist(), "col_ind": r["col_ind"].tolist(), "val": r["val"].tolist(),
+                            "bandwidth": r["bandwidth"], "text": r["text"]}
+            cases.append(rec)
+    with open(os.path.join(HERE, "mtx_other.json"), "w") as f:
+        json.dump({"note": "outputs of the reference's assemble_csr_matrix / assemble_simetric_csr_matrix / getBandwidth / printMatrix "
+                           "(csr_formatter.h:31-109, 146-183); printMatrix on the result with row_ptr[0] = 1", "cases": cases}, f, indent=1)
+
+
 def main():
     assert orc.have_ref(), "oracle/_ref/libmgg_ref.so is missing: run `make -C oracle` with the reference mounted"
     cases = []
@@ -124,6 +154,8 @@ def main():
     y = orc.ref_sag_ref(x, ptr, col)
     out["sag_ref"] = {"ptr": ptr.tolist(), "col": col.tolist(), "x_hex": x.tobytes().hex(), "y_hex": y.tobytes().hex(),
                       "shape": [40, 5]}
+
+    mtx_other()
 
     with open(os.path.join(HERE, "np_arrays.json"), "w") as f:
         json.dump(out, f, separators=(",", ":"))
