@@ -553,6 +553,24 @@ def gcn2_headline_only(args, torch, host, forward_stages, names):
             "detail": {"stage_ms": {n: round(v, 4) for n, v in r["stage_median"].items()}}}
 
 
+def paired_tables(torch, local, remote):
+    """The local and the remote feature table of an aggregation call as views into ONE device allocation (the remote table
+    256-byte aligned behind the local one).  How the library forms gather addresses -- 32-bit buffer offsets when both
+    tables lie inside one window of under 2 GiB, 64-bit addresses otherwise -- then follows from the table sizes and not
+    from where the allocator put two separate blocks: the same kernel variant in every run, under the profiler too.
+    `local` / `remote`: host arrays or device tensors.  -> (d_local, d_remote, block)"""
+    as_dev = lambda a: a if torch.is_tensor(a) else torch.from_numpy(np.ascontiguousarray(a))
+    local, remote = as_dev(local), as_dev(remote)
+    nl = local.numel() * local.element_size()
+    first = (nl + 255) & ~255
+    block = torch.empty(first + remote.numel() * remote.element_size(), dtype=torch.uint8, device="cuda")
+    d_l = block[:nl].view(local.dtype).view(local.shape)
+    d_r = block[first:].view(remote.dtype).view(remote.shape)
+    d_l.copy_(local)
+    d_r.copy_(remote)
+    return d_l, d_r, block
+
+
 def share_inputs(args, torch, host):
     """Rank 0's share of an 8-way partitioned RMAT graph (ids scrambled) with the remote rows pre-staged: host arrays,
     device tensors and the compactly staged remote table (one row per distinct remote id, most referenced first)."""
@@ -566,8 +584,7 @@ def share_inputs(args, torch, host):
     dev = "cuda"
     x_remote = host.fill_normal((num_gpus * npp, dim), seed=11)
     sh = dict(V=V, dim=dim, npp=npp, lb=lb, ub=ub, R=R, nnz=nnz, lp=lp, rp=rp, lc=lc, rc=rc, x_remote=x_remote)
-    sh["d_xr"] = torch.from_numpy(x_remote).to(dev)
-    sh["d_xl"] = torch.from_numpy(np.ascontiguousarray(x_remote[lb:ub])).to(dev)  # separate allocation
+    sh["d_xl"], sh["d_xr"], sh["tables"] = paired_tables(torch, x_remote[lb:ub], x_remote)  # the local rows are a table of their own
     sh["d"] = [torch.from_numpy(a).to(dev) if len(a) else torch.zeros(1, dtype=torch.int32, device=dev) for a in (lp, lc, rp, rc)]
     sh["d_out"] = torch.empty(R, dim, device=dev)
     return sh
@@ -583,7 +600,7 @@ def share_record(args, torch, host, with_cpu):
     lb, ub, dim, npp, R, nnz = sh["lb"], sh["ub"], sh["dim"], sh["npp"], sh["R"], sh["nnz"]
     nbytes = agg_bytes(nnz, R, dim, ptr_arrays=2)
 
-    def cold_leg(kn, col_r, table, want):
+    def cold_leg(kn, col_r, xl, table, want):
         """The same call with nothing of it left in the caches: each launch goes to the next of COLD_COPIES disjoint
         copies of everything the call touches (row pointers, column ids, both feature tables, the output, and -- a plan
         is keyed by its CSR's addresses -- its own descriptors and row offsets), so between two uses of a copy the others
@@ -591,7 +608,8 @@ def share_record(args, torch, host, with_cpu):
         n = COLD_COPIES
         sets = []
         for _ in range(n):
-            c = [t.clone() for t in (d[0], d[1], d[2], col_r, d_xl, table)]
+            c = [t.clone() for t in (d[0], d[1], d[2], col_r)]
+            c += list(paired_tables(torch, xl, table)[:2])
             c.append(torch.empty_like(d_out))
             sets.append(c)
         calls = [lambda c=c: host.mgg_SAG_np_div(c[6], c[4], c[0], c[1], c[2], c[3], lb, ub, dim, npp, 0, kn.ps, kn.wpb, kn.dist,
@@ -629,12 +647,12 @@ def share_record(args, torch, host, with_cpu):
         del sets, calls
         return out
 
-    def measure(col_r, table, key):
-        search = lambda ps, blk, core: host.tune_np_div(d_out, d_xl, d[0], d[1], d[2], col_r, lb, ub, dim, npp, ps, input_remote=table,
+    def measure(col_r, xl, table, key):
+        search = lambda ps, blk, core: host.tune_np_div(d_out, xl, d[0], d[1], d[2], col_r, lb, ub, dim, npp, ps, input_remote=table,
                                                         col_block_rows=blk, core_rows=core)
 
         def timed(kn):
-            call = lambda: host.mgg_SAG_np_div(d_out, d_xl, d[0], d[1], d[2], col_r, lb, ub, dim, npp, 0, kn.ps, kn.wpb, kn.dist, input_remote=table,
+            call = lambda: host.mgg_SAG_np_div(d_out, xl, d[0], d[1], d[2], col_r, lb, ub, dim, npp, 0, kn.ps, kn.wpb, kn.dist, input_remote=table,
                                                col_block_rows=kn.blk, core_rows=kn.core)
             kn.observe(host, call)
             r = time_steps(torch, [call], ["agg"], args.steps, args.warmup)
@@ -645,11 +663,12 @@ def share_record(args, torch, host, with_cpu):
         gbps = nbytes / (ms * 1e-3) / 1e9
         rec = {"avg_launch_ms": round(ms, 4), "median_launch_ms": round(med, 4), "achieved": round(gbps, 1),
                "frac": round(gbps / HBM_PEAK_GBPS, 4), "knobs": str(kn) + (" (searched)" if args.tune else " (library rules, no search)"),
-               "kernel": host.last_agg_kernel().split(" grid")[0], **load_traffic(key, args, kn.blk, kn.core)}
+               "kernel": host.last_agg_kernel().split(" grid")[0] + (" (%s gather addressing)" % re.search(r"addr=(\w+)", host.last_agg_kernel()).group(1)),
+               **load_traffic(key, args, kn.blk, kn.core)}
         call()
         torch.cuda.synchronize()
         result = d_out.cpu().numpy()
-        rec["cold"] = cold_leg(kn, col_r, table, result)
+        rec["cold"] = cold_leg(kn, col_r, xl, table, result)
         rec["frac_cold"] = rec["cold"]["frac"]
         if not args.tune and not args.no_search:
             t0 = time.perf_counter()
@@ -661,7 +680,7 @@ def share_record(args, torch, host, with_cpu):
                                "frac": round(nbytes / (ms_s * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "rules_over_searched": round(ms / ms_s, 4)}
         return rec, result
 
-    glob, out_glob = measure(d[3], d_xr, "share_agg")
+    glob, out_glob = measure(d[3], d_xl, d_xr, "share_agg")
     # compact staging: distinct remote ids most referenced first, column array rewritten, rows gathered into a small table
     host.compact_remote_device(d[3], len(sh["rc"]))  # first use: scratch allocation
     torch.cuda.synchronize()
@@ -669,10 +688,10 @@ def share_record(args, torch, host, with_cpu):
     d_rcc, d_ids = host.compact_remote_device(d[3], len(sh["rc"]))
     torch.cuda.synchronize()
     compaction_ms = (time.perf_counter() - t0) * 1e3
-    d_xc = torch.empty(len(d_ids), dim, device="cuda", dtype=d_xr.dtype)
+    d_xl2, d_xc, _block = paired_tables(torch, d_xl, torch.empty(len(d_ids), dim, device="cuda", dtype=d_xr.dtype))
     stage = lambda: host.gather_rows(d_xc, d_xr, d_ids, len(d_ids), dim * 4)
     rs = time_steps(torch, [stage], ["stage"], args.steps, 2)
-    comp, out_comp = measure(d_rcc, d_xc, "share_agg_compact")
+    comp, out_comp = measure(d_rcc, d_xl2, d_xc, "share_agg_compact")
     comp.update({"distinct_remote_rows": int(len(d_ids)), "table_bytes": int(len(d_ids)) * dim * 4,
                  "setup_ms": {"compaction_on_gpu_once_per_graph": round(compaction_ms, 2),
                               "staging_gather_per_layer": round(rs["stage_median"]["stage"], 4)},

@@ -73,6 +73,13 @@ int mggx_set_stream(void *hip_stream);
 int mggx_sync(void);
 int mggx_malloc(void **d_ptr, size_t bytes);
 int mggx_free(void *d_ptr);
+/* The two feature tables of an aggregation call (this rank's rows; the rows the reference reaches with remote GETs) out
+ * of ONE allocation, the remote table right behind the local one (256-byte aligned).  Where the two tables of a call lie
+ * is what decides how mggx_sag_np_div forms gather addresses: inside one window of under 2 GiB it uses 32-bit buffer
+ * offsets, otherwise 64-bit addresses -- same sums, but two kernel variants.  With tables from this call the variant
+ * is a function of their sizes, not of where an allocator happened to put two separate blocks.  Free with
+ * mggx_free(*d_local); *d_remote is an interior pointer and must not be freed on its own. */
+int mggx_malloc_tables(void **d_local, size_t local_bytes, void **d_remote, size_t remote_bytes);
 int mggx_memset(void *d_ptr, int value, size_t bytes);
 int mggx_memcpy_h2d(void *d_dst, const void *src, size_t bytes);
 int mggx_memcpy_d2h(void *dst, const void *d_src, size_t bytes);

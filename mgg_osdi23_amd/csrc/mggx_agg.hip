@@ -40,6 +40,21 @@ namespace {
 #ifndef MGGX_BATCH
 #define MGGX_BATCH 8
 #endif
+// Build-time experiment switches (both 0 in the library): a floor on the wavefronts per SIMD the compiler must leave room
+// for in k_agg's register budget, and extra dynamic LDS per workgroup (limits how many workgroups a CU holds).
+#ifndef MGGX_AGG_WAVES_PER_EU
+#define MGGX_AGG_WAVES_PER_EU 0
+#endif
+#ifndef MGGX_AGG_LDS_PAD
+#define MGGX_AGG_LDS_PAD 0
+#endif
+#if MGGX_AGG_WAVES_PER_EU > 0
+#define MGGX_AGG_OCCUPANCY __attribute__((amdgpu_waves_per_eu(MGGX_AGG_WAVES_PER_EU)))
+#elif defined(MGGX_AGG_NUM_VGPR)
+#define MGGX_AGG_OCCUPANCY __attribute__((amdgpu_num_vgpr(MGGX_AGG_NUM_VGPR)))
+#else
+#define MGGX_AGG_OCCUPANCY
+#endif
 
 constexpr int HDR_VALID = 1;   // entry holds a partial row
 constexpr int HDR_ENDS = 2;    // head entry: the row ends inside this unit
@@ -63,6 +78,8 @@ struct AggArgs {
     float *c_val;  // [2 * workgroups][cpad]
     long long ld_in, ld_out;
     int num_parts;
+    const int *num_parts_dev; // when set: the descriptor count is read from here (it was made on the device and never copied back;
+                              // num_parts is then a host-side upper bound that sizes the grid)
     int nnz_l, nnz_r;
     const int *nnz_l_dev;     // when set: the local edge count is read from here (a caller that may not copy it to the host)
     int lb, dim, ps, dist, cpad;
@@ -315,7 +332,7 @@ __device__ __forceinline__ void finish_row(const AggArgs &a, int row, int l, con
 // One wavefront-wide aggregation kernel; see the file header for the scheme.
 // Dynamic LDS: int2 hdr[2*wpb] (head, tail per wavefront), then float vals[2*wpb][cpad].
 template <int LPR, int MODE, bool BUF, bool SMX>
-__global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
+__global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a)
 {
     constexpr int NV = ModeTraits<MODE>::NV;
     constexpr int S = 64 / LPR;
@@ -332,6 +349,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     constexpr int STAGE = LPR >= 4 ? 4 : LPR == 2 ? 2 : 1;
     extern __shared__ float lds[];
     if (gate_closed(a.gate)) return;
+    const int num_parts = a.num_parts_dev ? *a.num_parts_dev : a.num_parts;
 
     const int lane = lane_id();
     const int wave = (int)(threadIdx.x >> 6);
@@ -378,7 +396,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     // A slot's descriptor, or an empty one (no row, no neighbors) past the end of the plan or of this wavefront's rounds.
     auto load_desc = [&](long long q, bool in_range) -> int4 {
         int4 d = make_int4(0, -1, 0, 0);
-        if (in_range && q < a.num_parts) {
+        if (in_range && q < num_parts) {
             if constexpr (STREAM) {
                 typedef int v4i_a __attribute__((ext_vector_type(4)));
                 const v4i_a dv = __builtin_nontemporal_load(reinterpret_cast<const v4i_a *>(a.desc + q));
@@ -466,7 +484,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
     int *st_ids = reinterpret_cast<int *>(lds + a.stage_off) + (size_t)wpb * (nst * S * 4) + (size_t)wave * (nst * S * CH);
 
     for (int j0 = 0; j0 < a.dist; j0 += nst) {
-        if (q_wave + (long long)j0 * S >= a.num_parts) break;
+        if (q_wave + (long long)j0 * S >= num_parts) break;
         {
             int4 dd[STAGE];
             int idv[STAGE][IPL];
@@ -497,9 +515,9 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
         const int j = j0 + u;
         if (j >= a.dist) break;
         const long long q0 = q_wave + (long long)j * S;
-        if (q0 >= a.num_parts) break;
+        if (q0 >= num_parts) break;
         const long long q = q0 + slot;
-        const bool pv = q < a.num_parts;
+        const bool pv = q < num_parts;
         const int4 d = st_desc[u * S + slot];
 
         // carried partial row of the previous round: slot S-1 -> slot 0
@@ -575,7 +593,7 @@ __global__ void __launch_bounds__(1024) k_agg(const AggArgs a)
         }
         const bool run_last = pv && nrow != row;
         const bool row_done = ((unsigned)d.z & DESC_LAST) != 0;
-        const bool last_round = (j == a.dist - 1) || (q0 + S >= a.num_parts);
+        const bool last_round = (j == a.dist - 1) || (q0 + S >= num_parts);
         bool keep_open = false;
         if (run_last) {
             if (row_done && has_first) {
@@ -876,6 +894,7 @@ struct FixedScratch {
     unsigned char *ptr;
     size_t bytes;
     const int *nnz_l_dev;
+    const int *num_parts_dev;  // NULL: the plan's own count is exact
 };
 
 // The dense core's side of a call, handed to the aggregation of the remaining CSR: where a column-blocked plan ends in
@@ -963,12 +982,13 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     a.ld_in = ld_in;
     a.ld_out = blocked ? ldp : ld_out;
     a.num_parts = plan->num_parts;
+    a.num_parts_dev = fixed ? fixed->num_parts_dev : nullptr;
     a.nnz_l = (int)plan->nnz_l;
     a.nnz_r = (int)plan->nnz_r;
     a.nnz_l_dev = fixed ? fixed->nnz_l_dev : nullptr;
     a.lb = lb;
     a.dim = dim;
-    a.ps = plan->ps;
+    a.ps = plan->unit;  // what a slot sums at a time: whole partitions of one row, at most max(ps, 16) neighbors
     a.dist = dist;
     a.cpad = cpad;
     a.parts_per_wg = (int)parts_per_wg;
@@ -1037,7 +1057,7 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         const size_t carry_lds = ((size_t)wpb * 2 * sizeof(int2) + (size_t)wpb * 2 * cpad * sizeof(float) + 15) & ~(size_t)15;
         a.stage_off = (int)(carry_lds / sizeof(float));
         a.stage_rounds = stage;
-        const size_t lds_bytes = carry_lds + (size_t)wpb * stage * round_bytes;
+        const size_t lds_bytes = carry_lds + (size_t)wpb * stage * round_bytes + (size_t)MGGX_AGG_LDS_PAD;
         if (lds_bytes > (160u << 10)) return fail(MGGX_ELIMIT, "aggregation: %zu bytes of LDS per workgroup (wpb %d, dim %d)", lds_bytes, wpb, dim);
         const dim3 grid((unsigned)num_wg), block((unsigned)(64 * wpb));
         const bool smx = (a.flags & MGGX_AGG_SOFTMAX) != 0;  // fp32 tables only (checked above)
@@ -1090,8 +1110,8 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
             MGGX_LAUNCH_CHECK("k_agg_tail");
         }
     }
-    snprintf(st.last_kernel, sizeof(st.last_kernel), "k_agg<%d,%d,%d> grid=%lld block=%d parts=%d blocks=%d ps=%d wpb=%d dist=%d", lpr, mode, (int)buf,
-             num_wg, 64 * wpb, plan->num_parts, plan->blocks, plan->ps, wpb, dist);
+    snprintf(st.last_kernel, sizeof(st.last_kernel), "k_agg<%d,%d,%d> grid=%lld block=%d parts=%d blocks=%d ps=%d wpb=%d dist=%d addr=%s", lpr, mode, (int)buf,
+             num_wg, 64 * wpb, plan->num_parts, plan->blocks, plan->ps, wpb, dist, buf ? "buffer32" : "flat64");
     return MGGX_OK;
 }
 
@@ -1460,25 +1480,34 @@ MGGX_EXPORT int mggx_sag_parts_static(float *d_out, const float *d_in, const int
     unsigned char *base = nullptr;
     rc = mggx::static_scratch_ptr(&base);
     if (rc) return rc;
-    // layout of the scratch: descriptors | first descriptor of each row | carry buffer (sized by run_agg)
+    // layout of the scratch: descriptors | first descriptor of each row | [scratch of the unit builder, ps < 16] | carry
+    // buffer (sized by run_agg)
     const auto pad = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    const bool grouped = mggx::unit_of(ps) != ps;
     const size_t desc_bytes = pad(sizeof(int4) * (size_t)num_parts), off_bytes = pad(sizeof(int) * ((size_t)num_nodes + 1));
-    if (desc_bytes + off_bytes >= (size_t)MGGX_STATIC_SCRATCH_BYTES)
+    const size_t tmp_bytes = grouped ? pad(sizeof(int) * mggx::explicit_tmp_ints(num_nodes)) : 0;
+    if (desc_bytes + off_bytes + tmp_bytes >= (size_t)MGGX_STATIC_SCRATCH_BYTES)
         return fail(MGGX_ELIMIT, "sag_parts_static: %d partitions over %d rows need %zu bytes of descriptors; the static scratch holds %zu",
-                    num_parts, num_nodes, desc_bytes + off_bytes, (size_t)MGGX_STATIC_SCRATCH_BYTES);
+                    num_parts, num_nodes, desc_bytes + off_bytes + tmp_bytes, (size_t)MGGX_STATIC_SCRATCH_BYTES);
     mggx::Plan plan;  // lives for this call only; its arrays are views into the scratch
     plan.d_ptr_l = d_row_ptr;
     plan.d_part_ptr = d_part_ptr;
     plan.d_part2node = d_part2node;
     plan.rows = plan.real_rows = num_nodes;
     plan.ps = ps;
-    plan.num_parts = num_parts;
+    plan.unit = mggx::unit_of(ps);
+    plan.caller_parts = num_parts;
     plan.d_desc = reinterpret_cast<int4 *>(base);
     plan.d_off = reinterpret_cast<int *>(base + desc_bytes);
     plan.nnz_l = 1;  // "has local edges"; the kernels read the count itself from d_row_ptr[num_nodes]
-    rc = mggx::explicit_desc_fill(d_row_ptr, d_part_ptr, d_part2node, num_nodes, num_parts, ps, plan.d_desc, plan.d_off);
+    long long bound = num_parts;
+    rc = mggx::explicit_desc_fill(d_row_ptr, d_part_ptr, d_part2node, num_nodes, num_parts, ps, plan.d_desc, plan.d_off,
+                                  reinterpret_cast<int *>(base + desc_bytes + off_bytes), &bound);
     if (rc) return rc;
-    const mggx::FixedScratch fx{base + desc_bytes + off_bytes, (size_t)MGGX_STATIC_SCRATCH_BYTES - desc_bytes - off_bytes, d_row_ptr + num_nodes};
+    // ps < 16: several partitions per descriptor; their number stays on the device (d_off[rows]) and the grid is sized by a bound
+    plan.num_parts = (int)bound;
+    const size_t used = desc_bytes + off_bytes + tmp_bytes;
+    const mggx::FixedScratch fx{base + used, (size_t)MGGX_STATIC_SCRATCH_BYTES - used, d_row_ptr + num_nodes, grouped ? plan.d_off + num_nodes : nullptr};
     mggx_agg_opts o{};
     o.flags = MGGX_AGG_ACCUMULATE;
     return mggx::run_agg(&plan, d_out, d_in, nullptr, d_col, nullptr, lowbound, dim, wpb, dist, o, mggx::Gate{}, &fx);

@@ -11,6 +11,7 @@
 #include <chrono>
 #include <cmath>
 #include <new>
+#include <type_traits>
 
 #include <rocprim/device/device_radix_sort.hpp>
 
@@ -21,6 +22,29 @@ namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned short us4 __attribute__((ext_vector_type(4)));
+
+#ifndef MGGX_CORE_WAVES_PER_EU
+#define MGGX_CORE_WAVES_PER_EU 0
+#endif
+#if MGGX_CORE_WAVES_PER_EU > 0
+#define MGGX_CORE_OCCUPANCY __attribute__((amdgpu_waves_per_eu(MGGX_CORE_WAVES_PER_EU)))
+#elif defined(MGGX_CORE_NUM_VGPR)
+#define MGGX_CORE_OCCUPANCY __attribute__((amdgpu_num_vgpr(MGGX_CORE_NUM_VGPR)))
+#else
+#define MGGX_CORE_OCCUPANCY
+#endif
+#ifndef MGGX_CORE_READS
+#define MGGX_CORE_READS 8  // LDS reads of one list entry issued back to back (see core_sell_body)
+#endif
+
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for_core(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for_core<I + 1, N>(f);
+    }
+}
 
 constexpr int CORE_TC = 256;    // core columns per LDS tile
 constexpr int CORE_WAVES = CORE_GROUP_ROWS / 64;  // slices (of 64 rows) per workgroup: as small as the aggregation's own
@@ -77,17 +101,15 @@ __device__ __forceinline__ void core_sell_body(const unsigned *__restrict__ blk_
             for (int j = 0; j < 4; ++j) {
                 const int c = cur[j];
                 const v4f *q = tile + (c < TC ? c : TC);
-                // at most eight LDS reads in flight per entry: wide rows otherwise cost a wavefront a hundred registers, and
-                // this kernel shares each SIMD's register file with the aggregation running beside it
-                constexpr int H = NS > 8 ? (NS + 1) / 2 : NS;
+                // at most MGGX_CORE_READS LDS reads in flight per entry: wide rows otherwise cost a wavefront a hundred
+                // registers, and this kernel shares each SIMD's register file with the aggregation running beside it
+                constexpr int GROUPS = (NS + MGGX_CORE_READS - 1) / MGGX_CORE_READS, H = (NS + GROUPS - 1) / GROUPS;
+                static_for_core<0, GROUPS>([&](auto gg) {
+                    constexpr int s0 = decltype(gg)::value * H, s1 = s0 + H < NS ? s0 + H : NS;
 #pragma unroll
-                for (int s = 0; s < H; ++s) acc[s] += q[s * TP];
-                if constexpr (H < NS) {
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int s = H; s < NS; ++s) acc[s] += q[s * TP];
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+                    for (int s = s0; s < s1; ++s) acc[s] += q[s * TP];
+                    if constexpr (GROUPS > 1) __builtin_amdgcn_sched_barrier(0);
+                });
             }
             cur = nxt;
             ++pos;
@@ -105,7 +127,7 @@ __device__ __forceinline__ void core_sell_body(const unsigned *__restrict__ blk_
 // launch has no tail of a few heavy ones.
 // partial[(slot * CORE_WAVES * 64 + row in the group) * N4 + s]
 template <int N4, bool SPLIT>
-__global__ void __launch_bounds__(CORE_WAVES * 64) k_core_sell(const unsigned *__restrict__ blk_off, const unsigned short *__restrict__ idx,
+__global__ void __launch_bounds__(CORE_WAVES * 64) MGGX_CORE_OCCUPANCY k_core_sell(const unsigned *__restrict__ blk_off, const unsigned short *__restrict__ idx,
                                                                const v4f *__restrict__ tab, v4f *__restrict__ partial,
                                                                const int4 *__restrict__ wgs, int core, int ntiles, const Gate gate)
 {

@@ -90,9 +90,16 @@ struct Plan {
     const int *d_part_ptr = nullptr;   // explicit-partition plans only
     const int *d_part2node = nullptr;  // explicit-partition plans only
     int rows = 0;
-    int ps = 0;
+    int ps = 0;                  // the caller's partition size (MGG's partSize)
+    int caller_parts = 0;        // explicit-partition plans: the caller's partition count (part of the cache key)
+    // What a slot of the kernel sums at a time: for ps >= 16 one partition; for smaller ps the largest whole number of
+    // consecutive partitions of one row and side with at most 16 neighbors between them (unit = ps * floor(16 / ps)
+    // neighbors).  Consecutive partitions of a row are consecutive edges, so such a group is one edge range: one
+    // descriptor and one slot instead of up to 16, each one sixteenth full.  The reference's kernel only ever sees
+    // dist * ps neighbors per warp (neighbor_utils.cuh:1395-1398); the summation order stays a function of the knobs.
+    int unit = 0;
     // contents (device)
-    int4 *d_desc = nullptr;      // [num_parts]
+    int4 *d_desc = nullptr;      // [num_parts] one per unit
     int *d_off = nullptr;        // [rows+1] first descriptor of each row
     int *d_empty_rows = nullptr; // rows without any partition
     int num_parts = 0;
@@ -235,8 +242,19 @@ int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, i
 int graph_info(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_l, const int *d_col_r, int rows, bool internal, GraphInfo **out);
 int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows,
                       int num_parts, int ps, Plan **out);
+// Neighbors per kernel slot for a partition size (see Plan::unit).
+inline int unit_of(int ps) { return ps >= 16 ? ps : ps * (16 / ps); }
+// Explicit partition arrays -> unit descriptors and the first unit of each row, into caller-provided device arrays, with
+// kernels on the library's stream only.  Partitions per unit g = unit_of(ps) / ps.  g == 1: one descriptor per partition,
+// d_tmp unused.  g > 1: d_tmp holds explicit_tmp_ints(rows) ints of scratch; the number of units stays on the device
+// (d_off[rows]) and *units_bound receives a host-side upper bound for it.
+size_t explicit_tmp_ints(int rows);
 int explicit_desc_fill(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows, int num_parts, int ps,
-                       int4 *d_desc, int *d_off);
+                       int4 *d_desc, int *d_off, int *d_tmp, long long *units_bound);
+// d_out[0..n] = exclusive prefix sum of d_in[0..n) with caller-provided scratch of scan_tmp_bytes(n) bytes: three kernels on
+// the library's stream, no allocation, no copy, no synchronisation (the total is d_out[n])
+size_t scan_tmp_bytes(int n);
+int exclusive_scan_i32_device(const int *d_in, int *d_out, int n, void *d_tmp);
 // Device address of the static scratch array of mggx_sag_parts_static on the current device.
 int static_scratch_ptr(unsigned char **out);
 void plan_free(Plan *p);

@@ -201,6 +201,34 @@ __global__ void __launch_bounds__(256) k_desc_from_parts(const int *__restrict__
     desc[q] = make_int4(beg, r, (int)z, 0);
 }
 
+// Explicit plans with several partitions per unit (ps < 16).  cnt[r] = units of row r = ceil(partitions of r / g).
+__global__ void __launch_bounds__(256) k_units_per_row(const int *__restrict__ off_p, int rows, int g, int *__restrict__ cnt)
+{
+    const int r = blockIdx.x * 256 + threadIdx.x;
+    if (r >= rows) return;
+    cnt[r] = (off_p[r + 1] - off_p[r] + g - 1) / g;
+}
+
+// One descriptor per unit: unit j of row r spans the partitions off_p[r] + j g .. (at most g of them, to the end of the row),
+// which build_part lays out as consecutive edge ranges of ps neighbors -- one edge range from the first one's start.
+// Threads past the device-side unit count off_u[rows] (the grid is sized by a host-side bound) do nothing.
+__global__ void __launch_bounds__(256) k_desc_from_units(const int *__restrict__ row_ptr, const int *__restrict__ part_ptr,
+                                                         const int *__restrict__ off_p, const int *__restrict__ off_u, int rows, int ps,
+                                                         int g, int4 *__restrict__ desc)
+{
+    const int q = blockIdx.x * 256 + threadIdx.x;
+    if (q >= off_u[rows]) return;
+    const int r = row_of_part(off_u, rows, q);
+    const int j = q - off_u[r];
+    const int p0 = off_p[r] + j * g;
+    const int np = min(g, off_p[r + 1] - p0);
+    const int beg = part_ptr[p0];
+    unsigned z = (unsigned)max(0, min(np * ps, row_ptr[r + 1] - beg));
+    if (j == 0) z |= DESC_FIRST;
+    if (q == off_u[r + 1] - 1) z |= DESC_LAST;
+    desc[q] = make_int4(beg, r, (int)z, 0);
+}
+
 // off[r] for explicit plans: first descriptor of row r = lower bound of r in part2node
 __global__ void __launch_bounds__(256) k_off_from_parts(const int *__restrict__ part2node, int num_parts, int rows,
                                                         int *__restrict__ off)
@@ -484,6 +512,25 @@ int stale_poll()
                              "plan was dropped; call again (and mggx_forget() before rewriting or freeing cached arrays)", (const void *)arrs[0]);
 }
 
+size_t scan_tmp_bytes(int n)
+{
+    const size_t tiles = ((size_t)std::max(n, 1) + SCAN_TILE - 1) / SCAN_TILE;
+    return sizeof(long long) * (tiles + 1);
+}
+
+int exclusive_scan_i32_device(const int *d_in, int *d_out, int n, void *d_tmp)
+{
+    State &s = state();
+    if (n <= 0) return fail(MGGX_EINVAL, "exclusive_scan: empty input");
+    const int tiles = (n + SCAN_TILE - 1) / SCAN_TILE;
+    long long *d_tile = static_cast<long long *>(d_tmp);
+    k_scan_tile_sums<<<tiles, SCAN_THREADS, 0, s.stream>>>(d_in, n, d_tile);
+    k_scan_tile_offsets<<<1, SCAN_THREADS, 0, s.stream>>>(d_tile, tiles);
+    k_scan_apply<<<tiles, SCAN_THREADS, 0, s.stream>>>(d_in, d_out, n, d_tile);
+    MGGX_LAUNCH_CHECK("exclusive scan");
+    return MGGX_OK;
+}
+
 int exclusive_scan_i32(const int *d_in, int *d_out, int n, long long *total_host)
 {
     State &s = state();
@@ -639,6 +686,8 @@ int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int row
     p->rows = rows;
     p->real_rows = rows;
     p->ps = ps;
+    p->unit = unit_of(ps);
+    const int unit = p->unit;  // neighbors per descriptor: whole partitions of one row and side, at most 16 neighbors (ps < 16)
     int rc = MGGX_OK;
     int *d_cnt = nullptr;
     do {
@@ -648,7 +697,7 @@ int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int row
             break;
         }
         if (rows > 0)
-            k_count_parts<<<(rows + 255) / 256, 256, 0, s.stream>>>(d_ptr_l, d_ptr_l + 1, d_ptr_r, d_ptr_r ? d_ptr_r + 1 : nullptr, rows, ps,
+            k_count_parts<<<(rows + 255) / 256, 256, 0, s.stream>>>(d_ptr_l, d_ptr_l + 1, d_ptr_r, d_ptr_r ? d_ptr_r + 1 : nullptr, rows, unit,
                                                                     d_cnt);
         long long total = 0;
         rc = exclusive_scan_i32(d_cnt, p->d_off, rows, &total);
@@ -690,7 +739,7 @@ int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int row
         }
         if (p->num_parts > 0) {
             k_fill_desc<<<(p->num_parts + 255) / 256, 256, 0, s.stream>>>(p->d_off, d_ptr_l, d_ptr_l + 1, d_ptr_r,
-                                                                          d_ptr_r ? d_ptr_r + 1 : nullptr, rows, ps, p->num_parts,
+                                                                          d_ptr_r ? d_ptr_r + 1 : nullptr, rows, unit, p->num_parts,
                                                                           p->d_desc);
             if (hipGetLastError() != hipSuccess) {
                 rc = fail(MGGX_EHIP, "plan: descriptor kernel launch failed");
@@ -709,16 +758,38 @@ int plan_get(const int *d_ptr_l, const int *d_ptr_r, const int *d_col_r, int row
     return MGGX_OK;
 }
 
-// Descriptors and row offsets of explicit partition arrays into caller-provided device arrays (two kernels on the
-// library's stream, nothing else).
+size_t explicit_tmp_ints(int rows)
+{
+    // first partition of each row | units per row | scan scratch
+    return 2 * ((size_t)rows + 1) + (scan_tmp_bytes(rows) + sizeof(int) - 1) / sizeof(int) + 2;
+}
+
+// Descriptors and row offsets of explicit partition arrays into caller-provided device arrays (kernels on the library's
+// stream, nothing else).
 int explicit_desc_fill(const int *d_row_ptr, const int *d_part_ptr, const int *d_part2node, int rows, int num_parts, int ps,
-                       int4 *d_desc, int *d_off)
+                       int4 *d_desc, int *d_off, int *d_tmp, long long *units_bound)
 {
     State &s = state();
-    k_off_from_parts<<<(rows + 1 + 255) / 256, 256, 0, s.stream>>>(d_part2node, num_parts, rows, d_off);
-    if (num_parts > 0)
-        k_desc_from_parts<<<(num_parts + 255) / 256, 256, 0, s.stream>>>(d_row_ptr, d_part_ptr, d_part2node, num_parts, ps, d_desc);
-    if (hipGetLastError() != hipSuccess) return fail(MGGX_EHIP, "plan: explicit descriptor kernel launch failed");
+    const int g = unit_of(ps) / ps;
+    if (g <= 1 || rows <= 0 || num_parts <= 0) {
+        k_off_from_parts<<<(rows + 1 + 255) / 256, 256, 0, s.stream>>>(d_part2node, num_parts, rows, d_off);
+        if (num_parts > 0)
+            k_desc_from_parts<<<(num_parts + 255) / 256, 256, 0, s.stream>>>(d_row_ptr, d_part_ptr, d_part2node, num_parts, ps, d_desc);
+        if (hipGetLastError() != hipSuccess) return fail(MGGX_EHIP, "plan: explicit descriptor kernel launch failed");
+        if (units_bound) *units_bound = num_parts;
+        return MGGX_OK;
+    }
+    int *off_p = d_tmp, *cnt = d_tmp + ((size_t)rows + 1);
+    long long *scan_tmp = reinterpret_cast<long long *>((reinterpret_cast<uintptr_t>(cnt + rows + 1) + 7) & ~(uintptr_t)7);
+    k_off_from_parts<<<(rows + 1 + 255) / 256, 256, 0, s.stream>>>(d_part2node, num_parts, rows, off_p);
+    k_units_per_row<<<(rows + 255) / 256, 256, 0, s.stream>>>(off_p, rows, g, cnt);
+    const int rc = exclusive_scan_i32_device(cnt, d_off, rows, scan_tmp);
+    if (rc) return rc;
+    // every row with partitions has at most (its partitions / g) + 1 units, and at most `rows` rows have any
+    const long long bound = std::min<long long>(num_parts, (long long)num_parts / g + std::min(rows, num_parts));
+    k_desc_from_units<<<(unsigned)((bound + 255) / 256), 256, 0, s.stream>>>(d_row_ptr, d_part_ptr, off_p, d_off, rows, ps, g, d_desc);
+    if (hipGetLastError() != hipSuccess) return fail(MGGX_EHIP, "plan: explicit unit kernel launch failed");
+    if (units_bound) *units_bound = bound;
     return MGGX_OK;
 }
 
@@ -729,7 +800,7 @@ int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_
     for (size_t i = 0; i < s.plans.size(); ++i) {
         const Plan *p = s.plans[i];
         if (p->d_ptr_l == d_row_ptr && p->d_part_ptr == d_part_ptr && p->d_part2node == d_part2node && p->rows == rows &&
-            p->ps == ps && p->num_parts == num_parts) {
+            p->ps == ps && p->caller_parts == num_parts) {
             *out = cache_hit(i);
             return MGGX_OK;
         }
@@ -743,22 +814,29 @@ int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_
     p->rows = rows;
     p->real_rows = rows;
     p->ps = ps;
+    p->unit = unit_of(ps);
+    p->caller_parts = num_parts;
     p->num_parts = num_parts;
     int rc = MGGX_OK;
+    int *d_tmp = nullptr;
     do {
+        long long bound = num_parts;
         if (hipMalloc((void **)&p->d_off, sizeof(int) * ((size_t)rows + 1)) != hipSuccess ||
-            hipMalloc((void **)&p->d_desc, sizeof(int4) * (size_t)std::max(num_parts, 1)) != hipSuccess) {
+            hipMalloc((void **)&p->d_desc, sizeof(int4) * (size_t)std::max(num_parts, 1)) != hipSuccess ||
+            (p->unit != ps && hipMalloc((void **)&d_tmp, sizeof(int) * explicit_tmp_ints(rows)) != hipSuccess)) {
             rc = fail(MGGX_ENOMEM, "plan: explicit arrays");
             break;
         }
-        rc = explicit_desc_fill(d_row_ptr, d_part_ptr, d_part2node, rows, num_parts, ps, p->d_desc, p->d_off);
+        rc = explicit_desc_fill(d_row_ptr, d_part_ptr, d_part2node, rows, num_parts, ps, p->d_desc, p->d_off, d_tmp, &bound);
         if (rc) break;
-        int end = 0;
+        int end = 0, units = num_parts;
         if (rows > 0 && (hipStreamSynchronize(s.stream) != hipSuccess ||
-                         hipMemcpy(&end, d_row_ptr + rows, sizeof(int), hipMemcpyDeviceToHost) != hipSuccess)) {
+                         hipMemcpy(&end, d_row_ptr + rows, sizeof(int), hipMemcpyDeviceToHost) != hipSuccess ||
+                         hipMemcpy(&units, p->d_off + rows, sizeof(int), hipMemcpyDeviceToHost) != hipSuccess)) {
             rc = fail(MGGX_EHIP, "plan: reading edge count");
             break;
         }
+        p->num_parts = rows > 0 ? units : 0;  // several partitions of a row per descriptor when ps < 16 (Plan::unit)
         p->nnz_l = end;
         rc = plan_finish(p);
         if (rc) break;
@@ -773,6 +851,7 @@ int plan_get_explicit(const int *d_row_ptr, const int *d_part_ptr, const int *d_
         p->guard.want_l = end;
         rc = guard_arm(p->guard);
     } while (0);
+    if (d_tmp) (void)hipFree(d_tmp);
     if (rc) {
         plan_free(p);
         return rc;
@@ -805,6 +884,8 @@ int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, i
     p->d_col_l = d_col_l;
     p->real_rows = rows;
     p->ps = ps;
+    p->unit = unit_of(ps);
+    const int unit = p->unit;
     p->block_rows = block_rows;
     p->block_lb = lb;
     int rc = MGGX_OK;
@@ -838,7 +919,7 @@ int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, i
         }
         k_block_bounds<<<(unsigned)((vrows + rows + 255) / 256), 256, 0, s.stream>>>(d_ptr_l, d_col_l, rows, lb, block_rows, (int)blocks,
                                                                                    d_vbeg);
-        k_count_parts<<<(unsigned)((vrows + 255) / 256), 256, 0, s.stream>>>(d_vbeg, d_vbeg + rows, nullptr, nullptr, (int)vrows, ps, d_cnt);
+        k_count_parts<<<(unsigned)((vrows + 255) / 256), 256, 0, s.stream>>>(d_vbeg, d_vbeg + rows, nullptr, nullptr, (int)vrows, unit, d_cnt);
         long long total = 0;
         rc = exclusive_scan_i32(d_cnt, p->d_off, (int)vrows, &total);
         if (rc) break;
@@ -854,7 +935,7 @@ int plan_get_blocked(const int *d_ptr_l, const int *d_col_l, int rows, int lb, i
             break;
         }
         if (p->num_parts > 0) {
-            k_fill_desc<<<(p->num_parts + 255) / 256, 256, 0, s.stream>>>(p->d_off, d_vbeg, d_vbeg + rows, nullptr, nullptr, (int)vrows, ps,
+            k_fill_desc<<<(p->num_parts + 255) / 256, 256, 0, s.stream>>>(p->d_off, d_vbeg, d_vbeg + rows, nullptr, nullptr, (int)vrows, unit,
                                                                           p->num_parts, p->d_desc);
             if (hipGetLastError() != hipSuccess) {
                 rc = fail(MGGX_EHIP, "plan: descriptor kernel launch failed");

@@ -1,5 +1,6 @@
 // Runtime half of libmggx.so: device selection, stream, memory, timers, the
 // library-owned workspace and small utility kernels.
+#include <algorithm>
 #include <cstdio>
 #include <cstring>
 
@@ -113,6 +114,21 @@ MGGX_EXPORT int mggx_malloc(void **d_ptr, size_t bytes)
     *d_ptr = nullptr;
     hipError_t e = hipMalloc(d_ptr, bytes ? bytes : 1);
     if (e != hipSuccess) return fail(MGGX_ENOMEM, "malloc of %zu bytes: %s", bytes, hipGetErrorString(e));
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_malloc_tables(void **d_local, size_t local_bytes, void **d_remote, size_t remote_bytes)
+{
+    if (!d_local || !d_remote) return fail(MGGX_EINVAL, "malloc_tables: NULL result pointer");
+    int rc = mggx::ensure_init();
+    if (rc) return rc;
+    *d_local = *d_remote = nullptr;
+    const size_t first = (std::max<size_t>(local_bytes, 1) + 255) & ~(size_t)255;
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, first + std::max<size_t>(remote_bytes, 1));
+    if (e != hipSuccess) return fail(MGGX_ENOMEM, "malloc_tables of %zu + %zu bytes: %s", local_bytes, remote_bytes, hipGetErrorString(e));
+    *d_local = p;
+    *d_remote = static_cast<char *>(p) + first;
     return MGGX_OK;
 }
 

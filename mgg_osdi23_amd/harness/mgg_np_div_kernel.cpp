@@ -16,8 +16,16 @@ int main(int argc, char *argv[])
 
     // Feature tables: ones, as the reference fills its inputs (:122).  The staged table stands for the
     // symmetric buffers of all ranks back to back; this rank's own rows sit in a separate allocation.
-    float *d_table = device_filled((size_t)a.num_GPUs * s.nodesPerPE * dim, 1.0f);
-    float *d_local = device_filled((size_t)s.nodesPerPE * dim, 1.0f);
+    // Both come out of one allocation (mggx_malloc_tables), so the kernel variant the aggregation picks -- 32-bit buffer
+    // offsets inside one window, or 64-bit addresses -- follows from the table sizes and is the same in every run.
+    const size_t table_count = (size_t)a.num_GPUs * s.nodesPerPE * dim, local_count = (size_t)s.nodesPerPE * dim;
+    float *d_table = nullptr, *d_local = nullptr;
+    MGG_CHECK(mggx_malloc_tables((void **)&d_local, local_count * sizeof(float), (void **)&d_table, table_count * sizeof(float)));
+    {
+        const std::vector<float> ones(table_count, 1.0f);
+        MGG_CHECK(mggx_memcpy_h2d(d_table, ones.data(), table_count * sizeof(float)));
+        MGG_CHECK(mggx_memcpy_h2d(d_local, ones.data(), local_count * sizeof(float)));
+    }
     float *dsp_out = device_filled((size_t)s.nodesPerPE * dim, 0.0f);
     mgg_stage_remote(d_table);
     mgg_options().accumulate = true;  // reference behaviour: every call adds into dsp_out

@@ -57,7 +57,7 @@ _lib = None
 # every symbol include/mggx.h declares
 EXPORTS = [
     "mggx_last_error", "mggx_version", "mggx_init", "mggx_device_name", "mggx_set_stream", "mggx_sync",
-    "mggx_malloc", "mggx_free", "mggx_memset", "mggx_memcpy_h2d", "mggx_memcpy_d2h", "mggx_memcpy_d2d",
+    "mggx_malloc", "mggx_malloc_tables", "mggx_free", "mggx_memset", "mggx_memcpy_h2d", "mggx_memcpy_d2h", "mggx_memcpy_d2d",
     "mggx_timer_create", "mggx_timer_start", "mggx_timer_stop", "mggx_timer_elapsed_ms", "mggx_timer_destroy",
     "mggx_release_cached", "mggx_forget", "mggx_set_plan_check", "mggx_cache_stats", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_core_layout_build", "mggx_core_layout_fetch", "mggx_core_layout_device", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",

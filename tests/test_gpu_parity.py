@@ -625,8 +625,31 @@ def test_graph_without_edges_and_zero_rows(gpu):
     gpu.sync()
 
 
+@pytest.mark.parametrize("ps", [1, 2, 3, 5, 6, 7, 8, 15])
+def test_small_partitions_are_summed_in_groups_of_at_most_16_neighbors(gpu, rmat_graph, ps):
+    """ps < 16: consecutive partitions of a row are consecutive edges, so a slot of the kernel takes floor(16 / ps) of them
+    at once -- one descriptor per group, not one per partition.  Same sums; and the plan holds about a sixteenth of a
+    descriptor (16 bytes) per edge at every ps, where one descriptor per partition would hold 16 / ps bytes per edge."""
+    V, ptr, col = rmat_graph
+    dim = 16
+    x = gpu.fill_normal((V, dim), seed=2)
+    sh = share_of(ptr, col, V, 2, 0)
+    xl = x[sh["lb"]:sh["ub"]]
+    gpu.release_cached()
+    got = run_agg(gpu, sh, to_dev(xl), to_dev(x), dim, ps, 4, 2)
+    want, mag = oracle_agg(sh, xl, x, dim)
+    assert_close_to_oracle(got, want, mag, FP32_TOL, "ps=%d" % ps)
+    st = gpu.cache_stats()
+    rows, nnz = sh["ub"] - sh["lb"], len(sh["col_l"]) + len(sh["col_r"])
+    unit = ps * (16 // ps)
+    units = int(np.sum(-(-np.diff(sh["ptr_l"]) // unit)) + np.sum(-(-np.diff(sh["ptr_r"]) // unit)))
+    assert st["plans"] == 1 and st["plan_bytes"] == 16 * units + 4 * (rows + 1) + 4 * rows
+    assert 16 * units <= 1.6 * nnz  # this graph: 36 neighbors per row and side on average, the last group of a row part full
+    gpu.release_cached()
+
+
 # --------------------------------------------------------------------------- explicit partition arrays
-@pytest.mark.parametrize("ps,wpb,dist", [(16, 4, 1), (3, 2, 2), (32, 8, 1)])
+@pytest.mark.parametrize("ps,wpb,dist", [(16, 4, 1), (3, 2, 2), (32, 8, 1), (1, 4, 2), (2, 1, 1), (5, 4, 4), (7, 8, 1)])
 def test_explicit_partition_arrays(gpu, rmat_graph, ps, wpb, dist):
     """SAG_host / SAG_host_fused_interleaved (local half): build_part arrays in, out += partition sums."""
     import torch

@@ -41,6 +41,10 @@ def test_static_entry_point_matches_sag_parts_twice(gpu):
     # other row widths and knobs, again larger then smaller
     _case(gpu, 20_000, 15, 600_000, 7, 41, 8, 8, 1)
     _case(gpu, 500, 9, 3_000, 9, 64, 3, 2, 3)
+    # partitions smaller than a slot (several per descriptor, their number left on the device): larger, then smaller
+    _case(gpu, 30_000, 15, 800_000, 11, 16, 1, 4, 4)
+    _case(gpu, 2_000, 11, 20_000, 13, 41, 5, 4, 1)
+    _case(gpu, 700, 10, 5_000, 15, 16, 2, 1, 1)
 
 
 def test_static_entry_point_runs_under_capture_and_allocates_nothing(gpu):
@@ -59,13 +63,15 @@ def test_static_entry_point_runs_under_capture_and_allocates_nothing(gpu):
     gpu.SAG_host_static(out, *args)  # code loaded, the array's address looked up
     gpu.sync()
     want = out.clone()
-    stats0, free0 = gpu.cache_stats(), torch.cuda.mem_get_info()[0]
     out.zero_()
+    torch.cuda.synchronize()
+    stats0, free0 = gpu.cache_stats(), torch.cuda.mem_get_info()[0]  # no torch operation between here and the second reading
     gpu.SAG_host_static(out, *args)
     gpu.sync()
-    assert torch.equal(out, want)
+    free1 = torch.cuda.mem_get_info()[0]
+    assert free1 == free0, "device memory was allocated or freed across the call"
     assert gpu.cache_stats() == stats0, "the static entry point touched the library's caches"
-    assert torch.cuda.mem_get_info()[0] == free0, "device memory was allocated or freed across the call"
+    assert torch.equal(out, want)
     side = torch.cuda.Stream()
     try:
         with torch.cuda.stream(side):
