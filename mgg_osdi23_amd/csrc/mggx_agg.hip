@@ -21,6 +21,7 @@
 // Index stream: a wavefront fetches the descriptors and the first ids of its next few rounds together into its own
 // piece of LDS (two HBM latencies per four rounds instead of per round, with no feature row in flight meanwhile) and
 // the rounds read them from there; the 16 lanes or so of a slot read the same words.
+#include <algorithm>
 #include <chrono>
 #include <cstring>
 #include <type_traits>
@@ -947,16 +948,18 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         return fail(MGGX_EINVAL, "aggregation: unknown input dtype %d", o.in_dtype);
     }
     const int slots = 64 / lpr;
-    // 0 = let the library choose (from sweeps of wpb x dist on the benchmark graphs; each choice within 5 % of the best
-    // setting of its sweep).  Few slots per wavefront (wide rows): 8 wavefronts and 16 rounds, so a workgroup still covers
-    // a few thousand neighbors -- 4 wavefronts where the kernel shares the chip with the dense core's 4-wavefront
-    // workgroups (column-blocked plans, and whatever a core leaves), and then 4 rounds in row-major order; 4 wavefronts
-    // also where rows are short (under 3 partitions per row: -3 % on the 13.9 M-row bf16 share).  Many slots
-    // (narrow rows): 4 wavefronts, 4 rounds; 8 rounds where a column-blocked plan is left with short rows (under 8
-    // partitions per row and block).
+    // 0 = let the library choose.  Few slots per wavefront (wide rows): 8 wavefronts and 16 rounds, so a workgroup still
+    // covers a few thousand neighbors; column-blocked plans: 4 wavefronts (they share the chip with the dense core's
+    // 4-wavefront workgroups); in row-major order beside a dense core: 8 wavefronts and 4 rounds; short rows (under 3
+    // partitions per row): 4 wavefronts.  Many slots (narrow rows): 4 wavefronts, 4 rounds; 8 rounds where a column-blocked
+    // plan is left with short rows (under 8 partitions per row and block).
+    // Provenance: wpb x dist sweeps on the three benchmark graphs and the bf16 share (each choice within 1 % of the best
+    // cell there), re-checked on eighteen graphs of other generators, sizes, degrees and widths: within 5.2 % of the best
+    // cell on every one, after one change the first of them forced -- beside a core in row-major order the first version
+    // took 4 wavefronts, which two 1 M-node graphs at widths 41 and 64 answered with 10 - 17 % over 8 wavefronts.
     const double per_row = (double)plan->num_parts / (double)(plan->rows > 0 ? plan->rows : 1);
     const bool beside_core = cm != nullptr;
-    if (wpb == 0) wpb = (blocked || beside_core || slots > 4 || per_row < 3.0) ? 4 : 8;
+    if (wpb == 0) wpb = (beside_core && !blocked && slots <= 4) ? 8 : (blocked || slots > 4 || per_row < 3.0) ? 4 : 8;
     if (dist == 0) {
         if (slots <= 4) dist = (beside_core && !blocked) ? 4 : 16;
         else if (blocked && per_row < 8.0) dist = 8;
@@ -1051,9 +1054,6 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         const size_t round_bytes = (size_t)slots * ((size_t)ch * 4 + 16);
         int stage = stage_max < dist ? stage_max : dist;
         while (stage > 1 && (size_t)wpb * stage * round_bytes > (40u << 10)) stage /= 2;
-        // beside a dense core whose table does not fit the caches the gathers wait for HBM anyway, and the LDS is worth
-        // more to the core's workgroups
-        if (cm && (unsigned long long)plan->real_rows * ld_bytes > (256ull << 20)) stage = 1;
         const size_t carry_lds = ((size_t)wpb * 2 * sizeof(int2) + (size_t)wpb * 2 * cpad * sizeof(float) + 15) & ~(size_t)15;
         a.stage_off = (int)(carry_lds / sizeof(float));
         a.stage_rounds = stage;
@@ -1126,11 +1126,12 @@ namespace {
 constexpr int DEFAULT_BLOCK_ROWS = 48 * 1024;  // neighbor ids per column block (sweeps on the 233 K-node benchmark graph)
 
 // A column-blocked plan re-reads and re-writes a partial output row per block: it pays off when rows are long.
+constexpr int MIN_NEIGHBORS_PER_ROW_AND_BLOCK = 20;
 bool blocking_eligible(const GraphInfo &g, int block_rows)
 {
     if (g.nnz_r > 0 || g.rows < 2 * (long long)block_rows) return false;
     const long long blocks = ((long long)g.rows + block_rows - 1) / block_rows;
-    return g.nnz_l >= 20 * blocks * (long long)g.rows;
+    return g.nnz_l >= MIN_NEIGHBORS_PER_ROW_AND_BLOCK * blocks * (long long)g.rows;
 }
 
 struct Knobs {
@@ -1165,7 +1166,7 @@ int resolve_knobs(GraphInfo &g, int dim, int dtype, int ps, int wpb, int dist, i
     if (k.core_rows == 0) {
         k.core_rows = -1;
         if (core_eligible(g, dim, dtype, 8192)) {
-            const int rc = predict_core_rows(g, dim, table_bytes, &k.core_rows);
+            const int rc = predict_core_rows(g, dim, table_bytes, k.block_rows, MIN_NEIGHBORS_PER_ROW_AND_BLOCK, &k.core_rows);
             if (rc) return rc;
         }
     }

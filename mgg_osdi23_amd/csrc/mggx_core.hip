@@ -10,6 +10,7 @@
 #include <algorithm>
 #include <chrono>
 #include <cmath>
+#include <functional>
 #include <new>
 #include <type_traits>
 
@@ -783,19 +784,31 @@ int core_partial_rows(CorePlan *p, int dim, const float4 **partial_out, const in
 // entries on average (D_t = degree sum of the tile's columns, at most 256), and the 64 lists of a slice are padded to
 // the longest of them, rounded up to 4: E[4 ceil(max of 64 Poisson(lambda) / 4)], tabulated once.  That gives the
 // useful and the padded entries of any core size from the degree histogram alone (within 3 % of the built plans on the
-// benchmark graphs).  Growing the core by a band of rows pays while the band's useful entries per padded entry stay
-// above theta = (cost of one padded entry in the LDS kernel) / (cost of one edge in the gather kernel)
-//             = ALPHA x ceil(dim/4) / (BETA x (1 + 64-byte sectors of a row) x (1 or HBM_FACTOR)),
-// constants fitted to sweeps of the core size on the 233 K-node width-16 / width-44 and the 2.45 M-node width-64
-// graphs (ALPHA 1.42 ps per padded 16-byte piece; BETA 9 ps per gathered row plus as much per 64-byte sector of it while
-// the table fits the 256 MB last-level cache, 3.2 x that beyond).  The staging of the tiles (core^2 / 65536 tiles of
-// 256 x ceil(dim/4) x 16 bytes per row group) is not in the model; it shows beyond 100,000 rows, where the model stops.
+// benchmark graphs).  Growing the core by a band of 4096 rows pays while what the band takes off the gather kernel
+// costs more there than it costs the LDS kernel:
+//     useful entries x BETA x (1 + 64-byte sectors of a row) x F  >=  padded entries x ALPHA x ceil(dim/4) [x HALVES]
+// (a gathered row: a fixed part plus one part per sector; a padded list entry: ceil(dim/4) 16-byte LDS reads; rows of more
+// than 12 pieces are summed in two halves by two workgroups, which leaves the gather kernel beside them more room:
+// HALVES).  F says where the gathers of what the core leaves are served from:
+//     1                            that rest is still gathered in column-blocked order (it has the neighbors per row and
+//                                  block that order asks for): the XCDs' L2s
+//     h + (1 - h) x F_CACHE        row-major order, table within the 256 MB last-level cache; h = the share of the rest's
+//     h + (1 - h) x F_MEMORY       gathers that go to its hottest 4 MB of rows (one XCD's L2) -- again from the degree
+//                                  histogram: a column of rank j < K keeps d_j (1 - S_K) of its edges outside the core
+//                                  (S_K = the core rows' share of all degrees), a column beyond the core all d_j
+// Provenance of the constants: BETA 9 ps is the scale; ALPHA 1.40, HALVES 0.7, F_CACHE 3.0, F_MEMORY 4.0 put the rule
+// into the flat bottom (within 2 %) of TWELVE measured core-size sweeps at once: the 233 K-node graph at widths 16 and
+// 44 and the 2.45 M-node graph at width 64 (the benchmark graphs; the first version of this model -- one threshold, a
+// factor of 3.2 beyond 256 MB -- was fitted on those three alone) and nine graphs from other RMAT settings (a from 0.45 to
+// 0.65), sizes (0.3 - 2 M nodes), mean degrees (70 - 620) and widths (16 - 64), on which the first version and two
+// intermediate ones were up to 29 % off; graphs and sweeps: dse.py --mode heldout.  The 4 MB are the size of an L2.
+// The model stops at 98,304 rows.
 namespace mggx {
 namespace {
 
 constexpr int PROFILE_SLICES = 2048;  // 131072 ranks
-constexpr double ALPHA_PS = 1.42, BETA_PS = 9.0, HBM_FACTOR = 3.2;
-constexpr unsigned long long LAST_LEVEL_CACHE_BYTES = 256ull << 20;
+constexpr double ALPHA_PS = 1.40, BETA_PS = 9.0, HALVES = 0.7, F_CACHE = 3.0, F_MEMORY = 4.0;
+constexpr unsigned long long L2_BYTES = 4ull << 20, LAST_LEVEL_CACHE_BYTES = 256ull << 20;
 constexpr int MODEL_STEP = 4096, MODEL_MAX_CORE = 98304;
 
 __global__ void __launch_bounds__(256) k_degrees(const int *__restrict__ ptr, int rows, int *__restrict__ deg)
@@ -878,14 +891,13 @@ int fetch_degree_profile(GraphInfo &g)
 
 }  // namespace
 
-int predict_core_rows(GraphInfo &g, int dim, unsigned long long table_bytes, int *core_rows)
+int predict_core_rows(GraphInfo &g, int dim, unsigned long long table_bytes, int block_rows, int min_per_row_block, int *core_rows)
 {
     static const PaddingTable padded;
     *core_rows = -1;
     if (g.rows < 2 * MODEL_STEP || g.nnz_l <= 0) return MGGX_OK;
-    const bool beyond_cache = table_bytes > LAST_LEVEL_CACHE_BYTES;
     for (const GraphInfo::Predicted &p : g.predicted)
-        if (p.dim == dim && p.beyond_cache == beyond_cache) {
+        if (p.dim == dim && p.block_rows == block_rows && p.table_bytes == table_bytes) {
             *core_rows = p.core_rows;
             return MGGX_OK;
         }
@@ -893,8 +905,7 @@ int predict_core_rows(GraphInfo &g, int dim, unsigned long long table_bytes, int
     if (rc) return rc;
     const int n4 = (dim + 3) / 4;
     const int sectors = (dim * 4 + 63) / 64;
-    // rows summed in two halves (more than 12 pieces) leave the gather kernel beside them more room: measured 0.75 of the cost
-    const double theta = ALPHA_PS * (n4 > 12 ? 0.75 : 1.0) * n4 / (BETA_PS * (1 + sectors) * (beyond_cache ? HBM_FACTOR : 1.0));
+    const double entry = ALPHA_PS * n4 * (n4 > 12 ? HALVES : 1.0);  // per padded list entry
     const double nnz = (double)g.nnz_l;
     const int max_core = std::min({MODEL_MAX_CORE, g.rows / 2 / MODEL_STEP * MODEL_STEP, (int)g.slice_deg.size() * 64 / MODEL_STEP * MODEL_STEP});
     // useful and padded entries of the block (slices [s0, s1) x tiles [t0, t1))
@@ -909,17 +920,43 @@ int predict_core_rows(GraphInfo &g, int dim, unsigned long long table_bytes, int
             }
         }
     };
+    // h: of the gathers a core of k rows leaves, the share that goes to the hottest L2_BYTES of table rows
+    const double row_bytes = (double)table_bytes / (double)g.rows;
+    const size_t hot_slices = (size_t)std::max(1.0, (double)L2_BYTES / row_bytes / 64.0);
+    std::vector<double> w(g.slice_deg.size());
+    const auto hot_share = [&](int k) {
+        double core_deg = 0.0;
+        for (int sl = 0; sl < k / 64; ++sl) core_deg += g.slice_deg[(size_t)sl];
+        const double outside = 1.0 - core_deg / nnz;  // of a core column's edges, the share whose row is not in the core
+        for (size_t sl = 0; sl < w.size(); ++sl) w[sl] = g.slice_deg[sl] * (sl < (size_t)(k / 64) ? outside : 1.0);
+        const size_t take = std::min(hot_slices, w.size());
+        std::partial_sort(w.begin(), w.begin() + (long)take, w.end(), std::greater<double>());
+        double hot = 0.0;
+        for (size_t i = 0; i < take; ++i) hot += w[i];
+        const double left = nnz - core_deg * (core_deg / nnz);  // all edges but the core x core block
+        return left > 0.0 ? std::min(1.0, hot / left) : 1.0;
+    };
+    const double far = table_bytes <= LAST_LEVEL_CACHE_BYTES ? F_CACHE : F_MEMORY;
+    const double blocks = block_rows > 0 ? std::ceil((double)g.rows / block_rows) : 0.0;
     int best = 0;
+    double taken = 0.0;
     for (int k = MODEL_STEP; k <= max_core; k += MODEL_STEP) {
         // the band the core grows by: new rows x all tiles, old rows x new tiles
         double useful = 0.0, pad = 0.0;
         block((k - MODEL_STEP) / 64, k / 64, 0, k / 256, &useful, &pad);
         block(0, (k - MODEL_STEP) / 64, (k - MODEL_STEP) / 256, k / 256, &useful, &pad);
-        if (pad <= 0.0 || useful / pad < theta) break;
+        double f = 1.0;
+        const bool rest_blocked = block_rows > 0 && nnz - taken - useful >= (double)min_per_row_block * blocks * (double)g.rows;
+        if (!rest_blocked) {
+            const double h = hot_share(k);
+            f = h + (1.0 - h) * far;
+        }
+        if (pad <= 0.0 || useful * BETA_PS * (1 + sectors) * f < pad * entry) break;
         best = k;
+        taken += useful;
     }
     if (best >= 2 * MODEL_STEP) *core_rows = best;
-    g.predicted.push_back({dim, beyond_cache, *core_rows});
+    g.predicted.push_back({dim, block_rows, table_bytes, *core_rows});
     return MGGX_OK;
 }
 

@@ -174,7 +174,7 @@ struct GraphInfo {
     // slices (rows ranked by falling degree), fetched once per record
     std::vector<float> slice_deg;
     bool have_profile = false;
-    struct Predicted { int dim; bool beyond_cache; int core_rows; };
+    struct Predicted { int dim; int block_rows; unsigned long long table_bytes; int core_rows; };
     std::vector<Predicted> predicted;  // what the cost model said for a row width (evaluated once, a millisecond of host time)
     bool internal = false;  // arrays owned by the library (the remainder CSR of a dense-core plan): no content check
     bool pinned = false;    // used inside a stream capture: never evicted
@@ -263,7 +263,10 @@ int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int 
 // Cost model of the dense core (degree histogram x row width): the core size that is predicted to pay for this CSR, a
 // multiple of 4096, or -1 for none.  table_bytes = rows x row pitch of the feature table.  Fetches the record's degree
 // profile on first use (one sort of the degrees on the device, 4 KiB to the host; synchronises).
-int predict_core_rows(GraphInfo &g, int dim, unsigned long long table_bytes, int *core_rows);
+// block_rows: the column-block size the call would use for this CSR (> 0), or <= 0 where it is not eligible for the
+// column-blocked order; min_per_row_block: neighbors per row and block a CSR needs for that order (what the core leaves is
+// held to the same bar).
+int predict_core_rows(GraphInfo &g, int dim, unsigned long long table_bytes, int block_rows, int min_per_row_block, int *core_rows);
 void core_plan_free(CorePlan *p);
 int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, const Gate &gate, hipStream_t stream);
 int run_core_sums(CorePlan *p, int dim, const Gate &gate, hipStream_t stream);

@@ -12,6 +12,8 @@ Prints ps x wpb (dist = 1) and dist x ps (wpb = 8) tables in ms, GB/s of algorit
     python -m mgg_osdi23_amd.dse --workload whole --dim 44 --ld 48 --mode wd      # wpb x dist at ps 16, everything else by rule
     python -m mgg_osdi23_amd.dse --workload sparse --dim 64 --gin --mode core     # dense-core size sweep, best of a few wpb x dist
 
+    python -m mgg_osdi23_amd.dse --mode heldout                                   # rules and cost model on graphs they never saw
+
 `--mode wd`: the wpb x dist table at ps 16 with the order and the dense core left to the library (its rules and cost
 model), and the time of the all-by-rule call beside the table's best.  `--mode core`: the aggregation time against the
 size of the dense core (no counterpart in the reference), with the entries of the built plans (useful, padded, left to
@@ -26,6 +28,123 @@ import sys
 import numpy as np
 
 from . import host
+
+
+# Graph families none of the library's rules or cost-model constants were fitted on (those came from sweeps on the three
+# benchmark graphs "share", "whole" and "sparse" below): other generators, other skews, other sizes, other mean degrees.
+#   name: (generator, generator arguments, ranks, row width, row pitch)
+HELD_OUT = {
+    "er32": ("er", dict(num_nodes=1_000_000, avg_degree=32.0, seed=101), 1, 64, 64),
+    "er200": ("er", dict(num_nodes=500_000, avg_degree=200.0, seed=102), 1, 16, 16),
+    "rmat45": ("rmat", dict(scale=20, num_nodes=1_000_000, num_draws=40_000_000, a=0.45, b=0.22, c=0.22, seed=103), 1, 41, 48),
+    "rmat65": ("rmat", dict(scale=19, num_nodes=500_000, num_draws=60_000_000, a=0.65, b=0.15, c=0.15, seed=104), 1, 16, 16),
+    "rmat57w64": ("rmat", dict(scale=20, num_nodes=1_000_000, num_draws=100_000_000, a=0.57, b=0.19, c=0.19, seed=105), 1, 64, 64),
+    "share2": ("rmat", dict(scale=21, num_nodes=2_000_000, num_draws=30_000_000, a=0.57, b=0.19, c=0.19, seed=106, scramble=True), 2, 16, 16),
+    # further batches: each was measured with the rules as they then stood, and what it showed went into them
+    "rmat50w32": ("rmat", dict(scale=20, num_nodes=750_000, num_draws=50_000_000, a=0.50, b=0.20, c=0.20, seed=107), 1, 32, 32),
+    "er64": ("er", dict(num_nodes=750_000, avg_degree=64.0, seed=108), 1, 41, 48),
+    "rmat60w64": ("rmat", dict(scale=21, num_nodes=2_000_000, num_draws=80_000_000, a=0.60, b=0.17, c=0.17, seed=109), 1, 64, 64),
+    "rmat57w24": ("rmat", dict(scale=19, num_nodes=400_000, num_draws=120_000_000, a=0.57, b=0.19, c=0.19, seed=110), 1, 24, 24),
+    "rmat55w16": ("rmat", dict(scale=21, num_nodes=1_500_000, num_draws=60_000_000, a=0.55, b=0.20, c=0.20, seed=111), 1, 16, 16),
+    "rmat62w41": ("rmat", dict(scale=20, num_nodes=600_000, num_draws=90_000_000, a=0.62, b=0.16, c=0.16, seed=112), 1, 41, 48),
+    "er24w64": ("er", dict(num_nodes=2_000_000, avg_degree=24.0, seed=113), 1, 64, 64),
+    "rmat48w64": ("rmat", dict(scale=19, num_nodes=300_000, num_draws=100_000_000, a=0.48, b=0.21, c=0.21, seed=114), 1, 64, 64),
+    # the last four have only ever been measured with the rules as they are now
+    "rmat52w48": ("rmat", dict(scale=20, num_nodes=900_000, num_draws=70_000_000, a=0.52, b=0.20, c=0.20, seed=115), 1, 48, 48),
+    "rmat63w64": ("rmat", dict(scale=20, num_nodes=700_000, num_draws=110_000_000, a=0.63, b=0.15, c=0.17, seed=116), 1, 64, 64),
+    "rmat58w20": ("rmat", dict(scale=21, num_nodes=1_800_000, num_draws=90_000_000, a=0.58, b=0.18, c=0.18, seed=117), 1, 20, 20),
+    "rmat46w16": ("rmat", dict(scale=19, num_nodes=350_000, num_draws=140_000_000, a=0.46, b=0.22, c=0.22, seed=118), 1, 16, 16),
+}
+
+
+def build_held_out(name: str, shrink: int = 0):
+    """One of the HELD_OUT graphs as a workload dict (see build_workload); shrink divides nodes and edges by 2^k."""
+    import torch
+    gen, kw, ranks, dim, ld = HELD_OUT[name]
+    kw = dict(kw)
+    if gen == "er":
+        kw["num_nodes"] >>= shrink
+        V = kw["num_nodes"]
+        ptr, col = host.gen_er(**kw)
+    else:
+        kw["num_nodes"] >>= shrink
+        kw["num_draws"] >>= shrink
+        kw["scale"] -= shrink
+        V = kw["num_nodes"]
+        if ranks > 1:
+            npp, lb, ub = host.range_partition(V, ranks, 0)
+            kw.update(row_lo=lb, row_hi=ub)
+        ptr, col = host.gen_rmat(**kw)
+    npp, lb, ub = host.range_partition(V, ranks, 0)
+    if ranks > 1:
+        lp, rp, lc, rc = host.split_CSR(ptr, col, lb, ub)
+    else:
+        lp, lc, rp, rc = ptr, col, np.zeros(V + 1, np.int32), np.zeros(0, np.int32)
+    rows_tbl = ranks * npp
+    x = np.zeros((rows_tbl, ld), np.float32)
+    x[:, :dim] = host.fill_normal((rows_tbl, dim), seed=11)
+    t = lambda a: torch.from_numpy(a).cuda() if len(a) else torch.zeros(1, dtype=torch.int32, device="cuda")
+    w = dict(lb=lb, ub=ub, npp=npp, nnz=len(lc) + len(rc), rows=ub - lb, dim=dim, ld=ld, xr=torch.from_numpy(x).cuda(),
+             xl=torch.from_numpy(np.ascontiguousarray(x[lb:ub])).cuda(), ptr_l=t(lp), col_l=t(lc), ptr_r=t(rp), col_r=t(rc),
+             host=dict(ptr_l=lp, col_l=lc, ptr_r=rp, col_r=rc, x=x))
+    w["out"] = torch.empty(ub - lb, ld, device="cuda")
+    w["bytes"] = w["nnz"] * (4 + dim * 4) + w["rows"] * dim * 4 + (w["rows"] + 1) * 4 * (2 if len(rc) else 1)
+    return w
+
+
+def tune(w, gin=False):
+    """The library's own search on a workload -> (knobs, ms)."""
+    return host.tune_np_div(w["out"], w["xl"], w["ptr_l"], w["col_l"], w["ptr_r"], w["col_r"], w["lb"], w["ub"], w["dim"], w["npp"], 16,
+                            input_remote=w["xr"], ld_in=w["ld"], ld_out=w["ld"], gin_eps=0.0 if gin else None)
+
+
+def held_out_table(args):
+    """Rules and cost model against measurement on the HELD_OUT graphs: by rule (every knob left at 0), the best cell of the
+    wpb x dist table (order and core by rule), the library's search (ps x order x core size x wpb x dist), and the dense-core
+    size the cost model predicts against the best of a sweep of sizes.  Prints one markdown table."""
+    import torch
+    rows = []
+    for name in (args.only.split(",") if args.only else HELD_OUT):
+        w = build_held_out(name, args.shrink)
+        med = lambda wpb=0, dist=0, **kw: sorted(time_setting(w, 16, wpb, dist, args.iters, **kw) for _ in range(3))[1]
+        for _ in range(3):
+            time_setting(w, 16, 0, 0, args.iters, core_rows=0)
+        rule = med(core_rows=0)
+        rule_kernel = host.last_agg_kernel()
+        grid = min((med(wpb=wpb, dist=d, core_rows=0), wpb, d) for wpb in (2, 4, 8, 16) for d in (1, 2, 4, 8, 16))
+        host.forget(w["ptr_l"])  # the search must not find the rule's plans warm and its own cold
+        knobs, _ = tune(w)
+        searched = med(core_rows=0)  # the zeros now mean the searched setting
+        host.forget(w["ptr_l"])
+        import re
+        m = re.search(r"core=(\d+)", rule_kernel)
+        predicted = int(m.group(1)) if m else -1
+        best_core = (rule if predicted < 0 else 1e30, -1)
+        if not len(w["host"]["col_r"]):
+            for K in (-1, 8192, 16384, 24576, 32768, 40960, 49152, 65536, 81920, 98304):
+                if K > w["rows"] // 2:
+                    continue
+                cells = [(med(wpb=a, dist=b, core_rows=K), a, b) for a, b in ((4, 4), (4, 16), (8, 4), (8, 16))]
+                print("  core %6d: " % K + "  ".join("wpb %d dist %2d %.4f" % (a, b, ms) for ms, a, b in cells) + "   by rule %.4f" % med(core_rows=K), flush=True)
+                best_core = min(best_core, (min(cells)[0], K))
+                host.forget(w["ptr_l"])
+            at_predicted = min(med(wpb=a, dist=b, core_rows=predicted) for a, b in ((4, 4), (4, 16), (8, 4), (8, 16))) if predicted > 0 else best_core[0]
+        else:
+            at_predicted = best_core[0]
+        rows.append((name, w["rows"], w["nnz"], w["dim"], rule, grid, searched, knobs, predicted, best_core, at_predicted, rule_kernel))
+        print("%s: rule %.4f ms [%s]; best wpb x dist cell %.4f (wpb %d dist %d); searched %.4f %s; core predicted %d, best of sweep %d (%.4f ms, "
+              "at the predicted size %.4f)" % (name, rule, rule_kernel, grid[0], grid[1], grid[2], searched, knobs, predicted, best_core[1],
+                                               best_core[0], at_predicted), flush=True)
+        host.release_cached()
+        del w
+        torch.cuda.empty_cache()
+    print("\n| graph | rows | nnz | width | by rule (ms) | best wpb x dist cell | rule / cell | searched (ms) | rule / searched | core: predicted | "
+          "core: best of sweep | predicted / best (ms ratio) |")
+    print("|---|---|---|---|---|---|---|---|---|---|---|---|")
+    for name, r, nnz, dim, rule, grid, searched, knobs, predicted, best_core, at_predicted, _k in rows:
+        print("| %s | %d | %d | %d | %.4f | %.4f (wpb %d, dist %d) | %.3f | %.4f | %.3f | %d | %d | %.3f |" %
+              (name, r, nnz, dim, rule, grid[0], grid[1], grid[2], rule / grid[0], searched, rule / searched, predicted, best_core[1],
+               at_predicted / best_core[0]))
 
 
 def build_workload(name: str, dim: int, small: bool, ld: int = 0, compact: bool = False):
@@ -135,8 +254,11 @@ def main():
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--small", action="store_true")
     ap.add_argument("--out", default="")
-    ap.add_argument("--mode", default="ps", choices=["ps", "wd", "core"], help="ps: the reference's ps x wpb and dist x ps tables; "
-                    "wd: wpb x dist at ps 16 with order and dense core by rule; core: dense-core size sweep")
+    ap.add_argument("--mode", default="ps", choices=["ps", "wd", "core", "heldout"], help="ps: the reference's ps x wpb and dist x ps tables; "
+                    "wd: wpb x dist at ps 16 with order and dense core by rule; core: dense-core size sweep; heldout: rules and cost "
+                    "model against measurement on graph families they were not fitted on")
+    ap.add_argument("--only", default="", help="--mode heldout: comma-separated names out of " + ", ".join(HELD_OUT))
+    ap.add_argument("--shrink", type=int, default=0, help="--mode heldout: divide nodes and edges by 2^k")
     ap.add_argument("--ld", type=int, default=0, help="row pitch of the tables in floats (default: dim)")
     ap.add_argument("--gin", action="store_true", help="aggregate with the GIN self term")
     ap.add_argument("--compact-remote", action="store_true", help="share: stage the remote rows compactly")
@@ -145,6 +267,8 @@ def main():
     torch.cuda.set_device(0)
     host.init(0)
     host.use_torch_stream()
+    if args.mode == "heldout":
+        return held_out_table(args)
     w = build_workload(args.workload, args.dim, args.small, args.ld, args.compact_remote)
     print("workload %s: rows=%d nnz=%d dim=%d algorithmic bytes=%d" % (args.workload, w["rows"], w["nnz"], args.dim, w["bytes"]))
     if args.mode == "wd":

@@ -351,3 +351,35 @@ def test_full_size_whole_graph_gcn_widths(gpu):
     gpu.sync()
     assert "blocks=5" in gpu.last_agg_kernel()
     assert np.array_equal(acc.cpu().numpy()[:, 3], np.diff(ptr).astype(np.float32) + 1.0)
+
+
+# --------------------------------------------------------------------------- rules and cost model on graphs they were not set on
+@pytest.mark.parametrize("name,shrink", [("rmat63w64", 1), ("rmat58w20", 2), ("rmat52w48", 2)])
+def test_rules_hold_on_graphs_they_never_saw(gpu, name, shrink):
+    """The knobs left at 0 (wpb, dist, partition order, dense-core size by the cost model) against the library's own search
+    on graph families that were only ever measured, never used to set a rule or a constant (mgg_osdi23_amd.dse.HELD_OUT,
+    the last four), at a fraction of their size: the rules' setting may be at most 10 % slower than the searched one, and
+    gives the oracle's sums on sampled rows."""
+    import torch
+    from mgg_osdi23_amd import dse
+    w = dse.build_held_out(name, shrink)
+    try:
+        timed = lambda: sorted(dse.time_setting(w, 16, 0, 0, 10, core_rows=0) for _ in range(5))[2]
+        timed()
+        by_rule = timed()
+        kernel = gpu.last_agg_kernel()
+        h = w["host"]
+        rng = np.random.default_rng(1)
+        rows = np.unique(np.concatenate([np.argsort(np.diff(h["ptr_l"]))[-10:], rng.integers(0, w["rows"], 300)])).astype(np.int32)
+        x = np.ascontiguousarray(h["x"][:, : w["dim"]])
+        want = orc.sag_np_div_rows(rows, x, x, h["ptr_l"], h["col_l"], None, None, 0, w["rows"], w["dim"], w["npp"])
+        mag = orc.sag_np_div_rows(rows, x, x, h["ptr_l"], h["col_l"], None, None, 0, w["rows"], w["dim"], w["npp"], abs_sum=True)
+        got = w["out"][torch.from_numpy(rows.astype(np.int64)).cuda()][:, : w["dim"]].cpu().numpy()
+        assert_close_to_oracle(got, want, mag, FP32_TOL, "%s by rule [%s]" % (name, kernel))
+        gpu.forget(w["ptr_l"])
+        knobs, _ = dse.tune(w)
+        searched = timed()
+        assert by_rule <= 1.10 * searched, "%s: by rule %.4f ms [%s], searched %.4f ms %s" % (name, by_rule, kernel, searched, knobs)
+    finally:
+        gpu.forget(w["ptr_l"])
+        gpu.release_cached()
