@@ -23,7 +23,8 @@ struct DenseArgs {
     int d1, d2;
     int relu;
     int vec_out;  // bit 0: rows of out may be written 4 elements at a time (alignment and stride allow it);
-                  // bit 1: and they are whole 128-byte lines written once: streaming stores
+                  // bit 1: and they are whole 128-byte lines written once: streaming stores;
+                  // bit 2: bf16 rows may be written 8 elements (16 bytes) at a time
     int stream_x; // rows of X are whole 128-byte lines per K group (d1 % 64 == 0, aligned base and pitch)
 };
 
@@ -105,6 +106,42 @@ __device__ __forceinline__ void store_tile_f32(const DenseArgs &a, const v4f (&a
 // The resident kernels form every product transposed -- W as the A operand, X as the B operand (both operand layouts
 // give lane L the element (L % 16, L / 16), so the loads are the same) -- which leaves lane L with
 // D[row L % 16][16 nb + 4 (L / 16) + r], r = 0..3: four consecutive columns of one output row, one 16-byte store.
+// bf16 output with the columns of W staged pairwise interleaved (paired_column below): lane (row, kq) holds the eight
+// consecutive columns 32 p + 8 kq .. + 7 in acc[2 p] and acc[2 p + 1] -- one 16-byte store, 64 contiguous bytes per row and
+// instruction (unpaired: 8-byte stores, 32 bytes per row and instruction, and the write path, not the reads, set the pace).
+template <int NB>
+__device__ __forceinline__ void store_rows_bf16_paired(void *out, long long ld_out, float scale, int relu, const v4f (&acc)[NB],
+                                                       long long row, bool row_ok, int c0, int kq)
+{
+    static_assert(NB % 2 == 0, "pairs of 16-column blocks");
+    if (!row_ok) return;
+    typedef unsigned v4u_s __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int p = 0; p < NB / 2; ++p) {
+        unsigned pk[4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                v[r] = acc[2 * p + h][r] * scale;
+                if (relu) v[r] = fmaxf(v[r], 0.f);
+            }
+            const v2bf q0 = __builtin_convertvector((v2f){v[0], v[1]}, v2bf), q1 = __builtin_convertvector((v2f){v[2], v[3]}, v2bf);
+            __builtin_memcpy(&pk[2 * h], &q0, 4);
+            __builtin_memcpy(&pk[2 * h + 1], &q1, 4);
+        }
+        __bf16 *o = static_cast<__bf16 *>(out) + row * ld_out + c0 + 32 * p + 8 * kq;
+        __builtin_nontemporal_store((v4u_s){pk[0], pk[1], pk[2], pk[3]}, reinterpret_cast<v4u_s *>(o));
+    }
+}
+// Which column of W the LDS column slot j (16-column block j / 16, position j % 16) holds when blocks are paired.
+__device__ __forceinline__ int paired_column(int j)
+{
+    const int nb = j >> 4, m = j & 15;
+    return 32 * (nb >> 1) + 8 * (m >> 2) + 4 * (nb & 1) + (m & 3);
+}
+
 template <int NB, bool OUT_BF16>
 __device__ __forceinline__ void store_rows(void *out, long long ld_out, int d2, float scale, int relu, int vec_out,
                                            const v4f (&acc)[NB], long long row, bool row_ok, int c0, int kq)
@@ -492,9 +529,13 @@ __global__ void __launch_bounds__(256) k_dense_xw_bf16(const DenseArgs a)
     const int KP = d1p + 8;  // row stride of Wt in bf16: the +8 (16 bytes) staggers rows over the banks
     const unsigned short *w = static_cast<const unsigned short *>(a.w);
     unsigned short *wts = reinterpret_cast<unsigned short *>(wt);
+    // bf16 output in whole 16-byte pieces (all NB blocks inside d2, rows of out on 16-byte boundaries): columns staged pairwise
+    // interleaved, so a lane ends up with eight consecutive columns (store_rows_bf16_paired)
+    const bool paired = OUT_BF16 && NB % 2 == 0 && (a.vec_out & 4) != 0 && c0 + NB * 16 <= a.d2;
     for (int idx = (int)threadIdx.x; idx < d1p * NB * 16; idx += 256) {
         const int k = idx / (NB * 16), j = idx % (NB * 16);
-        wts[j * KP + k] = (k < a.d1 && c0 + j < a.d2) ? w[(long long)k * a.d2 + c0 + j] : (unsigned short)0;
+        const int col = c0 + (paired ? paired_column(j) : j);
+        wts[j * KP + k] = (k < a.d1 && col < a.d2) ? w[(long long)k * a.d2 + col] : (unsigned short)0;
     }
     __syncthreads();
 
@@ -533,7 +574,12 @@ __global__ void __launch_bounds__(256) k_dense_xw_bf16(const DenseArgs a)
         }
         if (last_k) {
             const long long row = tile * 16 + i;
-            store_rows<NB, OUT_BF16>(a.out, a.ld_out, a.d2, scale, a.relu, a.vec_out, acc, row, row < a.n, c0, kb);
+            if constexpr (OUT_BF16 && NB % 2 == 0) {
+                if (paired) store_rows_bf16_paired<NB>(a.out, a.ld_out, scale, a.relu, acc, row, row < a.n, c0, kb);
+                else store_rows<NB, OUT_BF16>(a.out, a.ld_out, a.d2, scale, a.relu, a.vec_out, acc, row, row < a.n, c0, kb);
+            } else {
+                store_rows<NB, OUT_BF16>(a.out, a.ld_out, a.d2, scale, a.relu, a.vec_out, acc, row, row < a.n, c0, kb);
+            }
         }
         av = an;
         scale = scale_next;
@@ -814,6 +860,7 @@ MGGX_EXPORT int mggx_dense_xw_bf16(void *d_out, const void *d_x, const void *d_w
     a.d2 = d2;
     a.relu = o.relu != 0;
     a.vec_out = a.ld_out % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & (out_dtype == MGGX_BF16 ? 7u : 15u)) == 0;
+    if (out_dtype == MGGX_BF16 && a.ld_out % 8 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0) a.vec_out |= 4;  // 16-byte pieces of 8 bf16
     if (a.ld_x < d1 || a.ld_out < d2) return fail(MGGX_EINVAL, "dense_xw_bf16: row stride smaller than width");
     const int nb = mggx::pick_nb(d2);
     const int gy = ((d2 + 15) / 16 + nb - 1) / nb;
