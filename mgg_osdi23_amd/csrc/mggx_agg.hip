@@ -119,6 +119,16 @@ __device__ __forceinline__ float lane_read(float v, int src)
     return __int_as_float(__builtin_amdgcn_ds_bpermute(src << 2, __float_as_int(v)));
 }
 
+// Rows of 16 lanes swapped between two registers without a trip through the LDS crossbar (gfx950):
+// rows_from_even(v) = {v.row0, v.row0, v.row2, v.row2}, rows_from_odd(v) = {v.row1, v.row1, v.row3, v.row3},
+// low_half(v) = {v.row0, v.row1, v.row0, v.row1}.
+__device__ __forceinline__ int rows_from_even(int v) { return (int)__builtin_amdgcn_permlane16_swap((unsigned)v, (unsigned)v, false, false)[0]; }
+__device__ __forceinline__ int rows_from_odd(int v) { return (int)__builtin_amdgcn_permlane16_swap((unsigned)v, (unsigned)v, false, false)[1]; }
+__device__ __forceinline__ int low_half(int v) { return (int)__builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false)[0]; }
+__device__ __forceinline__ float rows_from_even(float v) { return __int_as_float(rows_from_even(__float_as_int(v))); }
+__device__ __forceinline__ float rows_from_odd(float v) { return __int_as_float(rows_from_odd(__float_as_int(v))); }
+__device__ __forceinline__ float low_half(float v) { return __int_as_float(low_half(__float_as_int(v))); }
+
 template <int MODE>
 struct ModeTraits {
     static constexpr int NV = MODE == MODE_BF16_VEC8 ? 8 : 4;
@@ -567,6 +577,30 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
             has_first |= c_first;
         }
         // segmented inclusive scan over slots, keyed by row (equal rows are adjacent)
+        if constexpr (LPR == 16 || LPR == 32) {
+            // Slots are whole rows of 16 lanes (or halves of the wavefront): the scan moves registers with the row- and
+            // half-swap instructions.  Two steps for four slots: slots 1 and 3 take slots 0 and 2; then slots 2 and 3
+            // take slot 1, which by then holds the sum of its run so far.
+            const auto step = [&](auto from, bool lower) {
+                const int prow = from(row);
+                const bool take = lower && prow == row && row >= 0;
+                if (__any(take)) {
+                    const int pf = from(has_first);
+                    has_first |= take ? pf : 0;
+#pragma unroll
+                    for (int i = 0; i < NV; ++i) {
+                        const float pvv = from(acc[i]);
+                        acc[i] += take ? pvv : 0.0f;
+                    }
+                }
+            };
+            if constexpr (LPR == 16) {
+                step([](auto v) { return rows_from_even(v); }, (slot & 1) != 0);
+                step([](auto v) { return low_half(rows_from_odd(v)); }, slot >= 2);
+            } else {
+                step([](auto v) { return low_half(v); }, slot == 1);
+            }
+        } else {
         static_for<0, 6>([&](auto oo) {
             constexpr int o = 1 << decltype(oo)::value;
             if constexpr (o < S) {
@@ -585,6 +619,7 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
                 }
             }
         });
+        }
         // the last slot of each run now holds the run's sum
         int nrow = -2;
         if constexpr (S > 1) {
