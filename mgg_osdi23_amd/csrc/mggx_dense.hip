@@ -1,5 +1,12 @@
 // Dense node update Out = X . W on the matrix cores (fp32 and bf16 MFMA), and the row softmax.
+#include <algorithm>
+
 #include "mggx_dev.h"
+
+// Where k_wt_image leaves the bf16 update's weight matrix for the workgroups of k_dense_xw_bf16_lines (one per GPU the
+// library runs on; calls on the library's stream follow one another).  In host code the name is only a handle for
+// hipGetSymbolAddress.
+static __device__ __align__(256) unsigned short wt_image[128 * (128 + 8)];
 
 namespace mggx {
 namespace {
@@ -26,6 +33,7 @@ struct DenseArgs {
                   // bit 1: and they are whole 128-byte lines written once: streaming stores;
                   // bit 2: bf16 rows may be written 8 elements (16 bytes) at a time
     int stream_x; // rows of X are whole 128-byte lines per K group (d1 % 64 == 0, aligned base and pitch)
+    int tiles_per_wave;  // k_dense_xw_bf16_lines: rounds of consecutive tiles per workgroup
 };
 
 // v_mfma_f32_16x16x4_f32 operand layout (wave64):
@@ -519,7 +527,7 @@ __device__ __forceinline__ v8bf load_x8_bf16(const void *xbase, long long row, l
 template <int NB, bool X_F32, bool OUT_BF16>
 __global__ void __launch_bounds__(256) k_dense_xw_bf16(const DenseArgs a)
 {
-    extern __shared__ float lds_raw[];
+    extern __shared__ __align__(16) float lds_raw[];
     __bf16 *wt = reinterpret_cast<__bf16 *>(lds_raw);
     const int lane = (int)(threadIdx.x & 63u);
     const int wave = (int)(threadIdx.x >> 6);
@@ -569,7 +577,7 @@ __global__ void __launch_bounds__(256) k_dense_xw_bf16(const DenseArgs a)
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             v8bf bv;
-            __builtin_memcpy(&bv, wt + (size_t)(nb * 16 + i) * KP + k, 16);
+            bv = *reinterpret_cast<const v8bf *>(wt + (size_t)(nb * 16 + i) * KP + k);  // one 16-byte LDS read (rows of Wt are 16-byte multiples)
             acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, av, acc[nb], 0, 0, 0);
         }
         if (last_k) {
@@ -586,6 +594,160 @@ __global__ void __launch_bounds__(256) k_dense_xw_bf16(const DenseArgs a)
         tile = ntile;
         k0 = nk;
         if (tile >= tiles) break;
+    }
+}
+
+// The same product for fp32 X and bf16 output with every access to memory in whole lines: a wavefront reads the 16 rows of
+// its tile as they lie in memory (a row's bytes on neighbouring lanes, streaming hint), rounds them to bf16 into its own
+// piece of LDS, and the matrix cores take their operand layout from there; the finished tile goes back through the same
+// piece of LDS and leaves as whole rows too.  The operand layout read straight from memory touches a quarter of a line per
+// lane and the memory system answers it at 5.4-5.9 TB/s where it answers whole lines at 6.8-7.0 (13.9 M rows of 128 -> 128:
+// 2.03 ms with the operand layout and a persistent grid, 1.85 with this kernel).  The next tile's rows are in flight while the current one is
+// converted, multiplied and stored.  D1 in {64, 128}, all NB * 16 columns of W, rows of X and of the output on 16-byte
+// boundaries.
+constexpr int LINES_WAVES = 8;
+constexpr int WT_IMAGE_MAX = 128 * (128 + 8);  // bf16 elements
+
+// image[j * (d1 + 8) + k] = W[k][paired_column(j)]: W transposed with its columns in the order the paired 16-byte stores
+// want, as the workgroups of k_dense_xw_bf16_lines copy it into LDS
+__global__ void __launch_bounds__(256) k_wt_image(unsigned short *__restrict__ image, const unsigned short *__restrict__ w, int d1, int d2)
+{
+    const int idx = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (idx >= d1 * d2) return;
+    const int k = idx / d2, c = idx % d2;  // reads along rows of W
+    // slot j with paired_column(j) == c
+    const int p = c >> 5, q = c & 31, kq = q >> 3, h = (q >> 2) & 1, m = q & 3;
+    const int j = 16 * (2 * p + h) + 4 * kq + m;
+    image[j * (d1 + 8) + k] = w[idx];
+}
+template <int NB, int D1>
+__global__ void __launch_bounds__(LINES_WAVES * 64) k_dense_xw_bf16_lines(const DenseArgs a)
+{
+    static_assert(NB % 2 == 0 && (D1 == 64 || D1 == 128), "shapes this variant is written for");
+    extern __shared__ __align__(16) float lds_raw[];
+    constexpr int D2 = NB * 16;
+    constexpr int KP = D1 + 8;                       // row stride of Wt in bf16 (staggers rows over the banks)
+    constexpr int XP = D1 * 2 + 16, OP = D2 * 2 + 16;  // bytes per row of a wavefront's X tile / output tile in LDS
+    constexpr int TILE_BYTES = 16 * (XP > OP ? XP : OP);
+    constexpr int LR = D1 / 4, RPI = 64 / LR, NLD = 16 / RPI;    // lanes per X row, rows per load instruction, loads per tile
+    constexpr int LRO = D2 / 8, RPO = 64 / LRO, NST = 16 / RPO;  // the same for the output rows (8 bf16 per lane)
+    typedef unsigned v4u_s __attribute__((ext_vector_type(4)));
+    typedef unsigned v2u_s __attribute__((ext_vector_type(2)));
+    const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
+    const int i = lane & 15, kb = lane >> 4;
+    unsigned short *wts = reinterpret_cast<unsigned short *>(lds_raw);
+    const __bf16 *wt = reinterpret_cast<const __bf16 *>(lds_raw);
+    char *mine = reinterpret_cast<char *>(lds_raw) + (size_t)D2 * KP * 2 + (size_t)wave * TILE_BYTES;
+    // Workgroups are short-lived and take their tiles in launch order -- a.tiles_per_wave rounds of LINES_WAVES
+    // consecutive tiles -- so what the whole chip has in flight at any moment is one narrow window of X and of the output
+    // moving through memory.  A 2:1 read/write stream converted by one-shot workgroups in launch order runs at
+    // 6.1-6.2 TB/s; by workgroups that each walk through 16 / 64 pieces, or stride over the whole array: 5.4 / 5.2.
+    // Against that stands what a workgroup pays before its first tile (the copy of W), so: 8 rounds (13.9 M rows of
+    // 128 -> 128: 1 / 2 / 4 / 8 / 16 rounds 2.12 / 1.93 / 1.88 / 1.85 / 1.92 ms; a persistent grid striding over all
+    // tiles 2.02).
+    const long long tiles = (a.n + 15) / 16;
+    const long long stride = LINES_WAVES;
+    const long long first = (long long)blockIdx.x * LINES_WAVES * a.tiles_per_wave;
+    const long long tiles_end = min(tiles, first + (long long)LINES_WAVES * a.tiles_per_wave);
+    long long tile = first + wave;
+    const bool any_tile = tile < tiles_end;
+    if (!any_tile) tile = tiles - 1;  // stays for the barrier below; stores nothing
+    const float *x = static_cast<const float *>(a.x);
+    const int xr = lane / LR, xc = lane % LR;
+    v4f xin[NLD];
+    const auto issue = [&](long long t) {
+#pragma unroll
+        for (int j = 0; j < NLD; ++j) {
+            const long long row = min(t * 16 + j * RPI + xr, a.n - 1);
+            xin[j] = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(x + row * a.ld_x + 4 * xc));
+        }
+    };
+    issue(tile);  // the first tile's rows are on their way while W is copied
+    float scale = a.rs ? a.rs[min(tile * 16 + i, a.n - 1)] : 1.0f;
+    {  // a.w: the image k_wt_image made of W (Wt[column slot][k], rows of KP bf16), copied as it lies
+        typedef unsigned v4u_c __attribute__((ext_vector_type(4)));
+        const v4u_c *src = static_cast<const v4u_c *>(a.w);
+        v4u_c *dst = reinterpret_cast<v4u_c *>(lds_raw);
+        for (int idx = (int)threadIdx.x; idx < D2 * KP * 2 / 16; idx += LINES_WAVES * 64) dst[idx] = src[idx];
+    }
+    __syncthreads();
+
+    if (!any_tile) return;
+    for (;;) {
+#pragma unroll
+        for (int j = 0; j < NLD; ++j) {
+            const v2bf p0 = __builtin_convertvector((v2f){xin[j][0], xin[j][1]}, v2bf), p1 = __builtin_convertvector((v2f){xin[j][2], xin[j][3]}, v2bf);
+            unsigned pk[2];
+            __builtin_memcpy(&pk[0], &p0, 4);
+            __builtin_memcpy(&pk[1], &p1, 4);
+            *reinterpret_cast<v2u_s *>(mine + (j * RPI + xr) * XP + xc * 8) = (v2u_s){pk[0], pk[1]};
+        }
+        const long long ntile = tile + stride;
+        const bool more = ntile < tiles_end;
+        float scale_next = 1.0f;
+        if (more) {  // wavefront-uniform
+            issue(ntile);
+            if (a.rs) scale_next = a.rs[min(ntile * 16 + i, a.n - 1)];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        v4f acc[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < D1 / 32; ++ks) {
+            v8bf av;
+            av = *reinterpret_cast<const v8bf *>(mine + i * XP + (32 * ks + 8 * kb) * 2);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                v8bf bv;
+                bv = *reinterpret_cast<const v8bf *>(wt + (size_t)(nb * 16 + i) * KP + 32 * ks + 8 * kb);
+                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, av, acc[nb], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int p = 0; p < NB / 2; ++p) {
+            unsigned pk[4];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    v[r] = acc[2 * p + h][r] * scale;
+                    if (a.relu) v[r] = fmaxf(v[r], 0.f);
+                }
+                const v2bf q0 = __builtin_convertvector((v2f){v[0], v[1]}, v2bf), q1 = __builtin_convertvector((v2f){v[2], v[3]}, v2bf);
+                __builtin_memcpy(&pk[2 * h], &q0, 4);
+                __builtin_memcpy(&pk[2 * h + 1], &q1, 4);
+            }
+            *reinterpret_cast<v4u_s *>(mine + i * OP + (32 * p + 8 * kb) * 2) = (v4u_s){pk[0], pk[1], pk[2], pk[3]};
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        {
+            const int orow = lane / LRO, oc = lane % LRO;
+            char *out = static_cast<char *>(a.out);
+#pragma unroll
+            for (int j = 0; j < NST; ++j) {
+                const int r = j * RPO + orow;
+                const v4u_s v = *reinterpret_cast<const v4u_s *>(mine + r * OP + oc * 16);
+                const long long row = tile * 16 + r;
+                if (row < a.n)
+                    __builtin_nontemporal_store(v, reinterpret_cast<v4u_s *>(out + (row * a.ld_out) * 2 + oc * 16));
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (!more) break;
+        tile = ntile;
+        scale = scale_next;
     }
 }
 
@@ -867,6 +1029,37 @@ MGGX_EXPORT int mggx_dense_xw_bf16(void *d_out, const void *d_x, const void *d_w
     const size_t lds = (size_t)(nb * 16) * (((d1 + 31) & ~31) + 8) * 2;
     if (lds > 150 * 1024) return fail(MGGX_ELIMIT, "dense_xw_bf16: W tile of %zu bytes does not fit in LDS (d1 <= ~580 at 128 columns)", lds);
     hipStream_t stream = mggx::state().stream;
+    if (x_dtype == MGGX_F32 && out_dtype == MGGX_BF16 && (d1 == 64 || d1 == 128) && (d2 == 64 || d2 == 128) && n >= 4096 && (a.vec_out & 4) != 0 &&
+        a.ld_x % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15u) == 0) {
+        static unsigned short *image_of[16] = {};
+        int dev = -1;
+        MGGX_HIP(hipGetDevice(&dev));
+        if (dev < 0 || dev >= 16) return fail(MGGX_ELIMIT, "dense_xw_bf16: device index %d", dev);
+        if (!image_of[dev]) {
+            void *q = nullptr;
+            const hipError_t e = hipGetSymbolAddress(&q, HIP_SYMBOL(wt_image));
+            if (e != hipSuccess || !q) return fail(MGGX_EHIP, "dense_xw_bf16: hipGetSymbolAddress: %s", hipGetErrorString(e));
+            image_of[dev] = static_cast<unsigned short *>(q);
+        }
+        mggx::k_wt_image<<<dim3((unsigned)((d1 * d2 + 255) / 256)), dim3(256), 0, stream>>>(image_of[dev], static_cast<const unsigned short *>(d_w_bf16), d1, d2);
+        MGGX_LAUNCH_CHECK("k_wt_image");
+        a.w = image_of[dev];
+        a.tiles_per_wave = 8;
+        const long long tiles = (n + 15) / 16, per_wg = (long long)mggx::LINES_WAVES * a.tiles_per_wave;
+        const unsigned wgs = (unsigned)((tiles + per_wg - 1) / per_wg);
+        const auto launch = [&](auto kernel, int nb_, int d1_) {
+            const size_t tile_bytes = 16 * (size_t)std::max(d1_ * 2 + 16, nb_ * 32 + 16);
+            const size_t lds_lines = (size_t)(nb_ * 16) * (d1_ + 8) * 2 + mggx::LINES_WAVES * tile_bytes;
+            mggx::allow_lds(kernel, lds_lines);
+            kernel<<<dim3(wgs), dim3(mggx::LINES_WAVES * 64), lds_lines, stream>>>(a);
+        };
+        if (d1 == 128 && d2 == 128) launch(mggx::k_dense_xw_bf16_lines<8, 128>, 8, 128);
+        else if (d1 == 128) launch(mggx::k_dense_xw_bf16_lines<4, 128>, 4, 128);
+        else if (d2 == 128) launch(mggx::k_dense_xw_bf16_lines<8, 64>, 8, 64);
+        else launch(mggx::k_dense_xw_bf16_lines<4, 64>, 4, 64);
+        MGGX_LAUNCH_CHECK("k_dense_xw_bf16_lines");
+        return MGGX_OK;
+    }
     const dim3 grid(mggx::persistent_blocks(n), (unsigned)gy);
     if (x_dtype == MGGX_F32 && out_dtype == MGGX_F32) mggx::dispatch_nb<mggx::LaunchBf16<true, false>::L>(nb, grid, lds, stream, a);
     else if (x_dtype == MGGX_F32) mggx::dispatch_nb<mggx::LaunchBf16<true, true>::L>(nb, grid, lds, stream, a);
