@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the neighbor-partitioned aggregation path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gcn2|share|gin|big|copy|gather|vendor] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gcn2|share|gin|big|copy|convert|gather|vendor] [--no-cpu]
 
 Default workload (`gcn2`): 2-layer GCN forward on the whole graph -- seeded RMAT
 power-law graph (a=.57 b=.19 c=.19), 233,000 nodes, ~114 M undirected edges,
@@ -22,7 +22,8 @@ A result outside its tolerance against the CPU oracle makes the run fail.
 `share` times the aggregation alone on rank 0's 1/8 share of a 4.2 M-node RMAT
 graph with the remote rows pre-staged in a second HBM table; `gin` the 5-layer
 GIN forward; `big` the bf16 large-share aggregation and update; `copy` the
-stream-copy yardstick; `gather` the random-gather yardstick (what the memory system sustains for row gathers from
+stream-copy yardstick; `convert` the 2:1 read/write yardstick of the dense update (a bare fp32 -> bf16 conversion, by
+the order in which the workgroups walk through memory); `gather` the random-gather yardstick (what the memory system sustains for row gathers from
 tables of the benchmark sizes); `vendor` the library's kernels beside torch.mm and
 torch.sparse.mm on the benchmark shapes.
 """
@@ -1068,6 +1069,37 @@ def bench_copy(args, torch, host):
             "detail": detail}
 
 
+def bench_convert(args, torch, host):
+    """fp32 -> bf16 conversion of the large share's 13.9 M x 128 table, nothing else: what the memory system gives the dense
+    update's 2 : 1 read / write stream, by the order in which the chip walks through the arrays -- workgroups in launch order
+    with 1 ... 64 consecutive pieces of 8 KB each, and persistent grids striding over everything."""
+    n = (13_875_000 >> args.big_scale) * 128
+    src = torch.randn(n, device="cuda")
+    dst = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+    cases = [("launch order, %d piece%s of 8 KB per workgroup" % (c, "" if c == 1 else "s"), c, 0) for c in (1, 2, 4, 8, 16, 64)] + \
+            [("persistent grid of %d workgroups striding over all pieces" % g, 1, g) for g in (2048, 8192)]
+    detail = {}
+    for name, per_wg, persistent in cases:
+        fn = lambda: host.convert_probe(dst, src, n, per_wg, persistent)
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        timer = StageTimer(torch, [name], args.steps)
+        for _ in range(args.steps):
+            timer.step([fn])
+        ms = timer.medians()[name]
+        detail[name] = {"ms": round(ms, 4), "gbps": round(6 * n / (ms * 1e-3) / 1e9, 1), "frac_of_hbm_peak": round(6 * n / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+        log(name, detail[name])
+    want = (src[:4096].view(torch.int32) >> 16).to(torch.int16)
+    assert bool((dst[:4096].view(torch.int16) == want).all()) and bool((dst[-4096:].view(torch.int16) == (src[-4096:].view(torch.int32) >> 16).to(torch.int16)).all())
+    best = max(detail, key=lambda k: detail[k]["gbps"])
+    return {"metric": "convert_stream_gbps", "value": detail[best]["gbps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": detail[best]["ms"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "fp32 -> bf16 conversion of %d values (%d bytes read, %d written per launch); best: %s" % (n, 4 * n, 2 * n, best)},
+            "detail": detail}
+
+
 def bench_gather(args, torch, host):
     """Random row gathers from tables of the benchmark shapes, with no index stream and no reduction: what the memory
     system sustains for the access pattern of the aggregation at each table size (the ceiling for cache-resident
@@ -1108,7 +1140,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20,
                     help="untimed steps before the timed ones (default 20: a dense-core plan built a moment ago runs up to 10 %% slower "
                          "for its first twenty calls)")
-    ap.add_argument("--workload", default="gcn2", choices=["gcn2", "share", "gin", "big", "copy", "gather", "vendor"])
+    ap.add_argument("--workload", default="gcn2", choices=["gcn2", "share", "gin", "big", "copy", "convert", "gather", "vendor"])
     ap.add_argument("--ps", type=int, default=16, help="partSize; 0 = let the library choose (the search then tries 16 and 32)")
     ap.add_argument("--col-block-rows", type=int, default=0, help="column-blocked partition order: 0 = library decides, -1 = off, "
                          "N = blocks of N neighbor ids")
@@ -1148,7 +1180,7 @@ def main():
         host.set_plan_check(0)
     log("device:", host.device_name())
     res = {"gcn2": bench_gcn2, "share": bench_share, "gin": bench_gin, "big": bench_big, "copy": bench_copy,
-           "gather": bench_gather, "vendor": bench_vendor}[args.workload](args, torch, host)
+           "convert": bench_convert, "gather": bench_gather, "vendor": bench_vendor}[args.workload](args, torch, host)
     checks = res.pop("_checks", None)
     if checks:
         fail_on_parity(res, checks)

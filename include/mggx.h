@@ -393,6 +393,13 @@ int mggx_copy_bytes(void *d_dst, const void *d_src, size_t n);
  * second copy kernel, so the copy ceiling quoted beside the bandwidth-bound kernels does not rest on one variant. */
 int mggx_copy_bytes_nt(void *d_dst, const void *d_src, size_t n);
 
+/* Yardstick for a 2 : 1 read / write stream (no counterpart in the reference): n fp32 values (n % 8 == 0, both arrays on
+ * 16-byte boundaries) to bf16 by truncation, 32 bytes in and 16 bytes out per lane with the streaming hint, in pieces of
+ * 2048 values.  persistent_workgroups = 0: workgroups in launch order, each converting pieces_per_workgroup consecutive
+ * pieces one after the other; > 0: that many workgroups striding over all pieces.  What the dense update's access
+ * pattern is measured against: the order in which the chip walks through memory decides 6.2 against 5.1 TB/s. */
+int mggx_convert_probe(void *d_dst, const float *d_src, int64_t n, int pieces_per_workgroup, int persistent_workgroups);
+
 /* Yardstick for row gathers (no counterpart in the reference): at least n_gathers loads of row_bytes bytes (16..256, in
  * 16-byte pieces) from rows at pseudo-random indices of a table of `rows` rows with a stride of ld_bytes, eight loads in
  * flight per lane group, no index array and no reduction; *n_done (optional) receives the exact number issued.  d_sink

@@ -331,6 +331,27 @@ __global__ void __launch_bounds__(256) k_cast_bf16(unsigned short *__restrict__ 
     }
 }
 
+// Yardstick: fp32 -> bf16 (truncated) of n8 groups of 8 values, 32 bytes in and 16 out per lane with the streaming hint.
+// Pieces of 2048 values (8 KB in, 4 KB out) per round of a workgroup; workgroup b takes pieces [b * per_wg, (b + 1) * per_wg)
+// one after the other, or, with stride_pieces > 0, pieces b, b + stride_pieces, ... (a persistent grid).
+__global__ void __launch_bounds__(256) k_convert_probe(unsigned *__restrict__ dst, const float *__restrict__ src, long long n8, long long pieces,
+                                                       int per_wg, long long stride_pieces)
+{
+    typedef float v4f_p __attribute__((ext_vector_type(4)));
+    typedef unsigned v4u_p __attribute__((ext_vector_type(4)));
+    const auto pack = [](float a, float b) { return (__float_as_uint(a) >> 16) | (__float_as_uint(b) & 0xFFFF0000u); };
+    long long piece = stride_pieces > 0 ? (long long)blockIdx.x : (long long)blockIdx.x * per_wg;
+    const long long end = stride_pieces > 0 ? pieces : min(pieces, piece + per_wg), step = stride_pieces > 0 ? stride_pieces : 1;
+    for (; piece < end; piece += step) {
+        const long long i = piece * 256 + threadIdx.x;
+        if (i >= n8) continue;
+        const v4f_p a = __builtin_nontemporal_load(reinterpret_cast<const v4f_p *>(src) + 2 * i);
+        const v4f_p b = __builtin_nontemporal_load(reinterpret_cast<const v4f_p *>(src) + 2 * i + 1);
+        const v4u_p o = {pack(a.x, a.y), pack(a.z, a.w), pack(b.x, b.y), pack(b.z, b.w)};
+        __builtin_nontemporal_store(o, reinterpret_cast<v4u_p *>(dst) + i);
+    }
+}
+
 // dst row i = table row ids[i]; rows of v16 16-byte pieces
 __global__ void __launch_bounds__(256) k_gather_rows(int4 *__restrict__ dst, const int4 *__restrict__ table, const int *__restrict__ ids,
                                                      long long n, int v16)
@@ -538,6 +559,21 @@ MGGX_EXPORT int mggx_cast_f32_to_bf16(void *d_dst, const float *d_src, int64_t n
     if (blocks > 256 * 64) blocks = 256 * 64;
     k_cast_bf16<<<dim3((unsigned)blocks), dim3(256), 0, state().stream>>>((unsigned short *)d_dst, d_src, (long long)n);
     MGGX_LAUNCH_CHECK("k_cast_bf16");
+    return MGGX_OK;
+}
+
+MGGX_EXPORT int mggx_convert_probe(void *d_dst, const float *d_src, int64_t n, int pieces_per_workgroup, int persistent_workgroups)
+{
+    if (n < 0 || n % 8 || pieces_per_workgroup < 1 || persistent_workgroups < 0 || (n && (!d_dst || !d_src)) ||
+        (reinterpret_cast<uintptr_t>(d_dst) & 15u) || (reinterpret_cast<uintptr_t>(d_src) & 15u))
+        return fail(MGGX_EINVAL, "convert_probe: bad argument");
+    if (!n) return MGGX_OK;
+    const long long n8 = n / 8, pieces = (n8 + 255) / 256;
+    const long long wgs = persistent_workgroups ? std::min<long long>(persistent_workgroups, pieces) : (pieces + pieces_per_workgroup - 1) / pieces_per_workgroup;
+    if (wgs > 0x7fffffffLL) return fail(MGGX_ELIMIT, "convert_probe: too many workgroups");
+    k_convert_probe<<<dim3((unsigned)wgs), dim3(256), 0, state().stream>>>((unsigned *)d_dst, d_src, n8, pieces, pieces_per_workgroup,
+                                                                          persistent_workgroups ? wgs : 0);
+    MGGX_LAUNCH_CHECK("k_convert_probe");
     return MGGX_OK;
 }
 

@@ -59,7 +59,7 @@ EXPORTS = [
     "mggx_last_error", "mggx_version", "mggx_init", "mggx_device_name", "mggx_set_stream", "mggx_sync",
     "mggx_malloc", "mggx_malloc_tables", "mggx_free", "mggx_memset", "mggx_memcpy_h2d", "mggx_memcpy_d2h", "mggx_memcpy_d2d",
     "mggx_timer_create", "mggx_timer_start", "mggx_timer_stop", "mggx_timer_elapsed_ms", "mggx_timer_destroy",
-    "mggx_release_cached", "mggx_forget", "mggx_set_plan_check", "mggx_cache_stats", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_core_layout_build", "mggx_core_layout_fetch", "mggx_core_layout_device", "mggx_graph_read",
+    "mggx_release_cached", "mggx_forget", "mggx_set_plan_check", "mggx_cache_stats", "mggx_range_partition", "mggx_split_csr", "mggx_compact_remote", "mggx_build_part", "mggx_core_layout_build", "mggx_core_layout_fetch", "mggx_core_layout_device", "mggx_convert_probe", "mggx_graph_read",
     "mggx_graph_write", "mggx_mtx_read", "mggx_gen_rmat", "mggx_gen_er", "mggx_gen_fetch", "mggx_fill_normal",
     "mggx_fill_uniform", "mggx_build_part_device", "mggx_split_csr_device", "mggx_compact_remote_device", "mggx_edgelist_to_bin", "mggx_sag_np_div", "mggx_sag_np_div_tune", "mggx_sag_parts", "mggx_sag_parts_static", "mggx_mlp2_xw", "mggx_spmm",
     "mggx_dense_xw", "mggx_dense_xw_bf16", "mggx_softmax_rows", "mggx_cast_f32_to_bf16", "mggx_copy_bytes", "mggx_copy_bytes_nt", "mggx_gather_probe", "mggx_lds_probe", "mggx_gather_rows", "mggx_last_agg_kernel", "mggx_set_gather_addressing",
@@ -491,6 +491,11 @@ def copy_bytes(dst, src, nbytes: int) -> None:
 
 def copy_bytes_nt(dst, src, nbytes: int) -> None:
     _check(lib().mggx_copy_bytes_nt(_dptr(dst), _dptr(src), C.c_size_t(nbytes)))
+
+
+def convert_probe(dst, src, n: int, pieces_per_workgroup: int = 1, persistent_workgroups: int = 0) -> None:
+    """fp32 -> bf16 (truncated) streaming conversion of n values: the 2:1 read/write yardstick of the dense update."""
+    _check(lib().mggx_convert_probe(_dptr(dst), _dptr(src), C.c_int64(n), pieces_per_workgroup, persistent_workgroups))
 
 
 def gather_probe(sink, table, rows: int, ld_bytes: int, row_bytes: int, n_gathers: int, seed: int = 1) -> int:
