@@ -801,9 +801,10 @@ __global__ void __launch_bounds__(256) k_agg_tail(const AggArgs a, int num_wg, i
 // plan's row offsets, so no fix-up pass, no zero fill and no separate reduction run.  G lanes per row (a power of two
 // >= dim/4), lane q holds columns 4 q .. 4 q + 3; the epilogue is the caller's (row scale, accumulate, ReLU, softmax).
 struct CoreMergeArgs {
-    const float4 *partial;  // [slot][CORE_GROUP_ROWS][n4] or NULL
+    const float4 *partial;  // [slot][group_rows][n4] or NULL
     const int *rank;        // [rows]: rank in the core or -1
-    const int *wg_base;     // [core / CORE_GROUP_ROWS + 1]: the slots of row group g are wg_base[g] .. wg_base[g + 1] - 1
+    const int *wg_base;     // [core / group_rows + 1]: the slots of row group g are wg_base[g] .. wg_base[g + 1] - 1
+    int group_rows;         // core rows per workgroup of the LDS kernel (CorePlan::group_rows)
 };
 
 __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp, int G,
@@ -853,11 +854,11 @@ __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, con
         if (cm.partial) {
             const int r = cm.rank[v];
             if (r >= 0) {
-                const int grp = r / CORE_GROUP_ROWS;
+                const int grp = r / cm.group_rows;
                 int slot = cm.wg_base[grp];
                 const int slot_end = cm.wg_base[grp + 1];
-                const size_t stride = (size_t)CORE_GROUP_ROWS * n4;
-                const float4 *src = cm.partial + (size_t)(r % CORE_GROUP_ROWS) * n4 + q;
+                const size_t stride = (size_t)cm.group_rows * n4;
+                const float4 *src = cm.partial + (size_t)(r % cm.group_rows) * n4 + q;
                 for (; slot + 4 <= slot_end; slot += 4) {  // four partial rows in flight, summed in order
                     const float4 p0 = src[(size_t)slot * stride], p1 = src[(size_t)(slot + 1) * stride];
                     const float4 p2 = src[(size_t)(slot + 2) * stride], p3 = src[(size_t)(slot + 3) * stride];
@@ -941,6 +942,7 @@ struct CoreMerge {
     const float4 *partial;
     const int *rank;
     const int *wg_base;
+    int group_rows;
     hipEvent_t join;
     bool merged;
 };
@@ -985,7 +987,8 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     const int slots = 64 / lpr;
     // 0 = let the library choose.  Few slots per wavefront (wide rows): 8 wavefronts and 16 rounds, so a workgroup still
     // covers a few thousand neighbors; column-blocked plans: 4 wavefronts (they share the chip with the dense core's
-    // 4-wavefront workgroups); in row-major order beside a dense core: 8 wavefronts and 4 rounds; short rows (under 3
+    // 4-wavefront workgroups); in row-major order beside a dense core: 8 wavefronts and 4 rounds (8 rounds are 2.4 % faster
+    // on the 2.45 M-node graph at width 64 and 9 % slower on a 700 K-node one of the same width); short rows (under 3
     // partitions per row): 4 wavefronts.  Many slots (narrow rows): 4 wavefronts, 4 rounds; 8 rounds where a column-blocked
     // plan is left with short rows (under 8 partitions per row and block).
     // Provenance: wpb x dist sweeps on the three benchmark graphs and the bf16 share (each choice within 1 % of the best
@@ -1121,10 +1124,10 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         r.ld_out = ld_out;
         r.rs_out = o.d_row_scale_out;
         r.flags = o.flags;
-        CoreMergeArgs cma{nullptr, nullptr, nullptr};
+        CoreMergeArgs cma{nullptr, nullptr, nullptr, CORE_GROUP_ROWS};
         if (cm) {
             MGGX_HIP(hipStreamWaitEvent(st.stream, cm->join, 0));
-            cma = CoreMergeArgs{cm->partial, cm->rank, cm->wg_base};
+            cma = CoreMergeArgs{cm->partial, cm->rank, cm->wg_base, cm->group_rows};
             cm->merged = true;
         }
         const int G = pow2_ceil((dim + 3) / 4);
@@ -1218,7 +1221,7 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
     if (k.core_rows > 0 && ub - lb >= 1024 && g.nnz_r == 0 && g.nnz_l > 0 && d_col_l && o.in_dtype == MGGX_F32 && dim >= 1 && dim <= 64 && d_out &&
         d_in_local) {
         CorePlan *cp = nullptr;
-        rc = core_plan_get(d_ptr_l, d_col_l, ub - lb, lb, k.core_rows, g.serial, &cp);
+        rc = core_plan_get(d_ptr_l, d_col_l, ub - lb, lb, k.core_rows, core_group_rows((dim + 3) / 4, std::min(k.core_rows, ub - lb)), g.serial, &cp);
         if (rc) return rc;
         if (!cp->unsuitable) {
             // The core block is bound by the LDS, the rest of the CSR by the caches: they run side by side.  The core's sums
@@ -1241,7 +1244,7 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
             const hipError_t er = hipEventRecord(join, side);
             int rc2 = MGGX_OK;
             GraphInfo *gr = nullptr;
-            CoreMerge cm{nullptr, cp->d_rank, nullptr, join, false};
+            CoreMerge cm{nullptr, cp->d_rank, nullptr, cp->group_rows, join, false};
             if (!rc) rc2 = core_partial_rows(cp, dim, &cm.partial, &cm.wg_base);
             if (!rc && !rc2) rc2 = graph_info(cp->d_rem_ptr, nullptr, cp->d_rem_col, nullptr, ub - lb, true, &gr);
             if (!rc && !rc2 && er == hipSuccess) {

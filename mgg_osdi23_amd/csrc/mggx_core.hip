@@ -48,9 +48,12 @@ __device__ __forceinline__ void static_for_core(F &&f)
 }
 
 constexpr int CORE_TC = 256;    // core columns per LDS tile
-constexpr int CORE_WAVES = CORE_GROUP_ROWS / 64;  // slices (of 64 rows) per workgroup: as small as the aggregation's own
-                                                  // workgroups, so the two kernels of a call, running side by side, find
-                                                  // room on a CU equally easily
+// Slices (of 64 rows) per workgroup, WAVES below: 4 -- as small as the aggregation's own workgroups, so the two kernels
+// of a call, running side by side, find room on a CU equally easily -- or 8 where rows are summed in two halves: every
+// workgroup stages every tile of its run, so the tiles staged per call are (row groups) x (tiles); with 98,304 core rows
+// of 256 bytes that is 9.7 GB of L2 reads per call at 4 slices and half of it at 8 (2.45 M-node graph, width 64: 2.93 ->
+// 2.68 ms per aggregation with two 8-wavefront workgroups per CU; one 16-wavefront workgroup: 2.66; at widths 16 and 44 on
+// the 233 K-node graph, whose 15 / 45 MB tables sit in the L2, 8 slices cost 15 and 33 %).
 
 // tab[s * tab_stride(core) + i] = elements 4 s .. 4 s + 3 of the feature row of the rank-i node (zero past dim)
 __global__ void __launch_bounds__(256) k_core_stage(v4f *__restrict__ tab, const float *__restrict__ in, const int *__restrict__ order,
@@ -70,14 +73,14 @@ __global__ void __launch_bounds__(256) k_core_stage(v4f *__restrict__ tab, const
 }
 
 // The body for the 16-byte pieces [S0, S0 + NS) of rows of N4 pieces.
-template <int N4, int S0, int NS>
+template <int N4, int S0, int NS, int WAVES>
 __device__ __forceinline__ void core_sell_body(const unsigned *__restrict__ blk_off, const unsigned short *__restrict__ idx,
                                                const v4f *__restrict__ tab, v4f *__restrict__ partial, const int4 wg, int core, int ntiles,
                                                v4f *tile)
 {
     constexpr int TC = CORE_TC, TP = TC + 1;  // column TC of every slice row is zero: what padding entries read; tile[NS][TP]
     const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
-    const int g = wg.x * CORE_WAVES + wave;
+    const int g = wg.x * WAVES + wave;
     const int t0 = wg.y, t1 = wg.z;
     v4f acc[NS];
 #pragma unroll
@@ -90,7 +93,7 @@ __device__ __forceinline__ void core_sell_body(const unsigned *__restrict__ blk_
     us4 cur = pos < end_run ? p[(size_t)pos * 64] : pad;  // the lists of a slice's tiles follow one another: read one chunk ahead
     for (int t = t0; t < t1; ++t) {
         __syncthreads();
-        for (int i = (int)threadIdx.x; i < NS * TC; i += CORE_WAVES * 64) {
+        for (int i = (int)threadIdx.x; i < NS * TC; i += WAVES * 64) {
             const int s = i / TC, c = i % TC;
             tile[s * TP + c] = tab[(size_t)(S0 + s) * tab_stride(core) + (size_t)t * TC + c];
         }
@@ -116,19 +119,19 @@ __device__ __forceinline__ void core_sell_body(const unsigned *__restrict__ blk_
             ++pos;
         }
     }
-    const size_t r = (size_t)wg.w * (CORE_WAVES * 64) + (size_t)(wave * 64 + lane);
+    const size_t r = (size_t)wg.w * (WAVES * 64) + (size_t)(wave * 64 + lane);
 #pragma unroll
     for (int s = 0; s < NS; ++s) partial[r * N4 + S0 + s] = acc[s];
 }
 
-// One workgroup = CORE_WAVES slices (a row group) x a run of column tiles [x all pieces of the rows, or one half of
+// One workgroup = WAVES slices (a row group) x a run of column tiles [x all pieces of the rows, or one half of
 // them when SPLIT: blockIdx.y]; lane = core row.  Row groups and tiles are both sorted by degree, so the work of a
 // (row group, tile) cell spans two orders of magnitude: the plan cuts every row group's tiles into runs of about equal
 // list length (wgs[i] = {row group, first tile, end tile, slot}), so all workgroups take about the same time and the
 // launch has no tail of a few heavy ones.
-// partial[(slot * CORE_WAVES * 64 + row in the group) * N4 + s]
-template <int N4, bool SPLIT>
-__global__ void __launch_bounds__(CORE_WAVES * 64) MGGX_CORE_OCCUPANCY k_core_sell(const unsigned *__restrict__ blk_off, const unsigned short *__restrict__ idx,
+// partial[(slot * WAVES * 64 + row in the group) * N4 + s]
+template <int N4, bool SPLIT, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64) MGGX_CORE_OCCUPANCY k_core_sell(const unsigned *__restrict__ blk_off, const unsigned short *__restrict__ idx,
                                                                const v4f *__restrict__ tab, v4f *__restrict__ partial,
                                                                const int4 *__restrict__ wgs, int core, int ntiles, const Gate gate)
 {
@@ -136,11 +139,11 @@ __global__ void __launch_bounds__(CORE_WAVES * 64) MGGX_CORE_OCCUPANCY k_core_se
     if (gate_closed(gate)) return;
     const int4 wg = wgs[blockIdx.x];
     if constexpr (!SPLIT) {
-        core_sell_body<N4, 0, N4>(blk_off, idx, tab, partial, wg, core, ntiles, tile);
+        core_sell_body<N4, 0, N4, WAVES>(blk_off, idx, tab, partial, wg, core, ntiles, tile);
     } else {
         constexpr int A = (N4 + 1) / 2;
-        if (blockIdx.y == 0) core_sell_body<N4, 0, A>(blk_off, idx, tab, partial, wg, core, ntiles, tile);
-        else core_sell_body<N4, A, N4 - A>(blk_off, idx, tab, partial, wg, core, ntiles, tile);
+        if (blockIdx.y == 0) core_sell_body<N4, 0, A, WAVES>(blk_off, idx, tab, partial, wg, core, ntiles, tile);
+        else core_sell_body<N4, A, N4 - A, WAVES>(blk_off, idx, tab, partial, wg, core, ntiles, tile);
     }
 }
 
@@ -151,8 +154,8 @@ __global__ void __launch_bounds__(CORE_WAVES * 64) MGGX_CORE_OCCUPANCY k_core_se
 // (index -> rank -> row); all_rows = 1: every row (needed when there is a post-operation).
 __global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, const v4f *__restrict__ partial, const int *__restrict__ rank,
                                                      const int *__restrict__ order, const float *__restrict__ rs, int rows, int dim,
-                                                     long long ld_out, int core, const int *__restrict__ wg_base, int G, int relu, int softmax,
-                                                     int all_rows, const Gate gate)
+                                                     long long ld_out, int core, const int *__restrict__ wg_base, int group_rows, int G, int relu,
+                                                     int softmax, int all_rows, const Gate gate)
 {
     if (gate_closed(gate)) return;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -169,9 +172,9 @@ __global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, co
     if (lane_on) {
         v4f sum = {0.f, 0.f, 0.f, 0.f};
         if (r >= 0) {
-            const int grp = r / (CORE_WAVES * 64), in_grp = r % (CORE_WAVES * 64);
+            const int grp = r / group_rows, in_grp = r % group_rows;
             const int s1 = wg_base[grp + 1];
-            for (int slot = wg_base[grp]; slot < s1; ++slot) sum += partial[((size_t)slot * (CORE_WAVES * 64) + in_grp) * n4 + q];
+            for (int slot = wg_base[grp]; slot < s1; ++slot) sum += partial[((size_t)slot * group_rows + in_grp) * n4 + q];
             if (rs) sum *= rs[v];
         }
 #pragma unroll
@@ -287,14 +290,14 @@ __global__ void __launch_bounds__(256) k_core_widths(const unsigned short *__res
     chunks[idx] = (w + 3) / 4;
 }
 
-// work[g * ntiles + t] = list chunks of the CORE_WAVES slices of row group g in tile t
-__global__ void __launch_bounds__(256) k_core_group_work(const int *__restrict__ chunks, int groups, int ntiles, int *__restrict__ work)
+// work[g * ntiles + t] = list chunks of the `waves` slices of row group g in tile t
+__global__ void __launch_bounds__(256) k_core_group_work(const int *__restrict__ chunks, int groups, int ntiles, int waves, int *__restrict__ work)
 {
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (long long)groups * ntiles) return;
     const int g = (int)(idx / ntiles), t = (int)(idx % ntiles);
     int w = 0;
-    for (int k = 0; k < CORE_WAVES; ++k) w += chunks[(size_t)(g * CORE_WAVES + k) * ntiles + t];
+    for (int k = 0; k < waves; ++k) w += chunks[(size_t)(g * waves + k) * ntiles + t];
     work[idx] = w;
 }
 
@@ -370,26 +373,35 @@ __global__ void __launch_bounds__(BUILD_WAVES * 64) k_core_fill(const int *__res
 }
 
 // Rows of more than 192 bytes are summed in two halves by two workgroups (blockIdx.y): half the accumulators per lane
-// (81 instead of 119 registers at 256 bytes), at the price of walking the index lists twice.  Three such workgroups per
-// CU, which a request of a little over a quarter of the LDS enforces, leave the aggregation beside them the room it had
-// (measured on the 2.45 M-node graph at width 64: 3.01 ms whole, 2.92 ms in halves with three per CU; 3.21 with four,
-// 2.97 with two; at width 44 halves gain nothing: 1.42 against 1.40 ms).
-template <int N4>
-int launch_sell(const CorePlan *p, const CorePlan::Cut &cut, const v4f *tab, v4f *partial, const Gate &gate, hipStream_t stream)
+// (81 instead of 119 registers at 256 bytes), at the price of walking the index lists twice.  Their workgroups have 8
+// wavefronts (see WAVES above) and ask for a third of the LDS, which holds a CU to two of them -- 16 wavefronts of this
+// kernel -- and leaves the aggregation beside them the room it had (2.45 M-node graph, width 64, per aggregation:
+// whole rows 3.01 ms; halves, 4 wavefronts, three workgroups per CU 2.92; halves, 8 wavefronts, two per CU 2.68, one per
+// CU 3.05; at width 44 halves gain nothing: 1.42 against 1.40 ms).
+template <int N4, int WAVES>
+int launch_sell_as(const CorePlan *p, const CorePlan::Cut &cut, const v4f *tab, v4f *partial, const Gate &gate, hipStream_t stream)
 {
     constexpr bool SPLIT = N4 > 12;
     constexpr int NS = SPLIT ? (N4 + 1) / 2 : N4;
     size_t lds = (size_t)NS * (CORE_TC + 1) * sizeof(v4f);
-    if (SPLIT) lds = std::max<size_t>(lds, (160u << 10) / 4 + 256);
+    if (SPLIT) lds = std::max<size_t>(lds, (160u << 10) / (WAVES == 8 ? 3 : 4) + 256);
     static bool raised = false;  // per instantiation
     if (lds > 48 * 1024 && !raised) {
-        MGGX_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_core_sell<N4, SPLIT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        MGGX_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_core_sell<N4, SPLIT, WAVES>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         raised = true;
     }
-    k_core_sell<N4, SPLIT><<<dim3((unsigned)cut.nwg, SPLIT ? 2u : 1u), dim3(CORE_WAVES * 64), lds, stream>>>(p->d_blk_off, p->d_idx, tab, partial, cut.d_wgs,
-                                                                                                          p->core, p->ntiles, gate);
+    k_core_sell<N4, SPLIT, WAVES><<<dim3((unsigned)cut.nwg, SPLIT ? 2u : 1u), dim3(WAVES * 64), lds, stream>>>(p->d_blk_off, p->d_idx, tab, partial, cut.d_wgs,
+                                                                                                            p->core, p->ntiles, gate);
     MGGX_LAUNCH_CHECK("k_core_sell");
     return MGGX_OK;
+}
+template <int N4>
+int launch_sell(const CorePlan *p, const CorePlan::Cut &cut, const v4f *tab, v4f *partial, const Gate &gate, hipStream_t stream)
+{
+    if (p->group_rows == CORE_GROUP_ROWS) return launch_sell_as<N4, CORE_GROUP_ROWS / 64>(p, cut, tab, partial, gate, stream);
+    if constexpr (N4 > 12)
+        if (p->group_rows == CORE_GROUP_ROWS_WIDE) return launch_sell_as<N4, CORE_GROUP_ROWS_WIDE / 64>(p, cut, tab, partial, gate, stream);
+    return fail(MGGX_EINVAL, "core: a plan with row groups of %d rows for rows of %d pieces", p->group_rows, N4);
 }
 
 // A plan that was used inside a stream capture: a captured graph still holds the addresses of its arrays, so they are
@@ -500,7 +512,7 @@ static int core_plan_build_device(CorePlan *p, int tc)
     if ((rc = tmp.get(&deg, (size_t)rows)) || (rc = tmp.get(&deg_sorted, (size_t)rows)) || (rc = tmp.get(&ids, (size_t)rows)) ||
         (rc = tmp.get(&sorted, (size_t)rows)) || (rc = tmp.get(&keep, (size_t)rows)) || (rc = tmp.get(&chunks, (size_t)nslices * ntiles)) ||
         (rc = tmp.get(&flag, 1)) || (rc = tmp.get(&cnt, (size_t)core * ntiles)) || (rc = tmp.get(&blk, (size_t)nslices * ntiles + 1)) ||
-        (rc = tmp.get(&work, (size_t)(nslices / CORE_WAVES) * ntiles)))
+        (rc = tmp.get(&work, (size_t)(nslices / (p->group_rows / 64)) * ntiles)))
         return rc;
     if ((rc = device_array(&p->d_order, (size_t)core)) || (rc = device_array(&p->d_rank, (size_t)rows)) ||
         (rc = device_array(&p->d_blk_off, (size_t)nslices * ntiles + 1)) || (rc = device_array(&p->d_rem_ptr, (size_t)rows + 1)))
@@ -548,8 +560,8 @@ static int core_plan_build_device(CorePlan *p, int tc)
     p->core_nnz = (int64_t)nnz - rem_nnz;
     // What cutting the LDS kernel's work into workgroups needs later: one number per (row group, tile), reduced on the GPU
     // (64 KB for a core of 32,768 rows)
-    const int groups = core / CORE_GROUP_ROWS;
-    k_core_group_work<<<(unsigned)(((long long)groups * ntiles + 255) / 256), 256, 0, s.stream>>>(chunks, groups, ntiles, work);
+    const int groups = core / p->group_rows;
+    k_core_group_work<<<(unsigned)(((long long)groups * ntiles + 255) / 256), 256, 0, s.stream>>>(chunks, groups, ntiles, p->group_rows / 64, work);
     MGGX_LAUNCH_CHECK("k_core_group_work");
     p->work.resize((size_t)groups * ntiles);
     MGGX_HIP(hipMemcpyAsync(p->work.data(), work, p->work.size() * sizeof(int), hipMemcpyDeviceToHost, s.stream));
@@ -559,14 +571,14 @@ static int core_plan_build_device(CorePlan *p, int tc)
     return MGGX_OK;
 }
 
-int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, int graph_serial, CorePlan **out)
+int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, int group_rows, int graph_serial, CorePlan **out)
 {
     State &s = state();
     for (size_t i = 0; i < s.cores.size(); ++i) {
         CorePlan *p = s.cores[i];
         // a plan belongs to the graph record it was built under (see drop_plans_of_record): it carries its own copy of that
         // graph's remaining CSR and index lists, and a later record of the same addresses may stand for another graph
-        if (p->d_ptr_l == d_ptr_l && p->d_col_l == d_col_l && p->rows == rows && p->lb == lb && p->asked == core && p->graph_serial == graph_serial) {
+        if (p->d_ptr_l == d_ptr_l && p->d_col_l == d_col_l && p->rows == rows && p->lb == lb && p->asked == core && p->group_rows == group_rows && p->graph_serial == graph_serial) {
             if (i + 1 != s.cores.size()) {  // most recently used last
                 s.cores.erase(s.cores.begin() + (long)i);
                 s.cores.push_back(p);
@@ -587,6 +599,7 @@ int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int 
     p->rows = rows;
     p->lb = lb;
     p->asked = core;
+    p->group_rows = group_rows;
     p->graph_serial = graph_serial;
     int rc = core_plan_build_device(p, CORE_TC);
     if (rc) {
@@ -627,7 +640,7 @@ static int core_cut(CorePlan *p, int n4, const CorePlan::Cut **out)
             return MGGX_OK;
         }
     if (capturing()) return fail(MGGX_EINVAL, "core: first use of this core with rows of this width inside a stream capture; call once outside the capture first");
-    const int groups = p->core / CORE_GROUP_ROWS, ntiles = p->ntiles;
+    const int groups = p->core / p->group_rows, ntiles = p->ntiles;
     const long long target = std::max<long long>((p->total_chunks + want - 1) / want, 1);
     std::vector<int4> runs;  // row-group-major: slot order
     std::vector<int> wg_base((size_t)groups + 1, 0);
@@ -685,7 +698,7 @@ static int core_scratch(CorePlan *p, int n4, v4f **tab, v4f **partial, const Cor
     if (rc_cut) return rc_cut;
     if (cut_out) *cut_out = cut;
     const size_t tab_bytes = (tab_stride(p->core) * n4 * sizeof(v4f) + 255) & ~(size_t)255;
-    const size_t part_bytes = (size_t)cut->nwg * CORE_GROUP_ROWS * n4 * sizeof(v4f);
+    const size_t part_bytes = (size_t)cut->nwg * p->group_rows * n4 * sizeof(v4f);
     if (tab_bytes + part_bytes > s.core_ws_bytes) {
         if (capturing()) return fail(MGGX_EINVAL, "core: the scratch block would have to grow inside a stream capture; run the largest call once outside it first");
         MGGX_HIP(hipDeviceSynchronize());  // both streams may still use the old block
@@ -757,7 +770,7 @@ int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const 
     while (G < n4) G <<= 1;
     const long long n = (long long)(all_rows ? p->rows : p->core) * G;
     k_core_finish<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(d_out, partial, p->d_rank, p->d_order, d_row_scale, p->rows, dim, ld_out,
-                                                                                p->core, cut->d_wg_base, G, relu, softmax, all_rows, gate);
+                                                                                p->core, cut->d_wg_base, p->group_rows, G, relu, softmax, all_rows, gate);
     MGGX_LAUNCH_CHECK("k_core_finish");
     return MGGX_OK;
 }
@@ -807,7 +820,10 @@ namespace mggx {
 namespace {
 
 constexpr int PROFILE_SLICES = 2048;  // 131072 ranks
-constexpr double ALPHA_PS = 1.40, BETA_PS = 9.0, HALVES = 0.7, F_CACHE = 3.0, F_MEMORY = 4.0;
+#ifndef MGGX_HALVES_WIDE
+#define MGGX_HALVES_WIDE 0.62
+#endif
+constexpr double ALPHA_PS = 1.40, BETA_PS = 9.0, HALVES = 0.7, HALVES_WIDE = MGGX_HALVES_WIDE, F_CACHE = 3.0, F_MEMORY = 4.0;
 constexpr unsigned long long L2_BYTES = 4ull << 20, LAST_LEVEL_CACHE_BYTES = 256ull << 20;
 constexpr int MODEL_STEP = 4096, MODEL_MAX_CORE = 98304;
 
@@ -905,7 +921,10 @@ int predict_core_rows(GraphInfo &g, int dim, unsigned long long table_bytes, int
     if (rc) return rc;
     const int n4 = (dim + 3) / 4;
     const int sectors = (dim * 4 + 63) / 64;
-    const double entry = ALPHA_PS * n4 * (n4 > 12 ? HALVES : 1.0);  // per padded list entry
+    // per padded list entry; rows in halves are cheaper beside the gather kernel, and cheaper again in wide row groups
+    const auto entry_at = [&](int k) {
+        return ALPHA_PS * n4 * (n4 > 12 ? (core_group_rows(n4, k) == CORE_GROUP_ROWS_WIDE ? HALVES_WIDE : HALVES) : 1.0);
+    };
     const double nnz = (double)g.nnz_l;
     const int max_core = std::min({MODEL_MAX_CORE, g.rows / 2 / MODEL_STEP * MODEL_STEP, (int)g.slice_deg.size() * 64 / MODEL_STEP * MODEL_STEP});
     // useful and padded entries of the block (slices [s0, s1) x tiles [t0, t1))
@@ -951,7 +970,7 @@ int predict_core_rows(GraphInfo &g, int dim, unsigned long long table_bytes, int
             const double h = hot_share(k);
             f = h + (1.0 - h) * far;
         }
-        if (pad <= 0.0 || useful * BETA_PS * (1 + sectors) * f < pad * entry) break;
+        if (pad <= 0.0 || useful * BETA_PS * (1 + sectors) * f < pad * entry_at(k)) break;
         best = k;
         taken += useful;
     }
@@ -974,7 +993,7 @@ MGGX_EXPORT int mggx_core_layout_device(const int *d_ptr, const int *d_col, int 
     rc = mggx::graph_info(d_ptr, nullptr, d_col, nullptr, rows, false, &g);
     if (rc) return rc;
     mggx::CorePlan *p = nullptr;
-    rc = mggx::core_plan_get(d_ptr, d_col, rows, lb, core_rows, g->serial, &p);
+    rc = mggx::core_plan_get(d_ptr, d_col, rows, lb, core_rows, mggx::CORE_GROUP_ROWS, g->serial, &p);
     if (rc) return rc;
     if (p->unsuitable) return fail(MGGX_EINVAL, "core layout: no core of whole 512-row units in %d rows, or a neighbor id outside [lb, lb + rows)", rows);
     const int64_t nblk = (int64_t)(p->core / 64) * p->ntiles + 1;

@@ -127,10 +127,18 @@ struct Plan {
 // Scratch layout of the dense core.  Staged table: slice s of the rank-i node's row at tab[s * tab_stride(core) + i]; the
 // stride carries a few rows more than the core size: with a power-of-two core the slices of a tile would otherwise all
 // start in the same memory channel.  Partial rows: one per workgroup of the LDS kernel and row of its row group, at
-// partial[(slot * CORE_GROUP_ROWS + rank % CORE_GROUP_ROWS) * n4 + piece]; the slots of row group g are
+// partial[(slot * group_rows + rank % group_rows) * n4 + piece]; the slots of row group g are
 // wg_base[g] .. wg_base[g + 1] - 1.
 __host__ __device__ inline size_t tab_stride(int core) { return (size_t)core + 16; }
-constexpr int CORE_GROUP_ROWS = 256;  // core rows per workgroup of the LDS kernel (4 wavefronts, one row per lane)
+constexpr int CORE_GROUP_ROWS = 256;  // core rows per workgroup of the LDS kernel (4 wavefronts, one row per lane) ...
+constexpr int CORE_GROUP_ROWS_WIDE = 512;  // ... and where rows are summed in two halves (CorePlan::group_rows)
+// Wide groups where rows are summed in halves and the staged table is well beyond an L2 (12 MB = three of them): every
+// row group re-reads that table once per call.  Held against graphs of width 64 that the setting was not read off: cores
+// of 16.8-21 MB gain 3-7 %, one of 10.5 MB lost 7 % with wide groups (profiles/rules_on_held_out_graphs.md).
+inline int core_group_rows(int n4, int core_rows)
+{
+    return n4 > 12 && (size_t)core_rows * (size_t)n4 * 16 > ((size_t)12 << 20) ? CORE_GROUP_ROWS_WIDE : CORE_GROUP_ROWS;
+}
 
 // Dense-core plan of a local-only CSR (layout: CoreLayout in mggx_internal.h), built on the GPU and kept there.
 struct CorePlan {
@@ -138,6 +146,7 @@ struct CorePlan {
     const int *d_ptr_l = nullptr;
     const int *d_col_l = nullptr;
     int rows = 0, lb = 0, asked = 0;
+    int group_rows = CORE_GROUP_ROWS;  // core rows per workgroup of the LDS kernel: 256 or 512
     // contents
     int core = 0, ntiles = 0;
     int64_t core_nnz = 0, rem_nnz = 0;
@@ -259,7 +268,7 @@ int exclusive_scan_i32_device(const int *d_in, int *d_out, int n, void *d_tmp);
 int static_scratch_ptr(unsigned char **out);
 void plan_free(Plan *p);
 int forget_pointer(const void *d_ptr);
-int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, int graph_serial, CorePlan **out);
+int core_plan_get(const int *d_ptr_l, const int *d_col_l, int rows, int lb, int core, int group_rows, int graph_serial, CorePlan **out);
 // Cost model of the dense core (degree histogram x row width): the core size that is predicted to pay for this CSR, a
 // multiple of 4096, or -1 for none.  table_bytes = rows x row pitch of the feature table.  Fetches the record's degree
 // profile on first use (one sort of the degrees on the device, 4 KiB to the host; synchronises).
