@@ -815,15 +815,15 @@ int core_partial_rows(CorePlan *p, int dim, const float4 **partial_out, const in
 // factor of 3.2 beyond 256 MB -- was fitted on those three alone) and nine graphs from other RMAT settings (a from 0.45 to
 // 0.65), sizes (0.3 - 2 M nodes), mean degrees (70 - 620) and widths (16 - 64), on which the first version and two
 // intermediate ones were up to 29 % off; graphs and sweeps: dse.py --mode heldout.  The 4 MB are the size of an L2.
+// HALVES_WIDE 0.62: rows in halves in row groups of 512 rows (core_group_rows) re-read the staged table half as often;
+// 0.55 put the core of a 700 K-node graph of width 64 at 86,016 rows, 4 % slower than 81,920; with 0.62 the four graphs
+// of that width are within 1.3 % of their sweeps' best.
 // The model stops at 98,304 rows.
 namespace mggx {
 namespace {
 
 constexpr int PROFILE_SLICES = 2048;  // 131072 ranks
-#ifndef MGGX_HALVES_WIDE
-#define MGGX_HALVES_WIDE 0.62
-#endif
-constexpr double ALPHA_PS = 1.40, BETA_PS = 9.0, HALVES = 0.7, HALVES_WIDE = MGGX_HALVES_WIDE, F_CACHE = 3.0, F_MEMORY = 4.0;
+constexpr double ALPHA_PS = 1.40, BETA_PS = 9.0, HALVES = 0.7, HALVES_WIDE = 0.62, F_CACHE = 3.0, F_MEMORY = 4.0;
 constexpr unsigned long long L2_BYTES = 4ull << 20, LAST_LEVEL_CACHE_BYTES = 256ull << 20;
 constexpr int MODEL_STEP = 4096, MODEL_MAX_CORE = 98304;
 

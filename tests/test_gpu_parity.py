@@ -894,6 +894,36 @@ def test_dense_update_bf16(gpu, n, d1, d2, x_bf16, out_bf16):
     assert_close_to_oracle(got, want_f, mag_f, BF16_TOL, "bf16 MFMA vs unrounded inputs")
 
 
+@pytest.mark.parametrize("n,d1,d2,ld_x,ld_out,relu", [(4096, 128, 128, 0, 0, False), (5003, 128, 128, 0, 0, True), (70001, 128, 64, 132, 72, False),
+                                                     (4099, 64, 128, 0, 136, True), (9000, 64, 64, 68, 0, False)])
+def test_dense_update_bf16_in_whole_lines(gpu, n, d1, d2, ld_x, ld_out, relu):
+    """fp32 rows of 64 or 128 to bf16 rows of 64 or 128, 4096 rows and more: the kernel that reads and writes whole rows through
+    LDS, takes its tiles in launch order and W from the image a small kernel prepares.  Ragged row counts (the last
+    workgroup and the last tile are partial), padded pitches, row scale and ReLU; two calls in a row with different W (the
+    image is rewritten per call); rows past n and the pitch padding stay untouched."""
+    import torch
+    x = gpu.fill_normal((n, d1), seed=60)
+    rs = (np.abs(gpu.fill_normal((n,), seed=61)) + 0.5).astype(np.float32)
+    px, po = ld_x or d1, ld_out or d2
+    xd = torch.zeros((n, px), device="cuda")
+    xd[:, :d1] = to_dev(x)
+    xr = xd[:, :d1].to(torch.bfloat16).to(torch.float32).cpu().numpy()
+    for seed in (62, 63):
+        w = gpu.glorot(d1, d2, seed=seed)
+        wb = to_dev(w).to(torch.bfloat16)
+        wf = wb.to(torch.float32).cpu().numpy()
+        out = torch.full((n + 3, po), 3.0, device="cuda", dtype=torch.bfloat16)
+        gpu.dense_forward_bf16(out, xd, wb, n, d1, d2, ld_x=px, ld_out=po, row_scale=to_dev(rs), relu=relu)
+        gpu.sync()
+        want = orc.dense(xr, wf, f64=True) * rs[:, None].astype(np.float64)
+        mag = (np.abs(xr).astype(np.float64) @ np.abs(wf).astype(np.float64)) * rs[:, None]
+        if relu:
+            want = np.maximum(want, 0.0)
+        got = out.to(torch.float32).cpu().numpy()
+        assert_close_to_oracle(got[:n, :d2], want, mag + np.abs(want) * 400, FP32_TOL, "whole-line bf16 update, W seed %d" % seed)
+        assert np.all(got[n:] == 3.0) and np.all(got[:, d2:] == 3.0)
+
+
 # --------------------------------------------------------------------------- softmax inside the aggregation
 def _softmax_want(sh, xl, x, dim, s):
     """softmax_forward(aggregate(...)) as the reference runs them back to back (src/mgg_np_div_mem.cu:221-225), in double."""
