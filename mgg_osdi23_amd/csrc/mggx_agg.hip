@@ -349,6 +349,8 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
     constexpr int S = 64 / LPR;
     constexpr int CH = LPR > 16 ? LPR : 16;  // neighbor ids fetched per slot per chunk
     constexpr int IPL = CH / LPR;            // ids fetched per lane
+    constexpr int CHP = CH + 4;              // words between the staged ids of neighbouring slots: 16 slots' 16-byte reads of
+                                             // the same position then fall into 16 different bank groups
     constexpr int BATCH = MGGX_BATCH;        // gathers issued back to back
     static_assert(CH % BATCH == 0, "the gathers of a chunk of ids are issued in whole batches");
     // With 16 slots a wavefront reads its ids 1 KiB at a time and its descriptors 256 B at a time -- whole cache lines
@@ -358,7 +360,7 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
     // rounds whose descriptors and first ids a wavefront fetches at once (1.3 - 5 KiB of LDS per wavefront; measured on
     // the benchmark graphs: 4 rounds are as good as 8, 1 round is 5 - 10 % slower where the feature table is cache resident)
     constexpr int STAGE = LPR >= 4 ? 4 : LPR == 2 ? 2 : 1;
-    extern __shared__ float lds[];
+    extern __shared__ __align__(16) float lds[];
     if (gate_closed(a.gate)) return;
     const int num_parts = a.num_parts_dev ? *a.num_parts_dev : a.num_parts;
 
@@ -453,15 +455,17 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
 #pragma unroll
         for (int t = 0; t < IPL; ++t) ids[t] = (kk + t < len) ? raw[t] - idbase : pad_id;
     };
-    // One window of gathers of a chunk of CH neighbors: get_rid(k) is the k-th neighbor's row in the slot's table.
-    auto gather_chunk = [&](int len, int k0, auto get_rid) {
+    // One window of gathers of a chunk of CH neighbors: get_rid4(q) gives neighbors 4 q .. 4 q + 3's rows in the slot's table.
+    static_assert(BATCH % 4 == 0, "ids are read four at a time");
+    auto gather_chunk = [&](int len, int k0, auto get_rid4) {
         static_for<0, CH / BATCH>([&](auto bb) {
             constexpr int b = decltype(bb)::value;
             if (__any(len > k0 + b * BATCH)) {
                 int rid[BATCH];
-                static_for<0, BATCH>([&](auto tt) {
-                    constexpr int t = decltype(tt)::value;
-                    rid[t] = get_rid(std::integral_constant<int, b * BATCH + t>{});
+                static_for<0, BATCH / 4>([&](auto qq) {  // four ids per 16-byte read
+                    constexpr int q4 = decltype(qq)::value;
+                    const int4 r4 = get_rid4(std::integral_constant<int, b * BATCH / 4 + q4>{});
+                    rid[4 * q4] = r4.x; rid[4 * q4 + 1] = r4.y; rid[4 * q4 + 2] = r4.z; rid[4 * q4 + 3] = r4.w;
                 });
                 // lanes past the row width neither load nor sum (their sums stay zero and are never stored): a quad
                 // of idle lanes costs the address unit nothing, and no register of the batch needs clearing
@@ -491,8 +495,9 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
     // STAGE rounds at a time -- all descriptor loads in flight together, then all id loads -- into its own piece of
     // LDS, and the rounds read them from there (every lane of a slot reads the same words).
     const int nst = a.stage_rounds < STAGE ? a.stage_rounds : STAGE;
-    int4 *st_desc = reinterpret_cast<int4 *>(lds + a.stage_off) + (size_t)wave * (nst * S);
-    int *st_ids = reinterpret_cast<int *>(lds + a.stage_off) + (size_t)wpb * (nst * S * 4) + (size_t)wave * (nst * S * CH);
+    float *const stage = static_cast<float *>(__builtin_assume_aligned(lds + a.stage_off, 16));  // stage_off is a multiple of 4
+    int4 *st_desc = reinterpret_cast<int4 *>(stage) + (size_t)wave * (nst * S);
+    int *st_ids = reinterpret_cast<int *>(stage) + (size_t)wpb * (nst * S * 4) + (size_t)wave * (nst * S * CHP);
 
     for (int j0 = 0; j0 < a.dist; j0 += nst) {
         if (q_wave + (long long)j0 * S >= num_parts) break;
@@ -511,7 +516,7 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
                 int ids[IPL];
                 finish_ids(dd[u], 0, idv[u], ids);
                 if (u < nst) {
-                    int *dst = st_ids + (u * S + slot) * CH + l * IPL;
+                    int *dst = st_ids + (u * S + slot) * CHP + l * IPL;
 #pragma unroll
                     for (int t = 0; t < IPL; ++t) dst[t] = ids[t];
                 }
@@ -551,7 +556,7 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
 
         // neighbors [0, CH) of the partition were staged; a longer partition (ps > CH) fetches each further chunk of ids
         // into the same words when it gets there
-        int *pid = st_ids + (u * S + slot) * CH;
+        int *pid = st_ids + (u * S + slot) * CHP;
         for (int k0 = 0; k0 < a.ps; k0 += CH) {
             if (!__any(len > k0)) break;
             if (k0 > 0) {
@@ -566,7 +571,7 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
                 __builtin_amdgcn_wave_barrier();
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             }
-            gather_chunk(len, k0, [&](auto kc) { return pid[decltype(kc)::value]; });
+            gather_chunk(len, k0, [&](auto q4) { return *reinterpret_cast<const int4 *>(static_cast<const int *>(__builtin_assume_aligned(pid, 16)) + 4 * decltype(q4)::value); });
         }
 
         // ---- combine the slots of this round ----
@@ -1089,7 +1094,7 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         // rounds are staged at a time when many wavefronts per workgroup would take more than 40 KiB
         const int stage_max = lpr >= 4 ? 4 : lpr == 2 ? 2 : 1;
         const int ch = lpr > 16 ? lpr : 16;
-        const size_t round_bytes = (size_t)slots * ((size_t)ch * 4 + 16);
+        const size_t round_bytes = (size_t)slots * ((size_t)(ch + 4) * 4 + 16);  // per slot: the staged ids (CHP words) and the descriptor
         int stage = stage_max < dist ? stage_max : dist;
         while (stage > 1 && (size_t)wpb * stage * round_bytes > (40u << 10)) stage /= 2;
         const size_t carry_lds = ((size_t)wpb * 2 * sizeof(int2) + (size_t)wpb * 2 * cpad * sizeof(float) + 15) & ~(size_t)15;
