@@ -416,6 +416,163 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_resident(const MlpArgs 
     }
 }
 
+// The same two-layer update, 64 -> 64 -> d3 (33 ... 64), on the bf16 matrix cores with fp32 results: every fp32 operand is
+// split exactly into three bf16 parts, x = x1 + x2 + x3 (x1 = bf16(x), x2 = bf16(x - x1), x3 = bf16(x - x1 - x2): 24
+// mantissa bits, the subtractions are exact), and a product x w becomes the six bf16 products that matter,
+// x1 w1 + (x1 w2 + x2 w1) + (x1 w3 + x2 w2 + x3 w1) -- each exact in the fp32 accumulator, what is dropped is below
+// 2^-24 of |x w|.  Six v_mfma_f32_16x16x32_bf16 do the work of eight v_mfma_f32_16x16x4_f32 at a sixteenth of the
+// cycles each, so the kernel that the fp32 matrix cores held at 68 % busy becomes bound by memory.
+// Layout as in k_mlp2_resident (transposed products; lane (i, kb) = (L % 16, L / 16)): the first product leaves the lane
+// with T[row i][16 nb + 4 kb + r], r = 0..3; the second wants eight K values per lane and step, and takes for step s the
+// columns {16 (2 s) + 4 kb + r} and {16 (2 s + 1) + 4 kb + r} -- Wb is staged with its K order permuted to match
+// (split_k_slot), so the intermediate never leaves the registers.
+// LDS: the three parts of Wa^T and of Wb^T, [part][column][72] bf16 (rows of 144 bytes: 16-byte reads, staggered banks).
+constexpr int SPLIT_KP = 64 + 8;
+
+// The three bf16 parts of two floats, packed in pairs (low half = first value).
+__device__ __forceinline__ void split_pair(float a, float b, unsigned &hi, unsigned &mid, unsigned &lo)
+{
+    const auto pack = [](float x, float y) {
+        const v2bf q = __builtin_convertvector((v2f){x, y}, v2bf);
+        unsigned u;
+        __builtin_memcpy(&u, &q, 4);
+        return u;
+    };
+    hi = pack(a, b);
+    float ra = a - __uint_as_float(hi << 16), rb = b - __uint_as_float(hi & 0xFFFF0000u);
+    mid = pack(ra, rb);
+    ra -= __uint_as_float(mid << 16);
+    rb -= __uint_as_float(mid & 0xFFFF0000u);
+    lo = pack(ra, rb);
+}
+__device__ __forceinline__ void split8(const float (&x)[8], v8bf &hi, v8bf &mid, v8bf &lo)
+{
+    unsigned h[4], m[4], l[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) split_pair(x[2 * t], x[2 * t + 1], h[t], m[t], l[t]);
+    __builtin_memcpy(&hi, h, 16);
+    __builtin_memcpy(&mid, m, 16);
+    __builtin_memcpy(&lo, l, 16);
+}
+// position in a staged row of Wb^T of the K index k (see above): step k / 32, lane group (k / 4) % 4, slot 4 ((k / 16) % 2) + k % 4
+__device__ __forceinline__ int split_k_slot(int k) { return 32 * (k >> 5) + 8 * ((k >> 2) & 3) + 4 * ((k >> 4) & 1) + (k & 3); }
+
+template <int NB2>
+__global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_split(const MlpArgs a)
+{
+    constexpr int NB1 = 4, KP = SPLIT_KP, WAVES = RES_THREADS / 64;
+    constexpr int PART_A = NB1 * 16 * KP, PART_B = NB2 * 16 * KP;  // bf16 elements per part
+    extern __shared__ __align__(16) float lds_raw[];
+    unsigned short *wa = reinterpret_cast<unsigned short *>(lds_raw), *wb = wa + 3 * PART_A;
+    const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
+    const int i = lane & 15, kb = lane >> 4;
+    // The weights, split and transposed, once per (persistent) workgroup.  Short-lived workgroups in launch order with the
+    // weights copied from a prepared image were measured too (as in k_dense_xw_bf16_lines): 0.32-0.34 ms against 0.31 --
+    // this kernel reads X in the operand layout and stores 64-byte pieces, and without whole-line traffic the launch order
+    // buys nothing.
+    for (int idx = (int)threadIdx.x; idx < 64 * 64; idx += RES_THREADS) {
+        const int k = idx >> 6, c = idx & 63;
+        unsigned h, m, l;
+        split_pair(a.wa[(long long)k * 64 + c], 0.f, h, m, l);
+        wa[c * KP + k] = (unsigned short)h;
+        wa[PART_A + c * KP + k] = (unsigned short)m;
+        wa[2 * PART_A + c * KP + k] = (unsigned short)l;
+    }
+    for (int idx = (int)threadIdx.x; idx < 64 * NB2 * 16; idx += RES_THREADS) {
+        const int k = idx / (NB2 * 16), c = idx % (NB2 * 16);
+        unsigned h, m, l;
+        split_pair(c < a.d3 ? a.wb[(long long)k * a.d3 + c] : 0.f, 0.f, h, m, l);
+        const int at = c * KP + split_k_slot(k);
+        wb[at] = (unsigned short)h;
+        wb[PART_B + at] = (unsigned short)m;
+        wb[2 * PART_B + at] = (unsigned short)l;
+    }
+    __syncthreads();
+    const __bf16 *wab = reinterpret_cast<const __bf16 *>(wa), *wbb = reinterpret_cast<const __bf16 *>(wb);
+
+    const long long tiles = (a.n + 15) / 16;
+    const long long stride = (long long)gridDim.x * WAVES;
+    long long tile = (long long)blockIdx.x * WAVES + wave;
+    if (tile >= tiles) return;
+    typedef float v4f_x __attribute__((ext_vector_type(4), aligned(16)));
+    v4f_x xn[4];  // the lane's 8 floats of K step 0 and of K step 1
+    const auto issue = [&](long long t) {
+        const float *xrow = a.x + min(t * 16 + i, a.n - 1) * a.ld_x + 8 * kb;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            xn[2 * ks] = *reinterpret_cast<const v4f_x *>(xrow + 32 * ks);
+            xn[2 * ks + 1] = *reinterpret_cast<const v4f_x *>(xrow + 32 * ks + 4);
+        }
+    };
+    issue(tile);
+    float scale = a.rs ? a.rs[min(tile * 16 + i, a.n - 1)] : 1.0f;
+    const float floor_mid = a.relu_mid ? 0.f : -3.4e38f;  // ReLU between the layers as one max per value
+    // acc += the six products of a split operand pair, smallest first
+    const auto six = [](v4f acc, const v8bf (&w)[3], const v8bf (&x)[3]) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[2], x[0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[1], x[1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[0], x[2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[1], x[0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[0], x[1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[0], x[0], acc, 0, 0, 0);
+        return acc;
+    };
+    for (;;) {
+        v8bf xs[2][3];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const float x8[8] = {xn[2 * ks][0], xn[2 * ks][1], xn[2 * ks][2], xn[2 * ks][3], xn[2 * ks + 1][0], xn[2 * ks + 1][1], xn[2 * ks + 1][2], xn[2 * ks + 1][3]};
+            split8(x8, xs[ks][0], xs[ks][1], xs[ks][2]);
+        }
+        const long long ntile = tile + stride;
+        const bool more = ntile < tiles;
+        float scale_next = 1.0f;
+        if (more) {  // wavefront-uniform
+            issue(ntile);
+            if (a.rs) scale_next = a.rs[min(ntile * 16 + i, a.n - 1)];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        v4f acc1[NB1];
+#pragma unroll
+        for (int nb = 0; nb < NB1; ++nb) acc1[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int nb = 0; nb < NB1; ++nb) {
+                v8bf w3[3];
+#pragma unroll
+                for (int p = 0; p < 3; ++p) w3[p] = *reinterpret_cast<const v8bf *>(wab + p * PART_A + (16 * nb + i) * KP + 32 * ks + 8 * kb);
+                acc1[nb] = six(acc1[nb], w3, xs[ks]);
+            }
+        }
+        v4f acc2[NB2];
+#pragma unroll
+        for (int nb = 0; nb < NB2; ++nb) acc2[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+            float t8[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                t8[e] = fmaxf(acc1[2 * st + (e >> 2)][e & 3], floor_mid);
+            }
+            v8bf ts[3];
+            split8(t8, ts[0], ts[1], ts[2]);
+#pragma unroll
+            for (int nb = 0; nb < NB2; ++nb) {
+                v8bf w3[3];
+#pragma unroll
+                for (int p = 0; p < 3; ++p) w3[p] = *reinterpret_cast<const v8bf *>(wbb + p * PART_B + (16 * nb + i) * KP + 32 * st + 8 * kb);
+                acc2[nb] = six(acc2[nb], w3, ts);
+            }
+        }
+        const long long row = tile * 16 + i;
+        store_rows<NB2, false>(a.out, a.ld_out, a.d3, scale, a.relu_out, a.vec_out, acc2, row, row < a.n, 0, kb);
+        if (!more) break;
+        tile = ntile;
+        scale = scale_next;
+    }
+}
+
 // W staged in K chunks (any d1): fallback when W does not fit in LDS.
 template <int NB>
 __global__ void __launch_bounds__(256) k_dense_xw(const DenseArgs a)
@@ -982,6 +1139,21 @@ MGGX_EXPORT int mggx_mlp2_xw(float *d_out, const float *d_x, const float *d_wa, 
     a.stream_x = d1 % 64 == 0 && a.ld_x % 32 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 127u) == 0;
     if (a.ld_x < d1 || a.ld_out < d3) return fail(MGGX_EINVAL, "mlp2_xw: row stride smaller than width");
     const int nb1 = (h + 15) / 16, nb2 = (d3 + 15) / 16;
+    if (d1 == 64 && h == 64 && d3 > 32 && n >= 4096 && a.ld_x % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15u) == 0) {
+        // the shape of a GIN layer's MLP: the split-operand kernel on the bf16 matrix cores (fp32 results)
+        const size_t lds_split = (size_t)3 * (64 + nb2 * 16) * mggx::SPLIT_KP * sizeof(unsigned short);
+        hipStream_t stream = mggx::state().stream;
+        const dim3 grid(mggx::persistent_blocks(n));
+        if (nb2 == 3) {
+            mggx::allow_lds(mggx::k_mlp2_split<3>, lds_split);
+            mggx::k_mlp2_split<3><<<grid, dim3(mggx::RES_THREADS), lds_split, stream>>>(a);
+        } else {
+            mggx::allow_lds(mggx::k_mlp2_split<4>, lds_split);
+            mggx::k_mlp2_split<4><<<grid, dim3(mggx::RES_THREADS), lds_split, stream>>>(a);
+        }
+        MGGX_LAUNCH_CHECK("k_mlp2_split");
+        return MGGX_OK;
+    }
     const size_t lds = ((size_t)((d1 + 63) & ~63) * (nb1 * 16 + 4) + (size_t)nb1 * 16 * (nb2 * 16 + 4)) * sizeof(float);
     if (lds > mggx::LDS_RESIDENT_LIMIT) return fail(MGGX_ELIMIT, "mlp2_xw: weights of %zu bytes do not fit in LDS (d1 <= ~%d at h = %d)", lds,
                                                     (int)(mggx::LDS_RESIDENT_LIMIT / 4 / (nb1 * 16 + 4)) - 64, h);

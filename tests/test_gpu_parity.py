@@ -781,7 +781,9 @@ def test_dense_closed_forms_and_epilogue(gpu):
 
 
 @pytest.mark.parametrize("n,d1,h,d3,relu_mid", [(1000, 64, 64, 64, True), (777, 64, 64, 47, True), (130, 100, 33, 5, False),
-                                                 (17, 7, 16, 64, True), (4099, 200, 48, 17, True)])
+                                                 (17, 7, 16, 64, True), (4099, 200, 48, 17, True),
+                                                 # 4096 rows and more of 64 -> 64 -> 33..64: the split-operand kernel on the bf16 matrix cores
+                                                 (4096, 64, 64, 64, True), (5003, 64, 64, 47, True), (70001, 64, 64, 33, False), (4100, 64, 64, 64, False)])
 def test_fused_two_layer_update(gpu, n, d1, h, d3, relu_mid):
     """act(X.Wa).Wb in one pass against the oracle's two dense updates (and against two library calls)."""
     import torch
