@@ -469,7 +469,9 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_split(const MlpArgs a)
     // The weights, split and transposed, once per (persistent) workgroup.  Short-lived workgroups in launch order with the
     // weights copied from a prepared image were measured too (as in k_dense_xw_bf16_lines): 0.32-0.34 ms against 0.31 --
     // this kernel reads X in the operand layout and stores 64-byte pieces, and without whole-line traffic the launch order
-    // buys nothing.
+    // buys nothing.  Whole rows through LDS (16 wavefronts, one workgroup per CU) were measured as well: 0.304 against
+    // 0.308 ms at 64 columns out, 0.394 against 0.374 at 47 -- memory is not what holds this kernel; per 16-row tile it
+    // issues 96 matrix-core instructions, 48 16-byte LDS reads of weights and some 260 vector instructions of splitting.
     for (int idx = (int)threadIdx.x; idx < 64 * 64; idx += RES_THREADS) {
         const int k = idx >> 6, c = idx & 63;
         unsigned h, m, l;
