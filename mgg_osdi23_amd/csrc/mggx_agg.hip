@@ -129,6 +129,43 @@ __device__ __forceinline__ float rows_from_even(float v) { return __int_as_float
 __device__ __forceinline__ float rows_from_odd(float v) { return __int_as_float(rows_from_odd(__float_as_int(v))); }
 __device__ __forceinline__ float low_half(float v) { return __int_as_float(low_half(__float_as_int(v))); }
 
+// Moves inside a row of 16 lanes with DPP (no LDS crossbar): CTRL = 0x110 + n: lane i takes lane i - n of its row (row_shr:n),
+// 0x120 + n: lane (i - n) mod 16 (row_ror:n); BANKS: which groups of four lanes of every row take the value (the others,
+// and lanes whose source falls outside the row, keep `keep`).
+template <int CTRL, int BANKS>
+__device__ __forceinline__ int row_move(int keep, int v) { return __builtin_amdgcn_update_dpp(keep, v, CTRL, 0xF, BANKS, false); }
+// every lane gets the value of the same lane position in the LAST slot of its 16-lane row
+template <int LPR>
+__device__ __forceinline__ int last_slot_of_row(int v)
+{
+    if constexpr (LPR == 8) {
+        return row_move<0x128, 0x3>(v, v);  // lanes 0-7 <- lanes 8-15
+    } else {
+        static_assert(LPR == 4, "slots of 4 or 8 lanes");
+        int b = row_move<0x124, 0x1>(v, v);  // lanes 0-3 <- 12-15
+        b = row_move<0x128, 0x2>(b, v);      // lanes 4-7 <- 12-15
+        return row_move<0x12C, 0x4>(b, v);   // lanes 8-11 <- 12-15
+    }
+}
+// The value of the slot a lane's slot combines with at level J of the slot scan below (valid where the slot takes one):
+// the last slot of the lower half of its group of 2^(J+1) slots.
+template <int LPR, int J>
+__device__ __forceinline__ int scan_source(int v)
+{
+    constexpr int PER_ROW = 16 / LPR;  // slots in a row of 16 lanes: 4 or 2
+    if constexpr ((1 << J) < PER_ROW) {
+        if constexpr (LPR == 8) return row_move<0x118, 0xF>(v, v);       // slot 1 of the row <- slot 0
+        else if constexpr (J == 0) return row_move<0x114, 0xF>(v, v);    // slots 1, 3 <- slots 0, 2
+        else return row_move<0x118, 0x8>(row_move<0x114, 0x4>(v, v), v); // slots 2, 3 <- slot 1
+    } else if constexpr ((1 << J) == PER_ROW) {
+        return rows_from_even(last_slot_of_row<LPR>(v));                 // rows 1, 3 <- the last slot of rows 0, 2
+    } else {
+        return low_half(rows_from_odd(last_slot_of_row<LPR>(v)));        // rows 2, 3 <- the last slot of row 1
+    }
+}
+template <int LPR, int J>
+__device__ __forceinline__ float scan_source(float v) { return __int_as_float(scan_source<LPR, J>(__float_as_int(v))); }
+
 template <int MODE>
 struct ModeTraits {
     static constexpr int NV = MODE == MODE_BF16_VEC8 ? 8 : 4;
@@ -582,10 +619,12 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
             has_first |= c_first;
         }
         // segmented inclusive scan over slots, keyed by row (equal rows are adjacent)
-        if constexpr (LPR == 16 || LPR == 32) {
-            // Slots are whole rows of 16 lanes (or halves of the wavefront): the scan moves registers with the row- and
-            // half-swap instructions.  Two steps for four slots: slots 1 and 3 take slots 0 and 2; then slots 2 and 3
-            // take slot 1, which by then holds the sum of its run so far.
+        if constexpr (LPR >= 4 && LPR <= 32) {
+            // No lane of this scan goes through the LDS crossbar.  At level j the slots whose bit j is set take the last
+            // slot of the lower half of their group of 2^(j+1) slots (which by then holds the sum of its run so far): S - 1
+            // additions in log2 S levels.  Slots that are whole rows of 16 lanes or halves of the wavefront move with the
+            // row- and half-swap instructions; narrower slots move inside their row with DPP (row_shr, row_ror with bank
+            // masks) and from row to row with a broadcast of the row's last slot followed by the same swaps.
             const auto step = [&](auto from, bool lower) {
                 const int prow = from(row);
                 const bool take = lower && prow == row && row >= 0;
@@ -602,8 +641,13 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
             if constexpr (LPR == 16) {
                 step([](auto v) { return rows_from_even(v); }, (slot & 1) != 0);
                 step([](auto v) { return low_half(rows_from_odd(v)); }, slot >= 2);
-            } else {
+            } else if constexpr (LPR == 32) {
                 step([](auto v) { return low_half(v); }, slot == 1);
+            } else {
+                static_for<0, 4>([&](auto jj) {
+                    constexpr int J = decltype(jj)::value;
+                    if constexpr ((1 << J) < S) step([](auto v) { return scan_source<LPR, J>(v); }, ((slot >> J) & 1) != 0);
+                });
             }
         } else {
         static_for<0, 6>([&](auto oo) {
