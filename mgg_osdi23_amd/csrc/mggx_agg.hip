@@ -121,13 +121,15 @@ __device__ __forceinline__ float lane_read(float v, int src)
 
 // Rows of 16 lanes swapped between two registers without a trip through the LDS crossbar (gfx950):
 // rows_from_even(v) = {v.row0, v.row0, v.row2, v.row2}, rows_from_odd(v) = {v.row1, v.row1, v.row3, v.row3},
-// low_half(v) = {v.row0, v.row1, v.row0, v.row1}.
+// low_half(v) = {v.row0, v.row1, v.row0, v.row1}, high_half(v) = {v.row2, v.row3, v.row2, v.row3}.
 __device__ __forceinline__ int rows_from_even(int v) { return (int)__builtin_amdgcn_permlane16_swap((unsigned)v, (unsigned)v, false, false)[0]; }
 __device__ __forceinline__ int rows_from_odd(int v) { return (int)__builtin_amdgcn_permlane16_swap((unsigned)v, (unsigned)v, false, false)[1]; }
 __device__ __forceinline__ int low_half(int v) { return (int)__builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false)[0]; }
+__device__ __forceinline__ int high_half(int v) { return (int)__builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false)[1]; }
 __device__ __forceinline__ float rows_from_even(float v) { return __int_as_float(rows_from_even(__float_as_int(v))); }
 __device__ __forceinline__ float rows_from_odd(float v) { return __int_as_float(rows_from_odd(__float_as_int(v))); }
 __device__ __forceinline__ float low_half(float v) { return __int_as_float(low_half(__float_as_int(v))); }
+__device__ __forceinline__ float high_half(float v) { return __int_as_float(high_half(__float_as_int(v))); }
 
 // Moves inside a row of 16 lanes with DPP (no LDS crossbar): CTRL = 0x110 + n: lane i takes lane i - n of its row (row_shr:n),
 // 0x120 + n: lane (i - n) mod 16 (row_ror:n); BANKS: which groups of four lanes of every row take the value (the others,
@@ -165,6 +167,16 @@ __device__ __forceinline__ int scan_source(int v)
 }
 template <int LPR, int J>
 __device__ __forceinline__ float scan_source(float v) { return __int_as_float(scan_source<LPR, J>(__float_as_int(v))); }
+// every lane gets the value of the same lane position in the last slot of the wavefront (slots of 4 to 32 lanes)
+template <int LPR>
+__device__ __forceinline__ int last_slot(int v)
+{
+    if constexpr (LPR == 32) return high_half(v);
+    else if constexpr (LPR == 16) return high_half(rows_from_odd(v));
+    else return high_half(rows_from_odd(last_slot_of_row<LPR>(v)));
+}
+template <int LPR>
+__device__ __forceinline__ float last_slot(float v) { return __int_as_float(last_slot<LPR>(__float_as_int(v))); }
 
 template <int MODE>
 struct ModeTraits {
@@ -577,10 +589,16 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
         float cv[NV];
         int c_first = 0;
         if (c_open) {
-            const int src = (lane + 64 - LPR) & 63;
+            if constexpr (LPR >= 4 && LPR <= 32) {
 #pragma unroll
-            for (int i = 0; i < NV; ++i) cv[i] = lane_read(acc[i], src);
-            c_first = lane_read(has_first, src);
+                for (int i = 0; i < NV; ++i) cv[i] = last_slot<LPR>(acc[i]);
+                c_first = last_slot<LPR>(has_first);
+            } else {
+                const int src = (lane + 64 - LPR) & 63;
+#pragma unroll
+                for (int i = 0; i < NV; ++i) cv[i] = lane_read(acc[i], src);
+                c_first = lane_read(has_first, src);
+            }
         }
 #pragma unroll
         for (int i = 0; i < NV; ++i) acc[i] = 0.0f;
@@ -669,15 +687,10 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
             }
         });
         }
-        // the last slot of each run now holds the run's sum
-        int nrow = -2;
-        if constexpr (S > 1) {
-            const int src = lane + LPR < 64 ? lane + LPR : lane;
-            nrow = lane_read(row, src);
-            if (slot == S - 1) nrow = -2;
-        }
-        const bool run_last = pv && nrow != row;
+        // The last slot of each run now holds the run's sum.  A run ends where its row ends (the descriptor of a row's last
+        // partition says so: the next descriptor, if any, belongs to another row) and at the last slot of the round.
         const bool row_done = ((unsigned)d.z & DESC_LAST) != 0;
+        const bool run_last = pv && (row_done || slot == S - 1);
         const bool last_round = (j == a.dist - 1) || (q0 + S >= num_parts);
         bool keep_open = false;
         if (run_last) {
