@@ -321,6 +321,120 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_dense_xw_resident(const Dens
     }
 }
 
+// Narrow updates (d2 <= 16) of densely packed rows that are not whole cache lines (602 floats = 2,408 bytes): read row by
+// row, every 64-float piece of a row straddles three lines and the lines are fetched more than once.  Here a tile of 16
+// rows is read as what it is in memory, one contiguous run of 16 d1 floats starting on a 64-byte boundary: the 512
+// threads of the workgroup load it 8 KB per instruction with the streaming hint and lay it down flat in LDS.  K is cut
+// into 8 slices, one per wavefront, so a wavefront keeps its slice of W in SW registers for the whole launch (lane
+// (column i, kq) holds W[KW w + 4 s + kq][i], s < SW) and reads its slice of the tile with 4-byte LDS reads in which
+// the four kq of a row are neighbors (two lanes per bank for every d1 that is not a multiple of 8); the 8 partial
+// tiles (16 x 16) meet in LDS and wavefront 0 stores the tile.  The loads of the next tile are in flight in registers
+// while this one is multiplied, so one LDS buffer is enough: 49 KB per workgroup at d1 = 602, three workgroups per CU
+// (80 registers).  A workgroup takes FLAT_TILES consecutive tiles and ends: short-lived workgroups in launch order keep
+// the chip inside a narrow moving window of the array (233,000 x 602 -> 16, ms: 2 tiles 0.120, 3 0.108, 4 0.106, 6 0.110,
+// 8 0.112, 16 0.116; as many long-lived workgroups as fit, equal contiguous shares: 0.109; W costs every workgroup
+// 38 KB of L2 reads).
+constexpr int FLAT_WAVES = 8;
+constexpr int FLAT_THREADS = FLAT_WAVES * 64;
+constexpr int FLAT_TILES = 4;  // consecutive tiles per workgroup
+// LDS floats of the tile: the 16 rows and what the last wavefront's K slice reads past them (masked), and never less than
+// the whole rounds of 16-byte pieces the workgroup lays down
+inline __host__ __device__ int flat_tile_floats(int d1, int sw)
+{
+    const int need = (16 * d1 + FLAT_WAVES * 4 * sw + 3) & ~3, laid = 4 * FLAT_WAVES * 64 * (sw / 4);
+    return need > laid ? need : laid;
+}
+
+template <int SW>
+__global__ void __launch_bounds__(FLAT_THREADS, SW <= 20 ? 6 : 4) k_dense_xw_flat(const DenseArgs a)
+{
+    constexpr int NL = SW / 4;   // 16-byte loads per thread and tile: 16 d1 floats <= 512 SW floats = NL x 512 x 4
+    constexpr int KW = 4 * SW;   // K values per wavefront
+    static_assert(SW % 4 == 0, "whole rounds of loads");
+    extern __shared__ __align__(16) float lds_flat[];
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int i = lane & 15, kq = lane >> 4;
+    const int d1 = a.d1;
+    float *xt = lds_flat;
+    float *red = lds_flat + flat_tile_floats(d1, SW);
+    const float *x = static_cast<const float *>(a.x);
+    const float *w = static_cast<const float *>(a.w);
+    const long long tiles = (a.n + 15) / 16;
+    const long long tile0 = (long long)blockIdx.x * a.tiles_per_wave;
+    const long long tile_end = min(tiles, tile0 + a.tiles_per_wave);
+    if (tile0 >= tiles) return;
+    // First row of a tile.  The last tile of an array whose rows are no multiple of 16 is the last 16 rows: it overlaps the
+    // tile before it (those rows are computed and stored twice, the same values) and may start off a 16-byte boundary.
+    const auto first_row = [&](long long tile) { return min(tile * 16, a.n - 16); };
+
+    typedef float v4f_any __attribute__((ext_vector_type(4), aligned(4)));
+    v4f xr[NL];
+    const auto issue = [&](long long tile) {
+        const char *src = reinterpret_cast<const char *>(x + first_row(tile) * d1);
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {  // uniform base + unsigned 32-bit lane offset: one register per load for the address
+            const unsigned f = 4u * (unsigned)(j * FLAT_THREADS + tid);
+            xr[j] = __builtin_nontemporal_load(reinterpret_cast<const v4f_any *>(src + 4u * min(f, (unsigned)(16 * d1 - 4))));
+        }
+    };
+    const auto lay_down = [&]() {
+#pragma unroll
+        for (int j = 0; j < NL; ++j)
+            *reinterpret_cast<v4f *>(xt + 4 * (j * FLAT_THREADS + tid)) = xr[j];  // past the tile: copies nobody reads
+    };
+
+    // The first tile and this wavefront's slice of W, all loads in flight together; every one of them has arrived before
+    // the loop below starts (a wait for W inside the loop would also wait for the next tile's loads, issued just before).
+    issue(tile0);
+    float wreg[SW];
+    const int kbase = KW * wave + kq;
+#pragma unroll
+    for (int s = 0; s < SW; ++s) wreg[s] = w[min(kbase + 4 * s, d1 - 1) * a.d2 + min(i, a.d2 - 1)];
+#pragma unroll
+    for (int s = 0; s < SW; ++s) {
+        // (the empty statement keeps the compiler from moving each load under the condition below, a branch and a wait per
+        // load)
+        asm volatile("" : "+v"(wreg[s]));
+        wreg[s] = (kbase + 4 * s < d1 && i < a.d2) ? wreg[s] : 0.f;
+    }
+    lay_down();
+    __syncthreads();
+
+    const float *xrow = xt + i * d1 + kbase;
+    // MORE: another tile follows; its loads are issued first.  (Two instantiations instead of a branch, so that every wait
+    // inside counts exactly the loads that were issued before it.)
+    const auto one_tile = [&](long long tile, auto more_c) {
+        constexpr bool MORE = decltype(more_c)::value;
+        const long long row = first_row(tile) + i;
+        float scale = 1.0f;  // asked for before the next tile: waiting for it later does not wait for the tile
+        if (wave == 0 && a.rs) scale = a.rs[row];
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (MORE) issue(tile + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        v4f acc = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < SW; ++s) {
+            const float xv = xrow[4 * s];
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wreg[s], kbase + 4 * s < d1 ? xv : 0.f, acc, 0, 0, 0);
+            if (s % 4 == 3) __builtin_amdgcn_sched_barrier(0);  // at most four LDS values waiting
+        }
+        *reinterpret_cast<v4f *>(red + (wave * 64 + lane) * 4) = acc;
+        __syncthreads();
+        if (wave == 0) {
+            v4f sum[1];
+            sum[0] = *reinterpret_cast<const v4f *>(red + lane * 4);
+#pragma unroll
+            for (int ww = 1; ww < FLAT_WAVES; ++ww) sum[0] += *reinterpret_cast<const v4f *>(red + (ww * 64 + lane) * 4);
+            store_rows<1, false>(a.out, a.ld_out, a.d2, scale, a.relu, a.vec_out, sum, row, true, 0, kq);
+        }
+        if constexpr (MORE) lay_down();
+        __syncthreads();
+    };
+    for (long long tile = tile0; tile + 1 < tile_end; ++tile) one_tile(tile, std::true_type{});
+    one_tile(tile_end - 1, std::false_type{});
+}
+
 // Two updates in one pass, Out = act(X . Wa) . Wb, both weight matrices resident in LDS (h <= 64, d3 <= 64).
 // The transposed first product leaves lane L with T[row L % 16][16 nb + 4 (L / 16) + r], r = 0..3: four consecutive
 // K values of one row of the intermediate, which is exactly the operand the second product wants.  The
@@ -1025,6 +1139,22 @@ struct LaunchBf16 {
     };
 };
 
+void launch_flat(int sw, dim3 grid, size_t lds, hipStream_t s, const DenseArgs &a)
+{
+    const auto go = [&](auto kernel) {
+        allow_lds(kernel, lds);
+        kernel<<<grid, dim3(FLAT_THREADS), lds, s>>>(a);
+    };
+    switch (sw) {
+        case 4: go(k_dense_xw_flat<4>); break;
+        case 8: go(k_dense_xw_flat<8>); break;
+        case 12: go(k_dense_xw_flat<12>); break;
+        case 16: go(k_dense_xw_flat<16>); break;
+        case 20: go(k_dense_xw_flat<20>); break;
+        default: go(k_dense_xw_flat<24>); break;
+    }
+}
+
 // persistent grid: enough workgroups to fill the device a few times over, never more than there are 64-row groups
 unsigned persistent_blocks(long long n)
 {
@@ -1065,6 +1195,17 @@ MGGX_EXPORT int mggx_dense_xw(float *d_out, const float *d_x, const float *d_w, 
     a.stream_x = d1 % 64 == 0 && a.ld_x % 32 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 127u) == 0;
     if (a.ld_x < d1 || a.ld_out < d2) return fail(MGGX_EINVAL, "dense_xw: row stride smaller than width");
     hipStream_t stream = mggx::state().stream;
+    if (d2 <= 16 && a.ld_x == d1 && d1 >= 128 && d1 <= 768 && d1 % 8 != 0 && n >= 4096 &&
+        (reinterpret_cast<uintptr_t>(d_x) & 15u) == 0) {
+        const int sw = ((d1 + 31) / 32 + 3) & ~3;  // K steps per wavefront, in whole rounds of loads
+        const size_t lds_flat = ((size_t)mggx::flat_tile_floats(d1, sw) + mggx::FLAT_WAVES * 256) * sizeof(float);
+        a.tiles_per_wave = mggx::FLAT_TILES;
+        const long long tiles = (n + 15) / 16;
+        const dim3 grid((unsigned)((tiles + a.tiles_per_wave - 1) / a.tiles_per_wave));
+        mggx::launch_flat(sw, grid, lds_flat, stream, a);
+        MGGX_LAUNCH_CHECK("k_dense_xw_flat");
+        return MGGX_OK;
+    }
     const int nb = mggx::pick_nb(d2);
     const int gy = ((d2 + 15) / 16 + nb - 1) / nb;
     const size_t lds = (size_t)((d1 + 63) & ~63) * (nb * 16 + 4) * sizeof(float);

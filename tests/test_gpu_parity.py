@@ -755,6 +755,36 @@ def test_dense_update(gpu, n, d1, d2):
     assert_close_to_oracle(out.cpu().numpy(), want, mag, FP32_TOL, "dense %dx%dx%d, strided X" % (n, d1, d2))
 
 
+@pytest.mark.parametrize("n,d1,d2,ld_out,relu,scale", [(4096, 602, 16, 16, False, False), (4099, 130, 7, 9, True, True),
+                                                         (5000, 767, 16, 16, False, True), (4111, 301, 1, 1, False, False),
+                                                         (70001, 250, 13, 16, True, False), (4111, 602, 16, 20, True, True)])
+def test_dense_update_in_flat_tiles(gpu, n, d1, d2, ld_out, relu, scale):
+    """4096 rows and more of densely packed rows that are no multiple of 32 bytes, at most 16 columns out: whole tiles of 16
+    rows go through the kernel that reads them as flat runs of memory (K split over the wavefronts of a workgroup), the
+    rows after the last whole tile through the general kernel."""
+    import torch
+    x = gpu.fill_normal((n, d1), seed=70)
+    w = gpu.glorot(d1, d2, seed=71)
+    s = gpu.fill_uniform((n,), 0.5, 1.5, seed=72) if scale else None
+    out = torch.full((n, ld_out), 9.0, device="cuda")
+    gpu.dense_forward(out, to_dev(x), to_dev(w), n, d1, d2, ld_out=ld_out, row_scale=to_dev(s) if scale else None, relu=relu)
+    gpu.sync()
+    want = orc.dense(x, w, f64=True)
+    mag = np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64)
+    if scale:
+        want, mag = want * s[:, None], mag * s[:, None]
+    if relu:
+        want = np.maximum(want, 0)
+    got = out.cpu().numpy()
+    assert_close_to_oracle(got[:, :d2], want, mag, FP32_TOL, "dense in flat tiles %dx%dx%d" % (n, d1, d2))
+    assert np.all(got[:, d2:] == 9.0)
+    # closed form: ones times ones is d1, exactly, in every row
+    out = torch.zeros(n, d2, device="cuda")
+    gpu.dense_forward(out, torch.ones(n, d1, device="cuda"), torch.ones(d1, d2, device="cuda"), n, d1, d2)
+    gpu.sync()
+    assert np.array_equal(out.cpu().numpy(), np.full((n, d2), float(d1), np.float32))
+
+
 def test_dense_closed_forms_and_epilogue(gpu):
     import torch
     n, d1, d2 = 200, 602, 16
