@@ -236,6 +236,17 @@ __device__ __forceinline__ void load_group(float (&x)[4][4], const float *xrow, 
     }
 }
 
+// The wait for loaded values happens where this is called.  The counter such a wait uses counts loads and stores alike, in
+// order: where the compiler places the wait for a prefetched operand after the stores of a finished tile (the end of a
+// loop body), the wavefront sits there until those stores are acknowledged; called before the stores, the wait only
+// covers the loads, which were issued long before, and the stores have the whole next tile to complete.
+__device__ __forceinline__ void arrived(float (&x)[4][4], float &s)
+{
+    asm volatile("" : "+v"(x[0][0]), "+v"(x[0][1]), "+v"(x[0][2]), "+v"(x[0][3]), "+v"(x[1][0]), "+v"(x[1][1]), "+v"(x[1][2]),
+                 "+v"(x[1][3]), "+v"(x[2][0]), "+v"(x[2][1]), "+v"(x[2][2]), "+v"(x[2][3]), "+v"(x[3][0]), "+v"(x[3][1]),
+                 "+v"(x[3][2]), "+v"(x[3][3]), "+v"(s));
+}
+
 // acc[nb] += Wt-block^T . X-group, transposed product (see store_rows)
 template <int NB, int RS>
 __device__ __forceinline__ void mfma_group(v4f (&acc)[NB], const float *wt_group, const float (&x)[4][4], int i, int kq, int ngg)
@@ -287,6 +298,7 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_dense_xw_resident(const Dens
         const long long row = min(tile * 16 + i, a.n - 1);
         load_group<KMODE>(xv, x + row * a.ld_x, 0, ngroups, a.d1, kq);
         if (a.rs) scale = a.rs[row];
+        arrived(xv, scale);
     }
     v4f acc[NB];
     int g = 0;
@@ -306,6 +318,8 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_dense_xw_resident(const Dens
             for (int nb = 0; nb < NB; ++nb) acc[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
         }
         mfma_group<NB, RS>(acc, wt + g * 64 * RS, xv, i, kq, ngg);
+        __builtin_amdgcn_sched_barrier(0);  // (not hoisted into the matrix-core work above)
+        arrived(xn, scale_next);    // before the stores
         if (last_g) {
             const long long row = tile * 16 + i;
             store_rows<NB, false>(a.out, a.ld_out, a.d2, scale, a.relu, a.vec_out, acc, row, row < a.n, c0, kq);
@@ -481,6 +495,7 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_resident(const MlpArgs 
         const long long row = min(tile * 16 + i, a.n - 1);
         load_group<KMODE>(xv, a.x + row * a.ld_x, 0, ngroups, a.d1, kq);
         if (a.rs) scale = a.rs[row];
+        arrived(xv, scale);
     }
     v4f acc1[NB1];
     int g = 0;
@@ -500,6 +515,8 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_resident(const MlpArgs 
             for (int nb = 0; nb < NB1; ++nb) acc1[nb] = (v4f){0.f, 0.f, 0.f, 0.f};
         }
         mfma_group<NB1, RS1>(acc1, wta + g * 64 * RS1, xv, i, kq, ngg);
+        __builtin_amdgcn_sched_barrier(0);  // (not hoisted into the matrix-core work above)
+        arrived(xn, scale_next);    // before the stores
         if (last_g) {
             v4f acc2[NB2];
 #pragma unroll
@@ -622,6 +639,7 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_split(const MlpArgs a)
     };
     issue(tile);
     float scale = a.rs ? a.rs[min(tile * 16 + i, a.n - 1)] : 1.0f;
+    asm volatile("" : "+v"(xn[0]), "+v"(xn[1]), "+v"(xn[2]), "+v"(xn[3]), "+v"(scale));  // waited for here, not at the head of the loop (see its end)
     const float floor_mid = a.relu_mid ? 0.f : -3.4e38f;  // ReLU between the layers as one max per value
     // acc += the six products of a split operand pair, smallest first
     const auto six = [](v4f acc, const v8bf (&w)[3], const v8bf (&x)[3]) {
@@ -681,6 +699,10 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_split(const MlpArgs a)
                 acc2[nb] = six(acc2[nb], w3, ts);
             }
         }
+        // The next tile's loads are waited for here, before this tile's stores are issued: the counter the wait uses
+        // counts loads and stores alike, in order, so a wait placed after the stores would sit until they are acknowledged.
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("" : "+v"(xn[0]), "+v"(xn[1]), "+v"(xn[2]), "+v"(xn[3]), "+v"(scale_next));
         const long long row = tile * 16 + i;
         store_rows<NB2, false>(a.out, a.ld_out, a.d3, scale, a.relu_out, a.vec_out, acc2, row, row < a.n, 0, kb);
         if (!more) break;
@@ -830,6 +852,7 @@ __global__ void __launch_bounds__(256) k_dense_xw_bf16(const DenseArgs a)
         const long long row = min(tile * 16 + i, a.n - 1);
         av = load_x8_bf16<X_F32>(a.x, row, a.ld_x, 8 * kb, a.d1, x_group_mode(0, 32, a.d1, 8));
         if (a.rs) scale = a.rs[row];
+        asm volatile("" : "+v"(av), "+v"(scale));  // as arrived()
     }
     v4f acc[NB];
     int k0 = 0;
@@ -838,7 +861,7 @@ __global__ void __launch_bounds__(256) k_dense_xw_bf16(const DenseArgs a)
         const long long ntile = last_k ? tile + stride : tile;
         const int nk = last_k ? 0 : k0 + 32;
         const long long nrow = min(ntile * 16 + i, a.n - 1);
-        const v8bf an = load_x8_bf16<X_F32>(a.x, nrow, a.ld_x, nk + 8 * kb, a.d1, x_group_mode(nk, 32, a.d1, 8));
+        v8bf an = load_x8_bf16<X_F32>(a.x, nrow, a.ld_x, nk + 8 * kb, a.d1, x_group_mode(nk, 32, a.d1, 8));
         scale_next = scale;
         if (last_k && a.rs) scale_next = a.rs[nrow];
         __builtin_amdgcn_sched_barrier(0);
@@ -853,6 +876,8 @@ __global__ void __launch_bounds__(256) k_dense_xw_bf16(const DenseArgs a)
             bv = *reinterpret_cast<const v8bf *>(wt + (size_t)(nb * 16 + i) * KP + k);  // one 16-byte LDS read (rows of Wt are 16-byte multiples)
             acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bv, av, acc[nb], 0, 0, 0);
         }
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("" : "+v"(an), "+v"(scale_next));  // as arrived(): before the stores
         if (last_k) {
             const long long row = tile * 16 + i;
             if constexpr (OUT_BF16 && NB % 2 == 0) {
