@@ -358,7 +358,9 @@ typedef struct mggx_mlp2_opts {
     int64_t ld_out;              /* 0 = d3 */
     const float *d_row_scale;    /* [n] multiplies each output row (NULL = 1) */
     uint32_t relu_mid;           /* max(0,.) between the two products */
-    uint32_t relu_out;           /* max(0,.) on the output */
+    uint32_t relu_out;           /* what follows the second product and the row scale: 0 nothing, 1 max(0,.),
+                                  * 2 the row softmax over the d3 columns (softmax_new_forward, include/gnn_layer.cuh:36-40,
+                                  * as the last call of a forward: the logits never make a round trip through memory) */
 } mggx_mlp2_opts;
 
 /* Two consecutive updates in one pass, Out[n x d3] = act(X[n x d1] . Wa[d1 x h]) . Wb[h x d3], fp32 on MFMA: what two

@@ -192,6 +192,40 @@ __device__ __forceinline__ void store_rows(void *out, long long ld_out, int d2, 
     }
 }
 
+// Row softmax of a finished 16-row tile in the transposed-product layout, before it is stored: lane (row i, kq) holds the
+// columns 16 nb + 4 kq + r of its row, so a row's values sit in the four lanes i, i + 16, i + 32, i + 48.  acc <- exp(scale
+// acc - max) / sum over the d2 columns that exist (the rest become 0 and are not stored).  All 64 lanes take part.
+template <int NB>
+__device__ __forceinline__ void tile_row_softmax(v4f (&acc)[NB], float scale, int d2, int kq)
+{
+    float m = -3.0e38f;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            acc[nb][r] *= scale;
+            if (16 * nb + 4 * kq + r < d2) m = fmaxf(m, acc[nb][r]);
+        }
+    m = fmaxf(m, __shfl_xor(m, 16));
+    m = fmaxf(m, __shfl_xor(m, 32));
+    float sum = 0.f;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float e = 16 * nb + 4 * kq + r < d2 ? __expf(acc[nb][r] - m) : 0.f;
+            acc[nb][r] = e;
+            sum += e;
+        }
+    sum += __shfl_xor(sum, 16);
+    sum += __shfl_xor(sum, 32);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[nb][r] *= inv;
+}
+
 // W kept whole in LDS; the 8 wavefronts of a workgroup walk over 16-row tiles of X.  K is cut into groups of 64.
 // FULL (d1 >= 64): every group is a whole 64 wide -- the last one is shifted back to [d1 - 64, d1) and the W rows
 // it shares with the group before are zero in LDS, so every X load is a plain in-row 16-byte load with no tail
@@ -458,7 +492,7 @@ struct MlpArgs {
     const float *x, *wa, *wb, *rs;
     long long n, ld_x, ld_out;
     int d1, h, d3;
-    int relu_mid, relu_out, vec_out, stream_x;
+    int relu_mid, relu_out, vec_out, stream_x;  // relu_out: 0 none, 1 ReLU, 2 row softmax
 };
 
 template <int NB1, int NB2, int KMODE>
@@ -534,7 +568,12 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_resident(const MlpArgs 
                 }
             }
             const long long row = tile * 16 + i;
-            store_rows<NB2, false>(a.out, a.ld_out, a.d3, scale, a.relu_out, a.vec_out, acc2, row, row < a.n, 0, kq);
+            if (a.relu_out == 2) {  // row softmax of the (scaled) result instead of ReLU
+                tile_row_softmax<NB2>(acc2, scale, a.d3, kq);
+                store_rows<NB2, false>(a.out, a.ld_out, a.d3, 1.0f, 0, a.vec_out, acc2, row, row < a.n, 0, kq);
+            } else {
+                store_rows<NB2, false>(a.out, a.ld_out, a.d3, scale, a.relu_out, a.vec_out, acc2, row, row < a.n, 0, kq);
+            }
         }
 #pragma unroll
         for (int gg = 0; gg < 4; ++gg)
@@ -704,7 +743,12 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_split(const MlpArgs a)
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("" : "+v"(xn[0]), "+v"(xn[1]), "+v"(xn[2]), "+v"(xn[3]), "+v"(scale_next));
         const long long row = tile * 16 + i;
-        store_rows<NB2, false>(a.out, a.ld_out, a.d3, scale, a.relu_out, a.vec_out, acc2, row, row < a.n, 0, kb);
+        if (a.relu_out == 2) {  // row softmax of the (scaled) result instead of ReLU
+            tile_row_softmax<NB2>(acc2, scale, a.d3, kb);
+            store_rows<NB2, false>(a.out, a.ld_out, a.d3, 1.0f, 0, a.vec_out, acc2, row, row < a.n, 0, kb);
+        } else {
+            store_rows<NB2, false>(a.out, a.ld_out, a.d3, scale, a.relu_out, a.vec_out, acc2, row, row < a.n, 0, kb);
+        }
         if (!more) break;
         tile = ntile;
         scale = scale_next;
@@ -1301,7 +1345,8 @@ MGGX_EXPORT int mggx_mlp2_xw(float *d_out, const float *d_x, const float *d_wa, 
     a.h = h;
     a.d3 = d3;
     a.relu_mid = o.relu_mid != 0;
-    a.relu_out = o.relu_out != 0;
+    if (o.relu_out > 2) return fail(MGGX_EINVAL, "mlp2_xw: relu_out=%u (0 none, 1 ReLU, 2 row softmax)", o.relu_out);
+    a.relu_out = (int)o.relu_out;
     a.vec_out = a.ld_out % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0;
     if (d3 % 32 == 0 && a.ld_out % 32 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 127u) == 0) a.vec_out |= 2;
     a.stream_x = d1 % 64 == 0 && a.ld_x % 32 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 127u) == 0;

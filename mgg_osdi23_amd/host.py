@@ -451,15 +451,17 @@ def dense_forward(out, x, w, n, d1, d2, ld_x=0, ld_out=0, row_scale=None, relu=F
     _check(lib().mggx_dense_xw(_dptr(out), _dptr(x), _dptr(w), C.c_int64(n), d1, d2, C.byref(o)))
 
 
-def mlp2_forward(out, x, wa, wb, n, d1, h, d3, ld_x=0, ld_out=0, row_scale=None, relu_mid=True, relu_out=False):
+def mlp2_forward(out, x, wa, wb, n, d1, h, d3, ld_x=0, ld_out=0, row_scale=None, relu_mid=True, relu_out=False,
+                 softmax_out=False):
     """Out = act(X . Wa) . Wb in one pass (h, d3 <= 64): two dense_hidden_forward calls without the round trip of the
-    intermediate through memory."""
+    intermediate through memory.  softmax_out: the row softmax of the result (softmax_new_forward) in the same pass."""
     o = _Mlp2Opts()
     o.ld_x = ld_x
     o.ld_out = ld_out
     o.d_row_scale = row_scale.data_ptr() if row_scale is not None else None
     o.relu_mid = int(relu_mid)
-    o.relu_out = int(relu_out)
+    assert not (relu_out and softmax_out)
+    o.relu_out = 2 if softmax_out else int(relu_out)
     _check(lib().mggx_mlp2_xw(_dptr(out), _dptr(x), _dptr(wa), _dptr(wb), C.c_int64(n), d1, h, d3, C.byref(o)))
 
 

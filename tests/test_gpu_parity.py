@@ -845,6 +845,37 @@ def test_fused_two_layer_update(gpu, n, d1, h, d3, relu_mid):
         gpu.mlp2_forward(out, to_dev(x), to_dev(wa), to_dev(wb), n, d1, 65, d3)
 
 
+@pytest.mark.parametrize("n,d1,h,d3", [(1000, 64, 64, 47), (5003, 64, 64, 47), (4100, 64, 64, 64), (130, 100, 33, 5), (70001, 64, 64, 33)])
+def test_fused_two_layer_update_ends_in_softmax(gpu, n, d1, h, d3):
+    """The last update of a forward with the row softmax in the same pass: against the oracle's softmax of its own two dense
+    updates, and against the library's separate calls (fused update, then mggx_softmax_rows)."""
+    import torch
+    x = gpu.fill_normal((n, d1), seed=80)
+    wa = gpu.glorot(d1, h, seed=81)
+    wb = gpu.glorot(h, d3, seed=82) * 4
+    s = gpu.fill_uniform((n,), 0.5, 1.5, seed=83)
+    ldo = d3 + 1
+    out = torch.full((n, ldo), 9.0, device="cuda")
+    gpu.mlp2_forward(out, to_dev(x), to_dev(wa), to_dev(wb), n, d1, h, d3, ld_out=ldo, row_scale=to_dev(s), relu_mid=True, softmax_out=True)
+    gpu.sync()
+    t = np.maximum(orc.dense(x, wa, f64=True), 0)
+    logits = (t @ wb.astype(np.float64)) * s[:, None]
+    e = np.exp(logits - logits.max(1, keepdims=True))
+    want = e / e.sum(1, keepdims=True)
+    got = out.cpu().numpy()
+    assert np.allclose(got[:, :d3], want, rtol=2e-5, atol=1e-7), np.abs(got[:, :d3] - want).max()
+    assert np.allclose(got[:, :d3].sum(1), 1.0, atol=1e-5)
+    assert np.all(got[:, d3:] == 9.0)
+    lg = torch.empty(n, d3, device="cuda")
+    two = torch.empty(n, d3, device="cuda")
+    gpu.mlp2_forward(lg, to_dev(x), to_dev(wa), to_dev(wb), n, d1, h, d3, row_scale=to_dev(s), relu_mid=True)
+    gpu.softmax_forward(two, lg, n, d3)
+    gpu.sync()
+    assert np.allclose(got[:, :d3], two.cpu().numpy(), rtol=1e-5, atol=1e-7)
+    with pytest.raises(AssertionError):
+        gpu.mlp2_forward(out, to_dev(x), to_dev(wa), to_dev(wb), n, d1, h, d3, relu_out=True, softmax_out=True)
+
+
 @pytest.mark.parametrize("n,c", [(1000, 41), (333, 47), (64, 1), (10, 200), (5, 64)])
 def test_softmax_rows(gpu, n, c):
     import torch
