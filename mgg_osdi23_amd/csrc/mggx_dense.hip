@@ -226,6 +226,36 @@ __device__ __forceinline__ void tile_row_softmax(v4f (&acc)[NB], float scale, in
         for (int r = 0; r < 4; ++r) acc[nb][r] *= inv;
 }
 
+// A finished 16-row tile whose rows are packed (ld_out = d2) but no multiple of 16 bytes (47 floats): stored from the
+// operand layout it would leave as 4-byte pieces, four lanes to a row.  The tile itself is one contiguous run of 16 d2
+// floats that starts on a 16-byte boundary, so it goes through the wavefront's piece of LDS, laid out as in memory, and
+// leaves in 16-byte stores of whole consecutive lines.  `v` already carries scale and activation.
+template <int NB>
+__device__ __forceinline__ void store_tile_flat(float *out, float *piece, int d2, long long n, const v4f (&v)[NB], long long tile, int i,
+                                                int kq, int lane)
+{
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int c = 16 * nb + 4 * kq + r;
+            if (c < d2) piece[i * d2 + c] = v[nb][r];
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int span = (int)min(16LL, n - tile * 16) * d2;  // floats of the tile that exist
+    float *dst = out + tile * 16 * d2;
+    for (int f = 4 * lane; f < span; f += 256) {
+        if (f + 3 < span) {
+            __builtin_nontemporal_store(*reinterpret_cast<const v4f *>(piece + f), reinterpret_cast<v4f *>(dst + f));
+        } else {
+            for (int t = 0; f + t < span; ++t) dst[f + t] = piece[f + t];
+        }
+    }
+    __builtin_amdgcn_wave_barrier();  // the piece is free for the next tile once every lane has read its part
+}
+
 // W kept whole in LDS; the 8 wavefronts of a workgroup walk over 16-row tiles of X.  K is cut into groups of 64.
 // FULL (d1 >= 64): every group is a whole 64 wide -- the last one is shifted back to [d1 - 64, d1) and the W rows
 // it shares with the group before are zero in LDS, so every X load is a plain in-row 16-byte load with no tail
@@ -493,6 +523,7 @@ struct MlpArgs {
     long long n, ld_x, ld_out;
     int d1, h, d3;
     int relu_mid, relu_out, vec_out, stream_x;  // relu_out: 0 none, 1 ReLU, 2 row softmax
+    int flat_out;  // k_mlp2_split: packed rows that are no multiple of 16 bytes leave as whole tiles (store_tile_flat)
 };
 
 template <int NB1, int NB2, int KMODE>
@@ -743,7 +774,20 @@ __global__ void __launch_bounds__(RES_THREADS, 4) k_mlp2_split(const MlpArgs a)
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("" : "+v"(xn[0]), "+v"(xn[1]), "+v"(xn[2]), "+v"(xn[3]), "+v"(scale_next));
         const long long row = tile * 16 + i;
-        if (a.relu_out == 2) {  // row softmax of the (scaled) result instead of ReLU
+        if (a.flat_out) {
+            if (a.relu_out == 2) {
+                tile_row_softmax<NB2>(acc2, scale, a.d3, kb);
+            } else {
+#pragma unroll
+                for (int nb = 0; nb < NB2; ++nb)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        acc2[nb][r] *= scale;
+                        if (a.relu_out) acc2[nb][r] = fmaxf(acc2[nb][r], 0.f);
+                    }
+            }
+            store_tile_flat<NB2>(a.out, reinterpret_cast<float *>(wb + 3 * PART_B) + wave * (16 * NB2 * 16), a.d3, a.n, acc2, tile, i, kb, lane);
+        } else if (a.relu_out == 2) {  // row softmax of the (scaled) result instead of ReLU
             tile_row_softmax<NB2>(acc2, scale, a.d3, kb);
             store_rows<NB2, false>(a.out, a.ld_out, a.d3, 1.0f, 0, a.vec_out, acc2, row, row < a.n, 0, kb);
         } else {
@@ -1354,7 +1398,9 @@ MGGX_EXPORT int mggx_mlp2_xw(float *d_out, const float *d_x, const float *d_wa, 
     const int nb1 = (h + 15) / 16, nb2 = (d3 + 15) / 16;
     if (d1 == 64 && h == 64 && d3 > 32 && n >= 4096 && a.ld_x % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15u) == 0) {
         // the shape of a GIN layer's MLP: the split-operand kernel on the bf16 matrix cores (fp32 results)
-        const size_t lds_split = (size_t)3 * (64 + nb2 * 16) * mggx::SPLIT_KP * sizeof(unsigned short);
+        size_t lds_split = (size_t)3 * (64 + nb2 * 16) * mggx::SPLIT_KP * sizeof(unsigned short);
+        a.flat_out = a.ld_out == d3 && d3 % 4 != 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0;  // (64 packed columns: 0.271 -> 0.352 ms, 16 rows to a bank)
+        if (a.flat_out) lds_split += (size_t)(mggx::RES_THREADS / 64) * 16 * nb2 * 16 * sizeof(float);  // a tile per wavefront
         hipStream_t stream = mggx::state().stream;
         const dim3 grid(mggx::persistent_blocks(n));
         if (nb2 == 3) {

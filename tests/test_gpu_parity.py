@@ -872,6 +872,20 @@ def test_fused_two_layer_update_ends_in_softmax(gpu, n, d1, h, d3):
     gpu.softmax_forward(two, lg, n, d3)
     gpu.sync()
     assert np.allclose(got[:, :d3], two.cpu().numpy(), rtol=1e-5, atol=1e-7)
+    # packed rows (ld_out = d3; where d3 is no multiple of 4 and there are 4096 rows or more, tiles leave as contiguous runs)
+    packed = torch.full((n + 1, d3), 9.0, device="cuda")
+    gpu.mlp2_forward(packed, to_dev(x), to_dev(wa), to_dev(wb), n, d1, h, d3, row_scale=to_dev(s), relu_mid=True, softmax_out=True)
+    gpu.sync()
+    pk = packed.cpu().numpy()
+    assert np.allclose(pk[:n], want, rtol=2e-5, atol=1e-7), np.abs(pk[:n] - want).max()
+    assert np.all(pk[n] == 9.0)  # nothing written past the last row
+    lgw = np.maximum(logits, 0)
+    gpu.mlp2_forward(packed, to_dev(x), to_dev(wa), to_dev(wb), n, d1, h, d3, row_scale=to_dev(s), relu_mid=True, relu_out=True)
+    gpu.sync()
+    pk = packed.cpu().numpy()
+    mag = ((np.abs(x).astype(np.float64) @ np.abs(wa).astype(np.float64)) @ np.abs(wb).astype(np.float64)) * s[:, None]
+    assert_close_to_oracle(pk[:n], lgw, mag, 2 * FP32_TOL, "packed rows, ReLU out")
+    assert np.all(pk[n] == 9.0)
     with pytest.raises(AssertionError):
         gpu.mlp2_forward(out, to_dev(x), to_dev(wa), to_dev(wb), n, d1, h, d3, relu_out=True, softmax_out=True)
 
