@@ -136,44 +136,33 @@ __device__ __forceinline__ float high_half(float v) { return __int_as_float(high
 // and lanes whose source falls outside the row, keep `keep`).
 template <int CTRL, int BANKS>
 __device__ __forceinline__ int row_move(int keep, int v) { return __builtin_amdgcn_update_dpp(keep, v, CTRL, 0xF, BANKS, false); }
-// every lane gets the value of the same lane position in the LAST slot of its 16-lane row
-template <int LPR>
-__device__ __forceinline__ int last_slot_of_row(int v)
+// every lane gets the value of the same lane position in the LAST 4-lane slot of its 16-lane row
+__device__ __forceinline__ int last_quad_of_row(int v)
 {
-    if constexpr (LPR == 8) {
-        return row_move<0x128, 0x3>(v, v);  // lanes 0-7 <- lanes 8-15
-    } else {
-        static_assert(LPR == 4, "slots of 4 or 8 lanes");
-        int b = row_move<0x124, 0x1>(v, v);  // lanes 0-3 <- 12-15
-        b = row_move<0x128, 0x2>(b, v);      // lanes 4-7 <- 12-15
-        return row_move<0x12C, 0x4>(b, v);   // lanes 8-11 <- 12-15
-    }
+    int b = row_move<0x124, 0x1>(v, v);  // lanes 0-3 <- 12-15
+    b = row_move<0x128, 0x2>(b, v);      // lanes 4-7 <- 12-15
+    return row_move<0x12C, 0x4>(b, v);   // lanes 8-11 <- 12-15
 }
-// The value of the slot a lane's slot combines with at level J of the slot scan below (valid where the slot takes one):
-// the last slot of the lower half of its group of 2^(J+1) slots.
+// The value of the slot a lane's 4-lane slot combines with at level J of the slot scan below (valid where the slot takes
+// one): the last slot of the lower half of its group of 2^(J+1) slots.
 template <int LPR, int J>
 __device__ __forceinline__ int scan_source(int v)
 {
-    constexpr int PER_ROW = 16 / LPR;  // slots in a row of 16 lanes: 4 or 2
-    if constexpr ((1 << J) < PER_ROW) {
-        if constexpr (LPR == 8) return row_move<0x118, 0xF>(v, v);       // slot 1 of the row <- slot 0
-        else if constexpr (J == 0) return row_move<0x114, 0xF>(v, v);    // slots 1, 3 <- slots 0, 2
-        else return row_move<0x118, 0x8>(row_move<0x114, 0x4>(v, v), v); // slots 2, 3 <- slot 1
-    } else if constexpr ((1 << J) == PER_ROW) {
-        return rows_from_even(last_slot_of_row<LPR>(v));                 // rows 1, 3 <- the last slot of rows 0, 2
-    } else {
-        return low_half(rows_from_odd(last_slot_of_row<LPR>(v)));        // rows 2, 3 <- the last slot of row 1
-    }
+    static_assert(LPR == 4, "slots of 4 lanes");
+    if constexpr (J == 0) return row_move<0x114, 0xF>(v, v);                                 // slots 1, 3 <- slots 0, 2
+    else if constexpr (J == 1) return row_move<0x118, 0x8>(row_move<0x114, 0x4>(v, v), v);   // slots 2, 3 <- slot 1
+    else if constexpr (J == 2) return rows_from_even(last_quad_of_row(v));                   // rows 1, 3 <- the last slot of rows 0, 2
+    else return low_half(rows_from_odd(last_quad_of_row(v)));                                // rows 2, 3 <- the last slot of row 1
 }
 template <int LPR, int J>
 __device__ __forceinline__ float scan_source(float v) { return __int_as_float(scan_source<LPR, J>(__float_as_int(v))); }
-// every lane gets the value of the same lane position in the last slot of the wavefront (slots of 4 to 32 lanes)
+// every lane gets the value of the same lane position in the last slot of the wavefront (slots of 4, 16 or 32 lanes)
 template <int LPR>
 __device__ __forceinline__ int last_slot(int v)
 {
     if constexpr (LPR == 32) return high_half(v);
     else if constexpr (LPR == 16) return high_half(rows_from_odd(v));
-    else return high_half(rows_from_odd(last_slot_of_row<LPR>(v)));
+    else return high_half(rows_from_odd(last_quad_of_row(v)));
 }
 template <int LPR>
 __device__ __forceinline__ float last_slot(float v) { return __int_as_float(last_slot<LPR>(__float_as_int(v))); }
@@ -409,6 +398,11 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
     // rounds whose descriptors and first ids a wavefront fetches at once (1.3 - 5 KiB of LDS per wavefront; measured on
     // the benchmark graphs: 4 rounds are as good as 8, 1 round is 5 - 10 % slower where the feature table is cache resident)
     constexpr int STAGE = LPR >= 4 ? 4 : LPR == 2 ? 2 : 1;
+    // Slots of 4, 16 and 32 lanes combine and carry their sums with DPP row moves and the row- / half-swap instructions
+    // instead of ds_bpermute.  Slots of 8 lanes keep ds_bpermute: their DPP form (written and measured) is 2 % faster to
+    // 11 % slower beside the LDS kernel (233 K-node graph at width 24 / 32: 0.80 -> 0.78 / 0.91 -> 0.97 ms, 2.45 M-node graph
+    // at width 32: 1.59 -> 1.77 ms) and the same without it.
+    constexpr bool OFF_CROSSBAR = LPR == 4 || LPR == 16 || LPR == 32;
     extern __shared__ __align__(16) float lds[];
     if (gate_closed(a.gate)) return;
     const int num_parts = a.num_parts_dev ? *a.num_parts_dev : a.num_parts;
@@ -589,7 +583,7 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
         float cv[NV];
         int c_first = 0;
         if (c_open) {
-            if constexpr (LPR >= 4 && LPR <= 32) {
+            if constexpr (OFF_CROSSBAR) {
 #pragma unroll
                 for (int i = 0; i < NV; ++i) cv[i] = last_slot<LPR>(acc[i]);
                 c_first = last_slot<LPR>(has_first);
@@ -637,11 +631,11 @@ __global__ void __launch_bounds__(1024) MGGX_AGG_OCCUPANCY k_agg(const AggArgs a
             has_first |= c_first;
         }
         // segmented inclusive scan over slots, keyed by row (equal rows are adjacent)
-        if constexpr (LPR >= 4 && LPR <= 32) {
+        if constexpr (OFF_CROSSBAR) {
             // No lane of this scan goes through the LDS crossbar.  At level j the slots whose bit j is set take the last
             // slot of the lower half of their group of 2^(j+1) slots (which by then holds the sum of its run so far): S - 1
             // additions in log2 S levels.  Slots that are whole rows of 16 lanes or halves of the wavefront move with the
-            // row- and half-swap instructions; narrower slots move inside their row with DPP (row_shr, row_ror with bank
+            // row- and half-swap instructions; slots of 4 lanes move inside their row with DPP (row_shr, row_ror with bank
             // masks) and from row to row with a broadcast of the row's last slot followed by the same swaps.
             const auto step = [&](auto from, bool lower) {
                 const int prow = from(row);
@@ -1049,9 +1043,10 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     const int slots = 64 / lpr;
     // 0 = let the library choose.  Few slots per wavefront (wide rows): 8 wavefronts and 16 rounds, so a workgroup still
     // covers a few thousand neighbors; column-blocked plans: 4 wavefronts (they share the chip with the dense core's
-    // 4-wavefront workgroups); in row-major order beside a dense core: 8 wavefronts and 4 rounds (8 rounds are 2.4 % faster
-    // on the 2.45 M-node graph at width 64 and 9 % slower on a 700 K-node one of the same width); short rows (under 3
-    // partitions per row): 4 wavefronts.  Many slots (narrow rows): 4 wavefronts, 4 rounds; 8 rounds where a column-blocked
+    // 4-wavefront workgroups); in row-major order beside a dense core: 8 wavefronts and 4 rounds, 8 rounds where the core
+    // works in wide row groups (width 52 to 64, staged table beyond 12 MB: seven graphs of 0.7 to 3 M nodes at width 64 are
+    // 1.4 - 3.7 % faster with 8 than with 4, one of them by 0.1 %; at width 48, narrow groups, 8 rounds cost 1.1 %); short
+    // rows (under 3 partitions per row): 4 wavefronts.  Many slots (narrow rows): 4 wavefronts, 4 rounds; 8 rounds where a column-blocked
     // plan is left with short rows (under 8 partitions per row and block).
     // Provenance: wpb x dist sweeps on the three benchmark graphs and the bf16 share (each choice within 1 % of the best
     // cell there), re-checked on eighteen graphs of other generators, sizes, degrees and widths: within 5.2 % of the best
@@ -1061,7 +1056,7 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     const bool beside_core = cm != nullptr;
     if (wpb == 0) wpb = (beside_core && !blocked && slots <= 4) ? 8 : (blocked || slots > 4 || per_row < 3.0) ? 4 : 8;
     if (dist == 0) {
-        if (slots <= 4) dist = (beside_core && !blocked) ? 4 : 16;
+        if (slots <= 4) dist = (beside_core && !blocked) ? (cm->group_rows == CORE_GROUP_ROWS_WIDE ? 8 : 4) : 16;
         else if (blocked && per_row < 8.0) dist = 8;
         else dist = 4;
     }
