@@ -195,7 +195,7 @@ MEASURED_TRAFFIC = {
     "share_agg": (1_213_309_056, (4, 4)),
     "share_agg_compact": (1_028_547_520, (4, 4)),   # remote rows staged compactly (one row per distinct remote id)
     "gin_agg": (25_550_513_561, (16, 1)),
-    "gin_agg_core98304": (15_672_682_896, (8, 4)),   # the size the cost model picks (row groups of 512 rows)
+    "gin_agg_core98304": (15_702_715_472, (8, 8)),   # the size the cost model picks (row groups of 512 rows), the knobs the rules pick
     "big_agg": (60_511_998_361, (4, 16)),
 }
 
