@@ -85,6 +85,7 @@ struct AggArgs {
     const int *nnz_l_dev;     // when set: the local edge count is read from here (a caller that may not copy it to the host)
     int lb, dim, ps, dist, cpad;
     int parts_per_wg;
+    int ppw_shift;            // log2(parts_per_wg) where that is a power of two (every setting of the rules), else -1
     int stage_off;            // dynamic LDS, in floats: where the wavefronts' staged descriptors and ids start
     int stage_rounds;         // rounds staged at a time (1 .. the kernel's STAGE)
     unsigned flags;
@@ -97,6 +98,10 @@ struct AggArgs {
     unsigned delta_l, delta_r;// ... the tables starting at these byte offsets;
     int sentinel;             // ... and a row index whose offset falls outside the window (reads as zero)
 };
+
+// Which workgroup descriptor q belongs to.  (An integer division by a run-time value costs some forty instructions; the
+// kernels that finish rows ask this several times per row.)
+__device__ __forceinline__ int wg_of_part(const AggArgs &a, int q) { return a.ppw_shift >= 0 ? q >> a.ppw_shift : q / a.parts_per_wg; }
 
 // What padding neighbors read on the 64-bit address path: 4 KiB of zeros.
 static __device__ __align__(256) float g_zero_row[1024];
@@ -811,7 +816,7 @@ __global__ void __launch_bounds__(256) k_agg_tail(const AggArgs a, int num_wg, i
         const int2 t = a.c_hdr[2 * b + 1];
         if (!(t.y & HDR_VALID)) return;
         row = t.x;
-        const int n = (a.off[row + 1] - 1) / a.parts_per_wg - (int)b;  // head entries of workgroups b+1 .. b+n
+        const int n = wg_of_part(a, a.off[row + 1] - 1) - (int)b;  // head entries of workgroups b+1 .. b+n
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int c = c0 + i * comp_lanes;
@@ -860,16 +865,18 @@ struct CoreMergeArgs {
     const float4 *partial;  // [slot][group_rows][n4] or NULL
     const int *rank;        // [rows]: rank in the core or -1
     const int *wg_base;     // [core / group_rows + 1]: the slots of row group g are wg_base[g] .. wg_base[g + 1] - 1
-    int group_rows;         // core rows per workgroup of the LDS kernel (CorePlan::group_rows)
+    int group_rows;         // core rows per workgroup of the LDS kernel (CorePlan::group_rows): 256 or 512
+    int group_shift;        // its log2
 };
 
-__global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp, int G,
+__global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp, int g_shift,
                                                             const CoreMergeArgs cm)
 {
     if (gate_closed(a.gate)) return;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    const long long v_ll = idx / G;
-    const int q = (int)(idx % G);
+    const int G = 1 << g_shift;  // lanes per row, a power of two
+    const long long v_ll = idx >> g_shift;
+    const int q = (int)(idx & (G - 1));
     const int n4 = (a.dim + 3) >> 2;
     if (v_ll >= rows) return;  // G divides 64: the lanes of a row leave together
     const int v = (int)v_ll;
@@ -890,14 +897,14 @@ __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, con
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const bool there = c0 + j < blocks && o1[j] > o0[j];
-                chain[j] = there && o0[j] / a.parts_per_wg != (o1[j] - 1) / a.parts_per_wg;
+                chain[j] = there && wg_of_part(a, o0[j]) != wg_of_part(a, o1[j] - 1);
                 p[j] = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (there && !chain[j]) p[j] = *reinterpret_cast<const float4 *>(part + ((long long)(c0 + j) * rows + v) * ldp + 4 * q);
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 if (chain[j]) {  // the row crossed workgroups in this block: tail entry of the first, head entries of the others
-                    const int w0 = o0[j] / a.parts_per_wg, w1 = (o1[j] - 1) / a.parts_per_wg;
+                    const int w0 = wg_of_part(a, o0[j]), w1 = wg_of_part(a, o1[j] - 1);
                     p[j] = *reinterpret_cast<const float4 *>(a.c_val + (size_t)(2 * w0 + 1) * a.cpad + 4 * q);
                     for (int w = w0 + 1; w <= w1; ++w) {
                         const float4 h = *reinterpret_cast<const float4 *>(a.c_val + (size_t)(2 * w) * a.cpad + 4 * q);
@@ -910,11 +917,11 @@ __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, con
         if (cm.partial) {
             const int r = cm.rank[v];
             if (r >= 0) {
-                const int grp = r / cm.group_rows;
+                const int grp = r >> cm.group_shift;
                 int slot = cm.wg_base[grp];
                 const int slot_end = cm.wg_base[grp + 1];
                 const size_t stride = (size_t)cm.group_rows * n4;
-                const float4 *src = cm.partial + (size_t)(r % cm.group_rows) * n4 + q;
+                const float4 *src = cm.partial + (size_t)(r & (cm.group_rows - 1)) * n4 + q;
                 for (; slot + 4 <= slot_end; slot += 4) {  // four partial rows in flight, summed in order
                     const float4 p0 = src[(size_t)slot * stride], p1 = src[(size_t)(slot + 1) * stride];
                     const float4 p2 = src[(size_t)(slot + 2) * stride], p3 = src[(size_t)(slot + 3) * stride];
@@ -1090,6 +1097,9 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     a.dist = dist;
     a.cpad = cpad;
     a.parts_per_wg = (int)parts_per_wg;
+    a.ppw_shift = -1;
+    if ((parts_per_wg & (parts_per_wg - 1)) == 0)
+        for (a.ppw_shift = 0; (1LL << a.ppw_shift) < parts_per_wg;) ++a.ppw_shift;
     a.flags = blocked ? 0u : o.flags;
     a.eps = o.eps;
     a.in_is_bf16 = o.in_dtype == MGGX_BF16;
@@ -1181,15 +1191,17 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         r.ld_out = ld_out;
         r.rs_out = o.d_row_scale_out;
         r.flags = o.flags;
-        CoreMergeArgs cma{nullptr, nullptr, nullptr, CORE_GROUP_ROWS};
+        CoreMergeArgs cma{nullptr, nullptr, nullptr, CORE_GROUP_ROWS, 8};
         if (cm) {
             MGGX_HIP(hipStreamWaitEvent(st.stream, cm->join, 0));
-            cma = CoreMergeArgs{cm->partial, cm->rank, cm->wg_base, cm->group_rows};
+            cma = CoreMergeArgs{cm->partial, cm->rank, cm->wg_base, cm->group_rows, cm->group_rows == CORE_GROUP_ROWS_WIDE ? 9 : 8};
             cm->merged = true;
         }
         const int G = pow2_ceil((dim + 3) / 4);
+        int g_shift = 0;
+        while ((1 << g_shift) < G) ++g_shift;
         const long long n = (long long)plan->real_rows * G;
-        k_agg_finish_blocked<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(r, part, plan->real_rows, plan->blocks, ldp, G, cma);
+        k_agg_finish_blocked<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(r, part, plan->real_rows, plan->blocks, ldp, g_shift, cma);
         MGGX_LAUNCH_CHECK("k_agg_finish_blocked");
     } else {
         // rows that cross workgroups and rows without neighbors, in one launch

@@ -57,18 +57,21 @@ constexpr int CORE_TC = 256;    // core columns per LDS tile
 
 // tab[s * tab_stride(core) + i] = elements 4 s .. 4 s + 3 of the feature row of the rank-i node (zero past dim)
 __global__ void __launch_bounds__(256) k_core_stage(v4f *__restrict__ tab, const float *__restrict__ in, const int *__restrict__ order,
-                                                    int core, int n4, int dim, long long ld_in, const Gate gate)
+                                                    int core, int n4, int dim, long long ld_in, int vec_in, const Gate gate)
 {
     if (gate_closed(gate)) return;
-    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (long long)core * n4) return;
-    const int s = (int)(idx / core), i = (int)(idx % core);
+    const int i = (int)(blockIdx.x * 256 + threadIdx.x), s = (int)blockIdx.y;  // (no division by a run-time value: one slice per grid row)
+    if (i >= core) return;
     const float *row = in + (long long)order[i] * ld_in + 4 * s;
     v4f v;
-    v.x = 4 * s < dim ? row[0] : 0.f;
-    v.y = 4 * s + 1 < dim ? row[1] : 0.f;
-    v.z = 4 * s + 2 < dim ? row[2] : 0.f;
-    v.w = 4 * s + 3 < dim ? row[3] : 0.f;
+    if (vec_in && 4 * s + 3 < dim) {
+        v = *reinterpret_cast<const v4f *>(row);
+    } else {
+        v.x = 4 * s < dim ? row[0] : 0.f;
+        v.y = 4 * s + 1 < dim ? row[1] : 0.f;
+        v.z = 4 * s + 2 < dim ? row[2] : 0.f;
+        v.w = 4 * s + 3 < dim ? row[3] : 0.f;
+    }
     tab[(size_t)s * tab_stride(core) + i] = v;
 }
 
@@ -154,13 +157,15 @@ __global__ void __launch_bounds__(WAVES * 64) MGGX_CORE_OCCUPANCY k_core_sell(co
 // (index -> rank -> row); all_rows = 1: every row (needed when there is a post-operation).
 __global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, const v4f *__restrict__ partial, const int *__restrict__ rank,
                                                      const int *__restrict__ order, const float *__restrict__ rs, int rows, int dim,
-                                                     long long ld_out, int core, const int *__restrict__ wg_base, int group_rows, int G, int relu,
-                                                     int softmax, int all_rows, const Gate gate)
+                                                     long long ld_out, int core, const int *__restrict__ wg_base, int group_shift, int g_shift, int relu,
+                                                     int softmax, int all_rows, int vec_out, const Gate gate)
 {
     if (gate_closed(gate)) return;
+    // lanes per row and core rows per row group are powers of two: shifts, not divisions by run-time values
+    const int G = 1 << g_shift, group_rows = 1 << group_shift;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-    const long long i_ll = idx / G;
-    const int q = (int)(idx % G), n4 = (dim + 3) >> 2;
+    const long long i_ll = idx >> g_shift;
+    const int q = (int)(idx & (G - 1)), n4 = (dim + 3) >> 2;
     if (i_ll >= (all_rows ? rows : core)) return;  // G divides 64: the lanes of a row leave together
     const int i = (int)i_ll;
     const int v = all_rows ? i : order[i];
@@ -169,18 +174,38 @@ __global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, co
     float val[4] = {0.f, 0.f, 0.f, 0.f};
     bool on[4];
     float *o = out + (long long)v * ld_out + 4 * q;
+    const bool whole = vec_out && 4 * q + 3 < dim;  // this lane's four elements as one 16-byte access
     if (lane_on) {
         v4f sum = {0.f, 0.f, 0.f, 0.f};
+        v4f cur = {0.f, 0.f, 0.f, 0.f};
+        if (whole) {
+            cur = *reinterpret_cast<const v4f *>(o);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (4 * q + j < dim) cur[j] = o[j];
+        }
         if (r >= 0) {
-            const int grp = r / group_rows, in_grp = r % group_rows;
+            const int grp = r >> group_shift, in_grp = r & (group_rows - 1);
             const int s1 = wg_base[grp + 1];
-            for (int slot = wg_base[grp]; slot < s1; ++slot) sum += partial[((size_t)slot * group_rows + in_grp) * n4 + q];
+            int slot = wg_base[grp];
+            const size_t stride = (size_t)group_rows * n4;
+            const v4f *src = partial + (size_t)in_grp * n4 + q;
+            for (; slot + 4 <= s1; slot += 4) {  // four partial rows in flight, summed in order
+                const v4f p0 = src[(size_t)slot * stride], p1 = src[(size_t)(slot + 1) * stride];
+                const v4f p2 = src[(size_t)(slot + 2) * stride], p3 = src[(size_t)(slot + 3) * stride];
+                sum += p0;
+                sum += p1;
+                sum += p2;
+                sum += p3;
+            }
+            for (; slot < s1; ++slot) sum += src[(size_t)slot * stride];
             if (rs) sum *= rs[v];
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             on[j] = 4 * q + j < dim;
-            val[j] = on[j] ? o[j] + sum[j] : 0.f;
+            val[j] = on[j] ? cur[j] + sum[j] : 0.f;
             if (relu) val[j] = fmaxf(val[j], 0.f);
         }
     } else {
@@ -205,9 +230,13 @@ __global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, co
         for (int j = 0; j < 4; ++j) val[j] *= inv;
     }
     if (lane_on) {
+        if (whole) {
+            *reinterpret_cast<v4f *>(o) = (v4f){val[0], val[1], val[2], val[3]};
+        } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (on[j]) o[j] = val[j];
+            for (int j = 0; j < 4; ++j)
+                if (on[j]) o[j] = val[j];
+        }
     }
 }
 
@@ -731,8 +760,8 @@ int run_core_stage(CorePlan *p, const float *d_in, int dim, long long ld_in, con
     v4f *tab = nullptr, *partial = nullptr;
     int rc = core_scratch(p, n4, &tab, &partial);
     if (rc) return rc;
-    const long long n = (long long)p->core * n4;
-    k_core_stage<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(tab, d_in, p->d_order, p->core, n4, dim, ld_in, gate);
+    const int vec_in = ld_in % 4 == 0 && (reinterpret_cast<uintptr_t>(d_in) & 15u) == 0;
+    k_core_stage<<<dim3((unsigned)((p->core + 255) / 256), (unsigned)n4), dim3(256), 0, stream>>>(tab, d_in, p->d_order, p->core, n4, dim, ld_in, vec_in, gate);
     MGGX_LAUNCH_CHECK("k_core_stage");
     return MGGX_OK;
 }
@@ -766,11 +795,13 @@ int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const 
     int rc = core_scratch(p, n4, &tab, &partial, &cut);  // sized by run_core_sums already: only hands the pointers out
     if (rc) return rc;
     const int all_rows = (relu || softmax) ? 1 : 0;
-    int G = 1;
-    while (G < n4) G <<= 1;
-    const long long n = (long long)(all_rows ? p->rows : p->core) * G;
+    int g_shift = 0;
+    while ((1 << g_shift) < n4) ++g_shift;
+    const long long n = (long long)(all_rows ? p->rows : p->core) << g_shift;
+    const int vec_out = ld_out % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0;
     k_core_finish<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(d_out, partial, p->d_rank, p->d_order, d_row_scale, p->rows, dim, ld_out,
-                                                                                p->core, cut->d_wg_base, p->group_rows, G, relu, softmax, all_rows, gate);
+                                                                                p->core, cut->d_wg_base, p->group_rows == CORE_GROUP_ROWS_WIDE ? 9 : 8, g_shift,
+                                                                                relu, softmax, all_rows, vec_out, gate);
     MGGX_LAUNCH_CHECK("k_core_finish");
     return MGGX_OK;
 }

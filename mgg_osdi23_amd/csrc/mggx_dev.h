@@ -132,6 +132,7 @@ struct Plan {
 __host__ __device__ inline size_t tab_stride(int core) { return (size_t)core + 16; }
 constexpr int CORE_GROUP_ROWS = 256;  // core rows per workgroup of the LDS kernel (4 wavefronts, one row per lane) ...
 constexpr int CORE_GROUP_ROWS_WIDE = 512;  // ... and where rows are summed in two halves (CorePlan::group_rows)
+static_assert(CORE_GROUP_ROWS == 1 << 8 && CORE_GROUP_ROWS_WIDE == 1 << 9, "the kernels that finish rows shift by 8 or 9");
 // Wide groups where rows are summed in halves and the staged table is well beyond an L2 (12 MB = three of them): every
 // row group re-reads that table once per call.  Held against graphs of width 64 that the setting was not read off: cores
 // of 16.8-21 MB gain 3-7 %, one of 10.5 MB lost 7 % with wide groups (profiles/rules_on_held_out_graphs.md).
