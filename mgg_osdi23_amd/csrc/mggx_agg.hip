@@ -862,11 +862,8 @@ __global__ void __launch_bounds__(256) k_agg_tail(const AggArgs a, int num_wg, i
 // plan's row offsets, so no fix-up pass, no zero fill and no separate reduction run.  G lanes per row (a power of two
 // >= dim/4), lane q holds columns 4 q .. 4 q + 3; the epilogue is the caller's (row scale, accumulate, ReLU, softmax).
 struct CoreMergeArgs {
-    const float4 *partial;  // [slot][group_rows][n4] or NULL
-    const int *rank;        // [rows]: rank in the core or -1
-    const int *wg_base;     // [core / group_rows + 1]: the slots of row group g are wg_base[g] .. wg_base[g + 1] - 1
-    int group_rows;         // core rows per workgroup of the LDS kernel (CorePlan::group_rows): 256 or 512
-    int group_shift;        // its log2
+    const float4 *sums;  // [core][n4]: the dense core's sum per core row, indexed by rank (k_core_reduce), or NULL
+    const int *rank;     // [rows]: rank in the core or -1
 };
 
 __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp, int g_shift,
@@ -914,26 +911,11 @@ __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, con
                 t.x += p[j].x; t.y += p[j].y; t.z += p[j].z; t.w += p[j].w;
             }
         }
-        if (cm.partial) {
+        if (cm.sums) {
             const int r = cm.rank[v];
             if (r >= 0) {
-                const int grp = r >> cm.group_shift;
-                int slot = cm.wg_base[grp];
-                const int slot_end = cm.wg_base[grp + 1];
-                const size_t stride = (size_t)cm.group_rows * n4;
-                const float4 *src = cm.partial + (size_t)(r & (cm.group_rows - 1)) * n4 + q;
-                for (; slot + 4 <= slot_end; slot += 4) {  // four partial rows in flight, summed in order
-                    const float4 p0 = src[(size_t)slot * stride], p1 = src[(size_t)(slot + 1) * stride];
-                    const float4 p2 = src[(size_t)(slot + 2) * stride], p3 = src[(size_t)(slot + 3) * stride];
-                    t.x += p0.x; t.y += p0.y; t.z += p0.z; t.w += p0.w;
-                    t.x += p1.x; t.y += p1.y; t.z += p1.z; t.w += p1.w;
-                    t.x += p2.x; t.y += p2.y; t.z += p2.z; t.w += p2.w;
-                    t.x += p3.x; t.y += p3.y; t.z += p3.z; t.w += p3.w;
-                }
-                for (; slot < slot_end; ++slot) {
-                    const float4 p = src[(size_t)slot * stride];
-                    t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
-                }
+                const float4 p = cm.sums[(size_t)r * n4 + q];
+                t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
             }
         }
     }
@@ -1002,10 +984,9 @@ struct FixedScratch {
 // the caller's whole epilogue (`merged` is set); otherwise the post-operations (ReLU, softmax) are left out here and the
 // caller adds the core afterwards.
 struct CoreMerge {
-    const float4 *partial;
+    const float4 *sums;
     const int *rank;
-    const int *wg_base;
-    int group_rows;
+    int group_rows;  // of the core beside this call (the rules look at it)
     hipEvent_t join;
     bool merged;
 };
@@ -1191,10 +1172,10 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         r.ld_out = ld_out;
         r.rs_out = o.d_row_scale_out;
         r.flags = o.flags;
-        CoreMergeArgs cma{nullptr, nullptr, nullptr, CORE_GROUP_ROWS, 8};
+        CoreMergeArgs cma{nullptr, nullptr};
         if (cm) {
             MGGX_HIP(hipStreamWaitEvent(st.stream, cm->join, 0));
-            cma = CoreMergeArgs{cm->partial, cm->rank, cm->wg_base, cm->group_rows, cm->group_rows == CORE_GROUP_ROWS_WIDE ? 9 : 8};
+            cma = CoreMergeArgs{cm->sums, cm->rank};
             cm->merged = true;
         }
         const int G = pow2_ceil((dim + 3) / 4);
@@ -1313,8 +1294,8 @@ int run_knobs(const GraphInfo &g, const Knobs &k, float *d_out, const void *d_in
             const hipError_t er = hipEventRecord(join, side);
             int rc2 = MGGX_OK;
             GraphInfo *gr = nullptr;
-            CoreMerge cm{nullptr, cp->d_rank, nullptr, cp->group_rows, join, false};
-            if (!rc) rc2 = core_partial_rows(cp, dim, &cm.partial, &cm.wg_base);
+            CoreMerge cm{nullptr, cp->d_rank, cp->group_rows, join, false};
+            if (!rc) rc2 = core_row_sums(cp, dim, &cm.sums);
             if (!rc && !rc2) rc2 = graph_info(cp->d_rem_ptr, nullptr, cp->d_rem_col, nullptr, ub - lb, true, &gr);
             if (!rc && !rc2 && er == hipSuccess) {
                 Knobs k2 = k;

@@ -155,14 +155,46 @@ __global__ void __launch_bounds__(WAVES * 64) MGGX_CORE_OCCUPANCY k_core_sell(co
 // and / or row softmax.
 // G lanes per row (a power of two >= ceil(dim/4)), lane q holds columns 4 q .. 4 q + 3.  all_rows = 0: the core rows only
 // (index -> rank -> row); all_rows = 1: every row (needed when there is a post-operation).
-__global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, const v4f *__restrict__ partial, const int *__restrict__ rank,
-                                                     const int *__restrict__ order, const float *__restrict__ rs, int rows, int dim,
-                                                     long long ld_out, int core, const int *__restrict__ wg_base, int group_shift, int g_shift, int relu,
-                                                     int softmax, int all_rows, int vec_out, const Gate gate)
+// The partial rows of a row group (one per workgroup that worked on it) summed, in slot order, into one row per core row:
+// sums[r * n4 + q], r = rank.  It follows the LDS kernel on its stream, which as a rule is done before the gather kernel
+// beside it, so the kernel that finishes the rows after the join reads one partial row per core row at an address the
+// rank alone gives (one dependent load instead of the row group's slot range and a walk over up to a dozen slots;
+// 36,864 core rows of the 233 K-node graph at width 41: 113 -> 62 us of finishing kernel went into that walk).  `sums` is
+// the staged table's memory, which nobody reads once the LDS kernel has finished.
+__global__ void __launch_bounds__(256) k_core_reduce(v4f *__restrict__ sums, const v4f *__restrict__ partial, const int *__restrict__ wg_base, int core,
+                                                     int n4, int group_shift, int g_shift, const Gate gate)
 {
     if (gate_closed(gate)) return;
-    // lanes per row and core rows per row group are powers of two: shifts, not divisions by run-time values
     const int G = 1 << g_shift, group_rows = 1 << group_shift;
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long r_ll = idx >> g_shift;
+    const int q = (int)(idx & (G - 1));
+    if (r_ll >= core || q >= n4) return;
+    const int r = (int)r_ll, grp = r >> group_shift, in_grp = r & (group_rows - 1);
+    const int s1 = wg_base[grp + 1];
+    int slot = wg_base[grp];
+    const size_t stride = (size_t)group_rows * n4;
+    const v4f *src = partial + (size_t)in_grp * n4 + q;
+    v4f sum = {0.f, 0.f, 0.f, 0.f};
+    for (; slot + 4 <= s1; slot += 4) {  // four partial rows in flight, summed in order
+        const v4f p0 = src[(size_t)slot * stride], p1 = src[(size_t)(slot + 1) * stride];
+        const v4f p2 = src[(size_t)(slot + 2) * stride], p3 = src[(size_t)(slot + 3) * stride];
+        sum += p0;
+        sum += p1;
+        sum += p2;
+        sum += p3;
+    }
+    for (; slot < s1; ++slot) sum += src[(size_t)slot * stride];
+    sums[(size_t)r * n4 + q] = sum;
+}
+
+__global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, const v4f *__restrict__ sums, const int *__restrict__ rank,
+                                                     const int *__restrict__ order, const float *__restrict__ rs, int rows, int dim,
+                                                     long long ld_out, int core, int g_shift, int relu, int softmax, int all_rows, int vec_out,
+                                                     const Gate gate)
+{
+    if (gate_closed(gate)) return;
+    const int G = 1 << g_shift;  // lanes per row, a power of two: shifts, not divisions by a run-time value
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     const long long i_ll = idx >> g_shift;
     const int q = (int)(idx & (G - 1)), n4 = (dim + 3) >> 2;
@@ -186,20 +218,7 @@ __global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, co
                 if (4 * q + j < dim) cur[j] = o[j];
         }
         if (r >= 0) {
-            const int grp = r >> group_shift, in_grp = r & (group_rows - 1);
-            const int s1 = wg_base[grp + 1];
-            int slot = wg_base[grp];
-            const size_t stride = (size_t)group_rows * n4;
-            const v4f *src = partial + (size_t)in_grp * n4 + q;
-            for (; slot + 4 <= s1; slot += 4) {  // four partial rows in flight, summed in order
-                const v4f p0 = src[(size_t)slot * stride], p1 = src[(size_t)(slot + 1) * stride];
-                const v4f p2 = src[(size_t)(slot + 2) * stride], p3 = src[(size_t)(slot + 3) * stride];
-                sum += p0;
-                sum += p1;
-                sum += p2;
-                sum += p3;
-            }
-            for (; slot < s1; ++slot) sum += src[(size_t)slot * stride];
+            sum = sums[(size_t)r * n4 + q];
             if (rs) sum *= rs[v];
         }
 #pragma unroll
@@ -782,7 +801,14 @@ int run_core_sums(CorePlan *p, int dim, const Gate &gate, hipStream_t stream)
 #undef MGGX_CASE
         default: rc = fail(MGGX_ELIMIT, "core: dim %d", dim);
     }
-    return rc;
+    if (rc) return rc;
+    int g_shift = 0;
+    while ((1 << g_shift) < n4) ++g_shift;
+    const long long n = (long long)p->core << g_shift;
+    k_core_reduce<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(tab, partial, cut->d_wg_base, p->core, n4,
+                                                                                p->group_rows == CORE_GROUP_ROWS_WIDE ? 9 : 8, g_shift, gate);
+    MGGX_LAUNCH_CHECK("k_core_reduce");
+    return MGGX_OK;
 }
 
 // out += scale * (partial rows of the core), then the ReLU and / or the row softmax if asked for, on `stream`.
@@ -799,22 +825,20 @@ int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const 
     while ((1 << g_shift) < n4) ++g_shift;
     const long long n = (long long)(all_rows ? p->rows : p->core) << g_shift;
     const int vec_out = ld_out % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0;
-    k_core_finish<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(d_out, partial, p->d_rank, p->d_order, d_row_scale, p->rows, dim, ld_out,
-                                                                                p->core, cut->d_wg_base, p->group_rows == CORE_GROUP_ROWS_WIDE ? 9 : 8, g_shift,
-                                                                                relu, softmax, all_rows, vec_out, gate);
+    k_core_finish<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream>>>(d_out, tab, p->d_rank, p->d_order, d_row_scale, p->rows, dim, ld_out,
+                                                                                p->core, g_shift, relu, softmax, all_rows, vec_out, gate);
     MGGX_LAUNCH_CHECK("k_core_finish");
     return MGGX_OK;
 }
 
-int core_partial_rows(CorePlan *p, int dim, const float4 **partial_out, const int **wg_base)
+// Where k_core_reduce leaves the core's sums of the call in flight: [core][n4] pieces of 16 bytes, indexed by rank.
+int core_row_sums(CorePlan *p, int dim, const float4 **sums)
 {
     const int n4 = (dim + 3) / 4;
     v4f *tab = nullptr, *partial = nullptr;
-    const CorePlan::Cut *cut = nullptr;
-    const int rc = core_scratch(p, n4, &tab, &partial, &cut);
+    const int rc = core_scratch(p, n4, &tab, &partial);
     if (rc) return rc;
-    *wg_base = cut->d_wg_base;
-    *partial_out = reinterpret_cast<const float4 *>(partial);
+    *sums = reinterpret_cast<const float4 *>(tab);
     return MGGX_OK;
 }
 

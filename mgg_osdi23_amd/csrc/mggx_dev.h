@@ -284,7 +284,7 @@ int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const 
                     hipStream_t stream);
 // Where run_core_sums leaves the core block's sums: [slot][row in its group][ceil(dim/4)] float4, and the first slot of
 // every row group (CorePlan::Cut::d_wg_base of the cut used for this width).
-int core_partial_rows(CorePlan *p, int dim, const float4 **partial, const int **wg_base);
+int core_row_sums(CorePlan *p, int dim, const float4 **sums);
 // Second stream of the dense-core path (created on first use, default priority) and the two events that fork and join it.
 int core_side_stream(hipStream_t *stream, hipEvent_t *fork, hipEvent_t *join);
 
