@@ -395,7 +395,7 @@ def bench_gcn2(args, torch, host):
         agg2["frac_traffic"] = round(agg2["traffic"] / (avg["agg2"] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)
     agg2["gather_ceiling"] = gather_ceiling(torch, host, pitch * 4, ldo * 4, V, nnz, avg["agg2"], core_edges if k2.core > 0 else 0)
     extra["launches_per_forward"] = ("dense 1 + aggregation %d + dense 1 + aggregation %d (softmax inside)" %
-                                     ((4, 4) if k2.core > 0 and k2.blk > 0 else ((5, 5) if k2.core > 0 else (2, 2))))
+                                     ((5, 5) if k2.core > 0 and k2.blk > 0 else ((6, 6) if k2.core > 0 else (2, 2))))
     extra["agg2_cache_resident"] = agg2
     extra.update({
         "stage_ms": {k: round(v, 4) for k, v in med.items()},
