@@ -603,6 +603,45 @@ MGGX_EXPORT int mggx_fill_uniform(float *dst, int64_t n, float lo, float hi, uin
 // Dense-core layout (see mggx_internal.h).
 namespace mggx {
 
+// The lists of every (slice, tile) block in bank order, as k_core_bank_order leaves them on the GPU: per lane and window of
+// 64 positions, the entries go by column mod 8 into eight queues (edge order inside a queue) and position p takes from
+// queue (lane + p) mod 8, or the next queue that still holds an entry.
+void core_bank_order(unsigned short *idx, const unsigned *blk_off, size_t cells)
+{
+#pragma omp parallel for schedule(dynamic, 64)
+    for (long long cell = 0; cell < (long long)cells; ++cell) {
+        const unsigned b0 = blk_off[cell], b1 = blk_off[cell + 1];
+        unsigned short win[64], srt[64];
+        for (int lane = 0; lane < 64; ++lane)
+            for (unsigned w0 = b0; w0 < b1; w0 += 16) {
+                const int nch = (int)std::min<unsigned>(16u, b1 - w0);
+                int n = 0, cnt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                for (int c = 0; c < nch; ++c)
+                    for (int j = 0; j < 4; ++j) {
+                        const unsigned short v = idx[((size_t)(w0 + c) * 64 + lane) * 4 + j];
+                        if (v != 0xFFFF) {
+                            win[n++] = v;
+                            ++cnt[v & 7];
+                        }
+                    }
+                if (n < 2) continue;
+                int head[8], tail[8], at = 0;
+                for (int g = 0; g < 8; ++g) {
+                    head[g] = tail[g] = at;
+                    at += cnt[g];
+                }
+                for (int p = 0; p < n; ++p) srt[tail[win[p] & 7]++] = win[p];
+                int g = lane & 7;
+                for (int p = 0; p < n; ++p) {
+                    while (head[g] == tail[g]) g = (g + 1) & 7;
+                    win[p] = srt[head[g]++];
+                    g = (g + 1) & 7;
+                }
+                for (int p = 0; p < n; ++p) idx[((size_t)(w0 + p / 4) * 64 + lane) * 4 + (p % 4)] = win[p];
+            }
+    }
+}
+
 int core_layout_build(const int *ptr, const int *col, int rows, int lb, int core, int tc, CoreLayout *out)
 {
     if (!ptr || rows < 0 || tc < 64 || tc > 4096 || (tc % 64)) return fail(MGGX_EINVAL, "core layout: bad arguments");
@@ -687,6 +726,7 @@ int core_layout_build(const int *ptr, const int *col, int rows, int lb, int core
         }
     }
     L.core_nnz = core_nnz;
+    core_bank_order(L.idx.data(), L.blk_off.data(), (size_t)nslices * ntiles);
     return MGGX_OK;
 }
 

@@ -293,11 +293,28 @@ def test_compact_remote_staging_order(seed):
         host.compact_remote(np.array([3, -1], np.int32))
 
 
+def _bank_order(entries, lane):
+    """A list of tile offsets in edge order -> the order the library stores it in (see test_dense_core_layout)."""
+    out = []
+    for w0 in range(0, len(entries), 64):
+        win = list(entries[w0:w0 + 64])
+        queues = [[e for e in win if e % 8 == g] for g in range(8)]
+        g = lane % 8
+        for _ in win:
+            while not queues[g]:
+                g = (g + 1) % 8
+            out.append(queues[g].pop(0))
+            g = (g + 1) % 8
+    return np.array(out, dtype=np.int64)
+
+
 @pytest.mark.parametrize("lb,core_rows,tile", [(0, 1024, 256), (0, 1700, 256), (300, 512, 64)])
 def test_dense_core_layout(lb, core_rows, tile):
     """The core x core block as index lists plus the remaining CSR, against numpy: ranks by degree (ties by id), every
-    core edge exactly once in the list of its (slice, tile) block at the right tile offset in edge order, padding
-    only behind the entries, everything else left in the CSR in its order."""
+    core edge exactly once in the list of its (slice, tile) block at the right tile offset, the list in bank order
+    (windows of 64 entries; inside a window position p takes the next entry, in edge order, whose column is
+    (lane + p) mod 8 mod 8, or of the next residue that still has one), padding only behind the entries, everything else
+    left in the CSR in its order."""
     V = 4000
     ptr, col = host.gen_rmat(12, V, 120_000, seed=4)
     col = (col + lb).astype(np.int32)  # a share whose rows start at lb: ids are global
@@ -332,7 +349,7 @@ def test_dense_core_layout(lb, core_rows, tile):
             b0, b1 = off[(i // 64) * ntiles + t], off[(i // 64) * ntiles + t + 1]
             got = idx[b0 * 256:b1 * 256].reshape(-1, 64, 4)[:, i % 64, :].reshape(-1)
             assert len(want) <= len(got)
-            assert np.array_equal(got[:len(want)], want) and np.all(got[len(want):] == 0xFFFF)
+            assert np.array_equal(got[:len(want)], _bank_order(want, i % 64)) and np.all(got[len(want):] == 0xFFFF)
             seen += len(want)
     assert seen > 0
     # every block is as long as its longest list, rounded up to 4
