@@ -150,11 +150,6 @@ __global__ void __launch_bounds__(WAVES * 64) MGGX_CORE_OCCUPANCY k_core_sell(co
     }
 }
 
-// Adds the core block's sums to output rows that already hold the rest of the aggregation:
-// out[v] = post(out[v] + scale[v] * sum over the workgroups of v's row group of their partial rows of v), post = ReLU
-// and / or row softmax.
-// G lanes per row (a power of two >= ceil(dim/4)), lane q holds columns 4 q .. 4 q + 3.  all_rows = 0: the core rows only
-// (index -> rank -> row); all_rows = 1: every row (needed when there is a post-operation).
 // The partial rows of a row group (one per workgroup that worked on it) summed, in slot order, into one row per core row:
 // sums[r * n4 + q], r = rank.  It follows the LDS kernel on its stream, which as a rule is done before the gather kernel
 // beside it, so the kernel that finishes the rows after the join reads one partial row per core row at an address the
@@ -188,6 +183,10 @@ __global__ void __launch_bounds__(256) k_core_reduce(v4f *__restrict__ sums, con
     sums[(size_t)r * n4 + q] = sum;
 }
 
+// Adds the core block's sums to output rows that already hold the rest of the aggregation:
+// out[v] = post(out[v] + scale[v] * sums[rank of v]), post = ReLU and / or row softmax.
+// G lanes per row (a power of two >= ceil(dim/4)), lane q holds columns 4 q .. 4 q + 3.  all_rows = 0: the core rows only
+// (index -> rank -> row); all_rows = 1: every row (needed when there is a post-operation).
 __global__ void __launch_bounds__(256) k_core_finish(float *__restrict__ out, const v4f *__restrict__ sums, const int *__restrict__ rank,
                                                      const int *__restrict__ order, const float *__restrict__ rs, int rows, int dim,
                                                      long long ld_out, int core, int g_shift, int relu, int softmax, int all_rows, int vec_out,
@@ -894,7 +893,7 @@ int run_core_sums(CorePlan *p, int dim, const Gate &gate, hipStream_t stream)
     return MGGX_OK;
 }
 
-// out += scale * (partial rows of the core), then the ReLU and / or the row softmax if asked for, on `stream`.
+// out += scale * (the core block's sum of the row, as k_core_reduce left it), then the ReLU and / or the row softmax if asked for, on `stream`.
 int run_core_finish(CorePlan *p, float *d_out, int dim, long long ld_out, const float *d_row_scale, int relu, int softmax, const Gate &gate,
                     hipStream_t stream)
 {
