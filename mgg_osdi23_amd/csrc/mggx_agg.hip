@@ -866,6 +866,7 @@ struct CoreMergeArgs {
     const int *rank;     // [rows]: rank in the core or -1
 };
 
+template <int B>  // blocks per batch: 4, or all of them where a plan has 5 to 8 (one round of dependent loads instead of two)
 __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, const float *__restrict__ part, int rows, int blocks, int ldp, int g_shift,
                                                             const CoreMergeArgs cm)
 {
@@ -880,26 +881,30 @@ __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, con
     float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
     const bool lane_on = q < n4;
     if (lane_on) {
-        // four blocks at a time: their row offsets first, then their partial rows, all in flight before the first sum
-        for (int c0 = 0; c0 < blocks; c0 += 4) {
-            int o0[4], o1[4];
+        int r = -1;  // rank in the dense core: asked for before anything else, its row of sums is read last
+        if (cm.sums) {
+            r = cm.rank[v];
+        }
+        // B blocks at a time: their row offsets first, then their partial rows, all in flight before the first sum
+        for (int c0 = 0; c0 < blocks; c0 += B) {
+            int o0[B], o1[B];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < B; ++j) {
                 const long long vr = (long long)min(c0 + j, blocks - 1) * rows + v;
                 o0[j] = a.off[vr];
                 o1[j] = a.off[vr + 1];
             }
-            float4 p[4];
-            bool chain[4];
+            float4 p[B];
+            bool chain[B];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < B; ++j) {
                 const bool there = c0 + j < blocks && o1[j] > o0[j];
                 chain[j] = there && wg_of_part(a, o0[j]) != wg_of_part(a, o1[j] - 1);
                 p[j] = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (there && !chain[j]) p[j] = *reinterpret_cast<const float4 *>(part + ((long long)(c0 + j) * rows + v) * ldp + 4 * q);
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < B; ++j) {
                 if (chain[j]) {  // the row crossed workgroups in this block: tail entry of the first, head entries of the others
                     const int w0 = wg_of_part(a, o0[j]), w1 = wg_of_part(a, o1[j] - 1);
                     p[j] = *reinterpret_cast<const float4 *>(a.c_val + (size_t)(2 * w0 + 1) * a.cpad + 4 * q);
@@ -912,7 +917,6 @@ __global__ void __launch_bounds__(256) k_agg_finish_blocked(const AggArgs a, con
             }
         }
         if (cm.sums) {
-            const int r = cm.rank[v];
             if (r >= 0) {
                 const float4 p = cm.sums[(size_t)r * n4 + q];
                 t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
@@ -1182,7 +1186,13 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
         int g_shift = 0;
         while ((1 << g_shift) < G) ++g_shift;
         const long long n = (long long)plan->real_rows * G;
-        k_agg_finish_blocked<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st.stream>>>(r, part, plan->real_rows, plan->blocks, ldp, g_shift, cma);
+        const dim3 fgrid((unsigned)((n + 255) / 256));
+        switch (plan->blocks) {
+#define MGGX_CASE(NB) case NB: k_agg_finish_blocked<NB><<<fgrid, dim3(256), 0, st.stream>>>(r, part, plan->real_rows, plan->blocks, ldp, g_shift, cma); break;
+            MGGX_CASE(5) MGGX_CASE(6) MGGX_CASE(7) MGGX_CASE(8)
+#undef MGGX_CASE
+            default: k_agg_finish_blocked<4><<<fgrid, dim3(256), 0, st.stream>>>(r, part, plan->real_rows, plan->blocks, ldp, g_shift, cma);
+        }
         MGGX_LAUNCH_CHECK("k_agg_finish_blocked");
     } else {
         // rows that cross workgroups and rows without neighbors, in one launch
