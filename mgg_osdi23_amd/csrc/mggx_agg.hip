@@ -1039,17 +1039,22 @@ int run_agg(Plan *plan, float *d_out, const void *d_in_l, const void *d_in_r, co
     // works in wide row groups (width 52 to 64, staged table beyond 12 MB: seven graphs of 0.7 to 3 M nodes at width 64 are
     // 1.4 - 3.7 % faster with 8 than with 4, one of them by 0.1 %; at width 48, narrow groups, 8 rounds cost 1.1 %); short
     // rows (under 3 partitions per row): 4 wavefronts.  Many slots (narrow rows): 4 wavefronts, 4 rounds; 8 rounds where a column-blocked
-    // plan is left with short rows (under 8 partitions per row and block).
+    // plan is left with short rows (under 8 partitions per row and block); 2 rounds for rows of 84 to 128 bytes (8 slots)
+    // in row-major order beside a dense core -- there a wavefront's share is 16 partitions, as with 4 slots and 4 rounds.
     // Provenance: wpb x dist sweeps on the three benchmark graphs and the bf16 share (each choice within 1 % of the best
-    // cell there), re-checked on eighteen graphs of other generators, sizes, degrees and widths: within 5.2 % of the best
-    // cell on every one, after one change the first of them forced -- beside a core in row-major order the first version
-    // took 4 wavefronts, which two 1 M-node graphs at widths 41 and 64 answered with 10 - 17 % over 8 wavefronts.
+    // cell there), re-checked on graphs of other generators, sizes, degrees and widths: within 4 % of the best cell on
+    // every one of twenty-four, after two changes they forced -- beside a core in row-major order the first version took
+    // 4 wavefronts, which two 1 M-node graphs at widths 41 and 64 answered with 10 - 17 % over 8 wavefronts; and it took 4
+    // rounds at 8 slots, 4 - 7 % over 2 rounds on two graphs of widths 24 and 32 (then, on three graphs made for the
+    // purpose: widths 24 / 28 / 28 -0.1 / -3.6 / -1.8 % with 2 rounds; two graphs of width 20 were 1.4 and 2.7 % slower with 2,
+    // three of widths 12 to 16 within 0.6 % except one 2.5 % faster: both stay at 4).
     const double per_row = (double)plan->num_parts / (double)(plan->rows > 0 ? plan->rows : 1);
     const bool beside_core = cm != nullptr;
     if (wpb == 0) wpb = (beside_core && !blocked && slots <= 4) ? 8 : (blocked || slots > 4 || per_row < 3.0) ? 4 : 8;
     if (dist == 0) {
         if (slots <= 4) dist = (beside_core && !blocked) ? (cm->group_rows == CORE_GROUP_ROWS_WIDE ? 8 : 4) : 16;
         else if (blocked && per_row < 8.0) dist = 8;
+        else if (beside_core && !blocked && slots == 8 && dim > 20) dist = 2;
         else dist = 4;
     }
     const long long parts_per_wg = (long long)wpb * slots * dist;

@@ -54,6 +54,14 @@ HELD_OUT = {
     "rmat63w64": ("rmat", dict(scale=20, num_nodes=700_000, num_draws=110_000_000, a=0.63, b=0.15, c=0.17, seed=116), 1, 64, 64),
     "rmat58w20": ("rmat", dict(scale=21, num_nodes=1_800_000, num_draws=90_000_000, a=0.58, b=0.18, c=0.18, seed=117), 1, 20, 20),
     "rmat46w16": ("rmat", dict(scale=19, num_nodes=350_000, num_draws=140_000_000, a=0.46, b=0.22, c=0.22, seed=118), 1, 16, 16),
+    # narrow rows beside a dense core in row-major order: made to check a candidate rule (2 rounds per wavefront there);
+    # the graphs of width 20, here and above, set its lower bound; rmat56w24 and rmat59w28 agreed with it and moved nothing
+    "rmat54w28": ("rmat", dict(scale=20, num_nodes=600_000, num_draws=80_000_000, a=0.54, b=0.20, c=0.20, seed=119), 1, 28, 28),
+    "rmat61w12": ("rmat", dict(scale=21, num_nodes=1_200_000, num_draws=70_000_000, a=0.61, b=0.16, c=0.16, seed=120), 1, 12, 12),
+    "rmat49w32": ("rmat", dict(scale=19, num_nodes=450_000, num_draws=110_000_000, a=0.49, b=0.21, c=0.21, seed=121), 1, 32, 32),
+    "rmat56w24": ("rmat", dict(scale=21, num_nodes=1_600_000, num_draws=85_000_000, a=0.56, b=0.19, c=0.19, seed=122), 1, 24, 24),
+    "rmat53w20": ("rmat", dict(scale=19, num_nodes=500_000, num_draws=65_000_000, a=0.53, b=0.20, c=0.20, seed=123), 1, 20, 20),
+    "rmat59w28": ("rmat", dict(scale=20, num_nodes=1_000_000, num_draws=75_000_000, a=0.59, b=0.18, c=0.18, seed=124), 1, 28, 28),
 }
 
 

@@ -354,11 +354,12 @@ def test_full_size_whole_graph_gcn_widths(gpu):
 
 
 # --------------------------------------------------------------------------- rules and cost model on graphs they were not set on
-@pytest.mark.parametrize("name,shrink", [("rmat63w64", 1), ("rmat58w20", 2), ("rmat52w48", 2)])
+@pytest.mark.parametrize("name,shrink", [("rmat63w64", 1), ("rmat59w28", 2), ("rmat52w48", 2)])
 def test_rules_hold_on_graphs_they_never_saw(gpu, name, shrink):
     """The knobs left at 0 (wpb, dist, partition order, dense-core size by the cost model) against the library's own search
-    on graph families that were only ever measured, never used to set a rule or a constant (mgg_osdi23_amd.dse.HELD_OUT,
-    the last four), at a fraction of their size: the rules' setting may be at most 10 % slower than the searched one, and
+    on graph families that were only ever measured, never used to set a rule or a constant (mgg_osdi23_amd.dse.HELD_OUT:
+    two of the four first measured with the rules finished, and one of those made later to check the rounds rule for
+    rows of 8 slots beside a core, which agreed with it), at a fraction of their size: the rules' setting may be at most 10 % slower than the searched one, and
     gives the oracle's sums on sampled rows."""
     import torch
     from mgg_osdi23_amd import dse
