@@ -181,7 +181,10 @@ def test_search_of_wpb_and_dist(gpu, rmat_graph, dim, gin):
 
 
 @pytest.mark.parametrize("dim,block_rows,flags", [(16, 100, "plain"), (44, 64, "scale"), (41, 37, "gin"), (8, 300, "acc_relu"),
-                                                  (64, 128, "plain")])
+                                                  (64, 128, "plain"),
+                                                  # 2 to 8 blocks: the finishing kernel takes all blocks of a row in one batch
+                                                  (16, 3000, "scale"), (12, 2000, "plain"), (41, 1200, "plain"), (16, 1000, "scale"),
+                                                  (24, 860, "acc_relu"), (44, 750, "gin")])
 def test_column_blocked_order(gpu, rmat_graph, dim, block_rows, flags):
     """The column-blocked partition order (whole graph, rows sorted by neighbor id): same sums as the plain order and
     the oracle, with every epilogue; unsorted rows fall back to the plain order silently."""
@@ -278,7 +281,7 @@ def test_dense_core_from_lds(gpu, rmat_graph, dim, core_rows, flags):
         want, mag = want * s[:, None], mag * s[:, None]
     if flags == "acc_relu":
         want, mag = np.maximum(want + base, 0), mag + np.abs(base)
-    for blk, ps, wpb, dist in ((-1, 16, 4, 1), (-1, 4, 2, 3), (300, 32, 8, 16), (0, 0, 0, 0)):
+    for blk, ps, wpb, dist in ((-1, 16, 4, 1), (-1, 4, 2, 3), (300, 32, 8, 16), (1000, 16, 4, 2), (0, 0, 0, 0)):  # 1000: six blocks in one batch
         got = run(core_rows, blk, ps, wpb, dist)
         assert "core=%d" % (core_rows // 512 * 512) in gpu.last_agg_kernel()
         assert_close_to_oracle(got, want, mag, FP32_TOL, "dense core, blk=%d ps=%d wpb=%d dist=%d" % (blk, ps, wpb, dist))
