@@ -146,8 +146,10 @@ int mggx_compact_remote(const int *remote_col, int64_t n_remote, int *remote_col
  * a local CSR by degree (ties by id), takes the first core_rows (rounded down to a multiple of 512) as the core, and
  * splits the CSR into the core x core block -- as index lists per 64-row slice and tile of tile_cols core columns
  * (256 in the library), lists of a slice padded with 0xFFFF to the longest, in chunks of 4:
- * idx[((blk_off[g * ntiles + t] + k / 4) * 64 + lane) * 4 + k % 4] = tile offset of the k-th core neighbor of the row
- * of rank 64 g + lane inside tile t -- and the remaining CSR (rem_ptr, rem_col: row and edge order kept, ids unchanged).
+ * idx[((blk_off[g * ntiles + t] + k / 4) * 64 + lane) * 4 + k % 4] = tile offset of a core neighbor of the row of rank
+ * 64 g + lane inside tile t.  A list is in bank order: inside each window of 64 positions, position k takes the next
+ * entry (in edge order) whose offset is (lane + k) mod 8 mod 8, or of the next residue that still has one --
+ * and the remaining CSR (rem_ptr, rem_col: row and edge order kept, ids unchanged).
  * build returns sizes[5] = {core rows, entries of blk_off, entries of idx, entries of rem_col, edges in the core block};
  * fetch copies the arrays out (any may be NULL) and releases the handle: order[core], rank[rows] (-1 outside the core),
  * blk_off, idx, rem_ptr[rows + 1], rem_col. */
