@@ -145,10 +145,11 @@ int mggx_compact_remote(const int *remote_col, int64_t n_remote, int *remote_col
 /* Layout of the dense-core path (no counterpart in the reference), exposed for inspection and tests: ranks the rows of
  * a local CSR by degree (ties by id), takes the first core_rows (rounded down to a multiple of 512) as the core, and
  * splits the CSR into the core x core block -- as index lists per 64-row slice and tile of tile_cols core columns
- * (256 in the library), lists of a slice padded with 0xFFFF to the longest, in chunks of 4:
+ * (256 in the library), lists of a slice padded to the longest, in chunks of 4:
  * idx[((blk_off[g * ntiles + t] + k / 4) * 64 + lane) * 4 + k % 4] = tile offset of a core neighbor of the row of rank
- * 64 g + lane inside tile t.  A list is in bank order: inside each window of 64 positions, position k takes the next
- * entry (in edge order) whose offset is (lane + k) mod 8 mod 8, or of the next residue that still has one --
+ * 64 g + lane inside tile t, or tile_cols + r (r < 16) for a padding slot: one of 16 zero columns the kernel keeps
+ * behind a tile.  A block is in bank order: entries and padding slots of the 16 lanes of a group are placed so that, as
+ * far as the lists allow, the 16 columns read at one position differ mod 16 (blocks of up to 256 positions) --
  * and the remaining CSR (rem_ptr, rem_col: row and edge order kept, ids unchanged).
  * build returns sizes[5] = {core rows, entries of blk_off, entries of idx, entries of rem_col, edges in the core block};
  * fetch copies the arrays out (any may be NULL) and releases the handle: order[core], rank[rows] (-1 outside the core),

@@ -48,6 +48,7 @@ __device__ __forceinline__ void static_for_core(F &&f)
 }
 
 constexpr int CORE_TC = 256;    // core columns per LDS tile
+constexpr int CORE_ZERO_COLS = 16;  // zero columns behind them: what the lists' padding entries point at (k_core_bank_order)
 // Slices (of 64 rows) per workgroup, WAVES below: 4 -- as small as the aggregation's own workgroups, so the two kernels
 // of a call, running side by side, find room on a CU equally easily -- or 8 where rows are summed in two halves: every
 // workgroup stages every tile of its run, so the tiles staged per call are (row groups) x (tiles); with 98,304 core rows
@@ -81,18 +82,19 @@ __device__ __forceinline__ void core_sell_body(const unsigned *__restrict__ blk_
                                                const v4f *__restrict__ tab, v4f *__restrict__ partial, const int4 wg, int core, int ntiles,
                                                v4f *tile)
 {
-    constexpr int TC = CORE_TC, TP = TC + 1;  // column TC of every slice row is zero: what padding entries read; tile[NS][TP]
+    constexpr int TC = CORE_TC, TP = TC + CORE_ZERO_COLS;  // columns TC .. TP - 1 of every slice row are zero: what padding entries read; tile[NS][TP]
     const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
     const int g = wg.x * WAVES + wave;
     const int t0 = wg.y, t1 = wg.z;
     v4f acc[NS];
 #pragma unroll
     for (int s = 0; s < NS; ++s) acc[s] = (v4f){0.f, 0.f, 0.f, 0.f};
-    if ((int)threadIdx.x < NS) tile[(int)threadIdx.x * TP + TC] = (v4f){0.f, 0.f, 0.f, 0.f};
+    if ((int)threadIdx.x < NS * CORE_ZERO_COLS)
+        tile[((int)threadIdx.x / CORE_ZERO_COLS) * TP + TC + (int)threadIdx.x % CORE_ZERO_COLS] = (v4f){0.f, 0.f, 0.f, 0.f};
     const us4 *p = reinterpret_cast<const us4 *>(idx) + lane;
     unsigned pos = blk_off[(size_t)g * ntiles + t0];
     const unsigned end_run = blk_off[(size_t)g * ntiles + t1];
-    const us4 pad = (us4){0xFFFF, 0xFFFF, 0xFFFF, 0xFFFF};
+    const us4 pad = (us4){TC, TC, TC, TC};
     us4 cur = pos < end_run ? p[(size_t)pos * 64] : pad;  // the lists of a slice's tiles follow one another: read one chunk ahead
     for (int t = t0; t < t1; ++t) {
         __syncthreads();
@@ -107,7 +109,7 @@ __device__ __forceinline__ void core_sell_body(const unsigned *__restrict__ blk_
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int c = cur[j];
-                const v4f *q = tile + (c < TC ? c : TC);
+                const v4f *q = tile + c;  // a column of the tile or, for a padding entry, one of the zero columns behind it
                 // at most MGGX_CORE_READS LDS reads in flight per entry: wide rows otherwise cost a wavefront a hundred
                 // registers, and this kernel shares each SIMD's register file with the aggregation running beside it
                 constexpr int GROUPS = (NS + MGGX_CORE_READS - 1) / MGGX_CORE_READS, H = (NS + GROUPS - 1) / GROUPS;
@@ -282,81 +284,127 @@ __global__ void __launch_bounds__(256) k_core_rank(const int *__restrict__ sorte
     }
 }
 
-// Bank order of the lists.  A wavefront of k_core_sell reads, per list position, one 16-byte piece per lane at the lanes'
-// own columns of the tile; pieces whose columns agree mod 8 share LDS banks, and with the columns in edge order a read
-// takes 1.45 x the cycles of a conflict-free one (54 against 74 TB/s over the chip with every eight neighbouring lanes on
-// eight different columns mod 8).  Which entry of its list a lane reads at which position is free -- the sum does not
-// care -- so every lane's list is re-ordered, 64 positions at a time: the entries of a window go by column mod 8 into
-// eight queues (edge order inside a queue), and position p takes from queue (lane + p) mod 8, or the next queue that
-// still holds one.  Neighbouring lanes then start on different banks and stay so while their queues last.  One
-// wavefront per (slice, tile) list block, lane = list.  The host-side builder does the same (core_bank_order).
-constexpr int BANK_WINDOW = 16;  // chunks of 4 entries per lane
+// Bank order of the lists.  The LDS has 64 banks of 4 bytes: a 16-byte read of a wavefront is served 16 lanes at a time
+// (lanes 16 k .. 16 k + 15 together), in one cycle when the 16 pieces lie in 16 different groups of four banks -- tile
+// columns that differ mod 16 -- and otherwise in as many cycles as the fullest group has distinct addresses (measured
+// with SQ_LDS_BANK_CONFLICT on access patterns made for it: 4 cycles per read at best, 12.2 with random columns; the
+// lists in edge order took 8.3, about a third of the kernel's time).  Which entry of its list a lane reads at which
+// position is free -- the sum does not care -- and so is where in the list its padding goes, so the entries of a
+// (slice, tile) block are placed for the 16 lanes of a group together: position by position, first the lanes that
+// have no padding left to spend, then the others, each in lane order, a lane takes the first of its remaining entries
+// (looking from residue (lane + p) mod 16 upwards, edge order inside a residue) whose residue no lane of the group has
+// taken at this position; a lane that finds none spends a padding slot if it has one, else takes a residue twice.
+// Padding slots point at one of CORE_ZERO_COLS zero columns behind the tile, tc + r, with r the residues still free
+// at that position in turn.  On the 233 K-node benchmark graph that leaves 4.01 cycles per read.  One wavefront per
+// block, lane = list; a block of more than BANK_MAX_POS positions (only a CSR with repeated edges has one) keeps its
+// edge order.  The host-side builder does the same (core_bank_order).
+constexpr int BANK_MAX_POS = 256;
+static_assert(CORE_TC <= 256, "k_core_bank_order keeps tile offsets in bytes");
 
-__global__ void __launch_bounds__(128) k_core_bank_order(const int *__restrict__ blk_off, unsigned short *__restrict__ idx, long long cells)
+// the lowest set bit of the 16-bit mask m when looking from bit k upwards, cyclically; -1 if m is empty
+__device__ __forceinline__ int first_from(unsigned m, int k)
 {
-    __shared__ unsigned short win[2][BANK_WINDOW * 4][64];   // [wavefront][position][lane]: a window in edge order
-    __shared__ unsigned short srt[2][BANK_WINDOW * 4][64];   // ... and by queue
-    const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
-    const long long cell = (long long)blockIdx.x * 2 + wave;
-    if (cell >= cells) return;
-    const unsigned b0 = (unsigned)blk_off[cell], b1 = (unsigned)blk_off[cell + 1];
+    const unsigned mr = ((m >> k) | (m << (16 - k))) & 0xFFFFu;
+    return mr ? ((__ffs((int)mr) - 1 + k) & 15) : -1;
+}
+
+__global__ void __launch_bounds__(64) k_core_bank_order(const int *__restrict__ blk_off, unsigned short *__restrict__ idx, int tc)  // tc <= 256
+{
+    __shared__ unsigned char srt[BANK_MAX_POS][64];    // [position][lane]: a lane's entries (tile offsets below 256) by residue, edge order inside one
+    const int lane = (int)threadIdx.x, i = lane & 15;
+    const unsigned b0 = (unsigned)blk_off[blockIdx.x], b1 = (unsigned)blk_off[blockIdx.x + 1];
+    const int P = 4 * (int)(b1 - b0);
+    if (P == 0) return;
     us4 *lists = reinterpret_cast<us4 *>(idx);
-    for (unsigned w0 = b0; w0 < b1; w0 += BANK_WINDOW) {
-        const int nch = (int)min((unsigned)BANK_WINDOW, b1 - w0);
-        int cnt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        int n = 0;
-        for (int c = 0; c < nch; ++c) {
-            const us4 e = lists[(size_t)(w0 + c) * 64 + lane];
+    if (P > BANK_MAX_POS) {  // more entries than columns (a CSR with repeated edges): edge order, padding on the first zero column
+        for (unsigned c = b0; c < b1; ++c) {
+            us4 e = lists[(size_t)c * 64 + lane];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const unsigned short v = e[j];
-                win[wave][4 * c + j][lane] = v;
-                if (v != 0xFFFF) {
-                    ++n;
+            for (int j = 0; j < 4; ++j) e[j] = e[j] == 0xFFFF ? (unsigned short)tc : e[j];
+            lists[(size_t)c * 64 + lane] = e;
+        }
+        return;
+    }
+    int cnt[16], head[16], tail[16];
 #pragma unroll
-                    for (int g = 0; g < 8; ++g) cnt[g] += (v & 7) == g;
-                }
+    for (int g = 0; g < 16; ++g) cnt[g] = 0;
+    int left = 0;
+    for (unsigned c = b0; c < b1; ++c) {
+        const us4 e = lists[(size_t)c * 64 + lane];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const unsigned short v = e[j];
+            if (v != 0xFFFF) {
+                ++left;
+#pragma unroll
+                for (int g = 0; g < 16; ++g) cnt[g] += (v & 15) == g;
             }
         }
-        if (!__any(n > 1)) continue;  // nothing to re-order in this window
-        // queues: start offsets, then a stable distribution
-        int head[8], tail[8];
+    }
+    unsigned have = 0;
+    {
         int at = 0;
 #pragma unroll
-        for (int g = 0; g < 8; ++g) {
-            head[g] = at;
+        for (int g = 0; g < 16; ++g) {
+            head[g] = tail[g] = at;
             at += cnt[g];
-            tail[g] = head[g];
+            have |= cnt[g] ? 1u << g : 0u;
         }
-        for (int p = 0; p < n; ++p) {  // (padding only follows the entries: the first n positions are the entries)
-            const unsigned short v = win[wave][p][lane];
+    }
+    for (unsigned c = b0; c < b1; ++c) {
+        const us4 e = lists[(size_t)c * 64 + lane];
 #pragma unroll
-            for (int g = 0; g < 8; ++g)
-                if ((v & 7) == g) srt[wave][tail[g]++][lane] = v;
-        }
-        int g = lane & 7;  // window starts are multiples of 64 positions
-        for (int p = 0; p < n; ++p) {
-            int hg = 0, tg = 0;
-            for (int tries = 0; tries < 8; ++tries) {
+        for (int j = 0; j < 4; ++j) {
+            const unsigned short v = e[j];
+            if (v != 0xFFFF) {
 #pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    hg = g == k ? head[k] : hg;
-                    tg = g == k ? tail[k] : tg;
-                }
-                if (hg < tg) break;
-                g = (g + 1) & 7;
+                for (int g = 0; g < 16; ++g)
+                    if ((v & 15) == g) srt[tail[g]++][lane] = (unsigned char)v;
             }
-            win[wave][p][lane] = srt[wave][hg][lane];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) head[k] += g == k;
-            g = (g + 1) & 7;
         }
-        for (int c = 0; c < nch; ++c) {
-            us4 e;
+    }
+    for (int p0 = 0; p0 < P; p0 += 4) {
+        us4 e;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) e[j] = win[wave][4 * c + j][lane];
-            lists[(size_t)(w0 + c) * 64 + lane] = e;
+        for (int j = 0; j < 4; ++j) {
+            const int p = p0 + j;
+            const int slack = P - p - left;  // padding slots this lane has yet to place
+            const int k0 = (i + p) & 15;
+            unsigned used = 0;               // residues taken at this position, the same in all lanes of a group
+            int r = -1;
+            for (int pass = 0; pass < 2; ++pass) {
+                const bool mine = left > 0 && (slack == 0) == (pass == 0);
+                for (int t = 0; t < 16; ++t) {
+                    int rr = -1;
+                    if (mine && i == t) {
+                        rr = first_from(have & ~used, k0);
+                        if (rr < 0 && slack == 0) rr = first_from(have, k0);
+                        r = rr;
+                    }
+                    used |= (unsigned)__shfl(rr >= 0 ? 1 << rr : 0, (lane & 48) | t);
+                }
+            }
+            unsigned short v;
+            const unsigned long long pads = __ballot(r < 0);
+            if (r >= 0) {
+                int h = 0;
+#pragma unroll
+                for (int g = 0; g < 16; ++g) {
+                    h = r == g ? head[g] : h;
+                    head[g] += r == g;
+                    if (r == g && head[g] == tail[g]) have &= ~(1u << g);
+                }
+                v = srt[h][lane];
+                --left;
+            } else {
+                const int k = __popc((unsigned)(pads >> (lane & 48)) & ((1u << i) - 1u));  // padding lanes of the group before this one
+                unsigned f = ~used & 0xFFFFu;
+                for (int t = 0; t < k && f; ++t) f &= f - 1;
+                v = (unsigned short)(tc + (f ? __ffs((int)f) - 1 : (k & 15)));
+            }
+            e[j] = v;
         }
+        lists[(size_t)(b0 + p0 / 4) * 64 + lane] = e;
     }
 }
 
@@ -508,7 +556,7 @@ int launch_sell_as(const CorePlan *p, const CorePlan::Cut &cut, const v4f *tab, 
 {
     constexpr bool SPLIT = N4 > 12;
     constexpr int NS = SPLIT ? (N4 + 1) / 2 : N4;
-    size_t lds = (size_t)NS * (CORE_TC + 1) * sizeof(v4f);
+    size_t lds = (size_t)NS * (CORE_TC + CORE_ZERO_COLS) * sizeof(v4f);
     if (SPLIT) lds = std::max<size_t>(lds, (160u << 10) / (WAVES == 8 ? 3 : 4) + 256);
     static bool raised = false;  // per instantiation
     if (lds > 48 * 1024 && !raised) {
@@ -680,7 +728,7 @@ static int core_plan_build_device(CorePlan *p, int tc)
     MGGX_LAUNCH_CHECK("k_core_fill");
     {
         const long long cells = (long long)(core / 64) * ntiles;
-        k_core_bank_order<<<(unsigned)((cells + 1) / 2), 128, 0, s.stream>>>(blk, p->d_idx, cells);
+        k_core_bank_order<<<(unsigned)cells, 64, 0, s.stream>>>(blk, p->d_idx, tc);
         MGGX_LAUNCH_CHECK("k_core_bank_order");
     }
     MGGX_HIP(hipStreamSynchronize(s.stream));

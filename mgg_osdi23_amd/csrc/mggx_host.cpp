@@ -603,42 +603,78 @@ MGGX_EXPORT int mggx_fill_uniform(float *dst, int64_t n, float lo, float hi, uin
 // Dense-core layout (see mggx_internal.h).
 namespace mggx {
 
-// The lists of every (slice, tile) block in bank order, as k_core_bank_order leaves them on the GPU: per lane and window of
-// 64 positions, the entries go by column mod 8 into eight queues (edge order inside a queue) and position p takes from
-// queue (lane + p) mod 8, or the next queue that still holds an entry.
-void core_bank_order(unsigned short *idx, const unsigned *blk_off, size_t cells)
+// The lists of every (slice, tile) block in bank order, as k_core_bank_order leaves them on the GPU.  The 16 lanes of a
+// group are placed together: position by position, first the lanes without padding left to spend, then the others, each
+// in lane order, a lane takes the first of its remaining entries (looking from residue (lane + p) mod 16 upwards, edge
+// order inside a residue) whose residue no lane of the group has taken at this position; a lane that finds none spends
+// a padding slot if it has one, else takes a residue twice.  Padding slots become tc + r, r being the residues still
+// free at that position in turn (the k-th padding lane of the group takes the k-th free one, or k mod 16).
+static int first_from(unsigned m, int k)
+{
+    const unsigned mr = ((m >> k) | (m << (16 - k))) & 0xFFFFu;
+    return mr ? ((__builtin_ctz(mr) + k) & 15) : -1;
+}
+
+void core_bank_order(unsigned short *idx, const unsigned *blk_off, size_t cells, int tc)
 {
 #pragma omp parallel for schedule(dynamic, 64)
     for (long long cell = 0; cell < (long long)cells; ++cell) {
         const unsigned b0 = blk_off[cell], b1 = blk_off[cell + 1];
-        unsigned short win[64], srt[64];
-        for (int lane = 0; lane < 64; ++lane)
-            for (unsigned w0 = b0; w0 < b1; w0 += 16) {
-                const int nch = (int)std::min<unsigned>(16u, b1 - w0);
-                int n = 0, cnt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-                for (int c = 0; c < nch; ++c)
-                    for (int j = 0; j < 4; ++j) {
-                        const unsigned short v = idx[((size_t)(w0 + c) * 64 + lane) * 4 + j];
-                        if (v != 0xFFFF) {
-                            win[n++] = v;
-                            ++cnt[v & 7];
-                        }
+        const int P = 4 * (int)(b1 - b0);
+        if (P == 0) continue;
+        auto at = [&](int p, int lane) -> unsigned short & { return idx[((size_t)(b0 + p / 4) * 64 + lane) * 4 + (p % 4)]; };
+        if (P > 256) {  // as on the GPU: such a block keeps its edge order, its padding points at the first zero column
+            for (int p = 0; p < P; ++p)
+                for (int lane = 0; lane < 64; ++lane)
+                    if (at(p, lane) == 0xFFFF) at(p, lane) = (unsigned short)tc;
+            continue;
+        }
+        for (int grp = 0; grp < 4; ++grp) {
+            std::vector<unsigned short> q[16][16];  // [lane of the group][residue]: entries in edge order
+            size_t head[16][16] = {};
+            int left[16];
+            unsigned have[16];
+            for (int i = 0; i < 16; ++i) {
+                left[i] = 0;
+                have[i] = 0;
+                for (int p = 0; p < P; ++p) {
+                    const unsigned short v = at(p, 16 * grp + i);
+                    if (v != 0xFFFF) {
+                        q[i][v & 15].push_back(v);
+                        have[i] |= 1u << (v & 15);
+                        ++left[i];
                     }
-                if (n < 2) continue;
-                int head[8], tail[8], at = 0;
-                for (int g = 0; g < 8; ++g) {
-                    head[g] = tail[g] = at;
-                    at += cnt[g];
                 }
-                for (int p = 0; p < n; ++p) srt[tail[win[p] & 7]++] = win[p];
-                int g = lane & 7;
-                for (int p = 0; p < n; ++p) {
-                    while (head[g] == tail[g]) g = (g + 1) & 7;
-                    win[p] = srt[head[g]++];
-                    g = (g + 1) & 7;
-                }
-                for (int p = 0; p < n; ++p) idx[((size_t)(w0 + p / 4) * 64 + lane) * 4 + (p % 4)] = win[p];
             }
+            for (int p = 0; p < P; ++p) {
+                unsigned used = 0;
+                int r[16];
+                for (int i = 0; i < 16; ++i) r[i] = -1;
+                for (int pass = 0; pass < 2; ++pass)
+                    for (int i = 0; i < 16; ++i) {
+                        const int slack = P - p - left[i];
+                        if (left[i] == 0 || (slack == 0) != (pass == 0)) continue;
+                        const int k0 = (i + p) & 15;
+                        int rr = first_from(have[i] & ~used, k0);
+                        if (rr < 0 && slack == 0) rr = first_from(have[i], k0);
+                        r[i] = rr;
+                        if (rr >= 0) used |= 1u << rr;
+                    }
+                int k = 0;
+                for (int i = 0; i < 16; ++i) {
+                    if (r[i] >= 0) {
+                        at(p, 16 * grp + i) = q[i][r[i]][head[i][r[i]]++];
+                        if (head[i][r[i]] == q[i][r[i]].size()) have[i] &= ~(1u << r[i]);
+                        --left[i];
+                    } else {
+                        unsigned f = ~used & 0xFFFFu;
+                        for (int t = 0; t < k && f; ++t) f &= f - 1;
+                        at(p, 16 * grp + i) = (unsigned short)(tc + (f ? __builtin_ctz(f) : (k & 15)));
+                        ++k;
+                    }
+                }
+            }
+        }
     }
 }
 
@@ -726,7 +762,7 @@ int core_layout_build(const int *ptr, const int *col, int rows, int lb, int core
         }
     }
     L.core_nnz = core_nnz;
-    core_bank_order(L.idx.data(), L.blk_off.data(), (size_t)nslices * ntiles);
+    core_bank_order(L.idx.data(), L.blk_off.data(), (size_t)nslices * ntiles, tc);
     return MGGX_OK;
 }
 

@@ -32,8 +32,8 @@ static inline uint64_t rnd64(uint64_t seed, uint64_t i, uint64_t j)
 // Dense-core layout of a local CSR (host arrays).  The `core` highest-degree rows, ranked by degree (ties by id), form
 // a core x core block whose edges leave the CSR and are stored as sliced ELL lists: slice g = ranks [64 g, 64 g + 64),
 // tile t = core columns (by rank) [tc t, tc t + tc); block (g, t) holds, per lane (= rank inside the slice), the tile
-// offsets of that row's neighbors inside the tile in bank order (core_bank_order), 0xFFFF-padded to the longest list of
-// the slice rounded up to 4:
+// offsets of that row's neighbors inside the tile and padding slots (tc + r, r < 16: zero columns behind the tile) up to
+// the longest list of the slice rounded up to 4, in bank order (core_bank_order):
 // idx[((blk_off[g * ntiles + t] + k / 4) * 64 + lane) * 4 + k % 4].  Every other edge stays in (rem_ptr, rem_col),
 // row order and edge order kept, column ids unchanged.
 struct CoreLayout {

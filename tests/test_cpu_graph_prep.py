@@ -293,28 +293,57 @@ def test_compact_remote_staging_order(seed):
         host.compact_remote(np.array([3, -1], np.int32))
 
 
-def _bank_order(entries, lane):
-    """A list of tile offsets in edge order -> the order the library stores it in (see test_dense_core_layout)."""
-    out = []
-    for w0 in range(0, len(entries), 64):
-        win = list(entries[w0:w0 + 64])
-        queues = [[e for e in win if e % 8 == g] for g in range(8)]
-        g = lane % 8
-        for _ in win:
-            while not queues[g]:
-                g = (g + 1) % 8
-            out.append(queues[g].pop(0))
-            g = (g + 1) % 8
-    return np.array(out, dtype=np.int64)
+def _first_from(mask, k):
+    """The lowest set bit of a 16-bit mask when looking from bit k upwards, cyclically; -1 if the mask is empty."""
+    if mask == 0:
+        return -1
+    m = ((mask >> k) | (mask << (16 - k))) & 0xFFFF
+    return ((m & -m).bit_length() - 1 + k) & 15
+
+
+def _bank_order(lists, P, tile):
+    """16 lists of tile offsets in edge order (the lanes of a group) and the block's length P -> [P][16] as the library
+    stores the block (see test_dense_core_layout)."""
+    if P > 256:   # longer than the library re-orders: edge order, padding on the first zero column
+        return np.array([[e[p] if p < len(e) else tile for e in lists] for p in range(P)], np.int64)
+    q = [[[x for x in e if x % 16 == r] for r in range(16)] for e in lists]
+    left = [len(e) for e in lists]
+    out = np.zeros((P, 16), np.int64)
+    for p in range(P):
+        used, r = 0, [-1] * 16
+        for first in (True, False):
+            for i in range(16):
+                slack = P - p - left[i]
+                if left[i] == 0 or (slack == 0) != first:
+                    continue
+                have = sum(1 << k for k in range(16) if q[i][k])
+                rr = _first_from(have & ~used, (i + p) % 16)
+                if rr < 0 and slack == 0:
+                    rr = _first_from(have, (i + p) % 16)
+                r[i] = rr
+                if rr >= 0:
+                    used |= 1 << rr
+        free = [k for k in range(16) if not (used >> k) & 1]
+        npad = 0
+        for i in range(16):
+            if r[i] >= 0:
+                out[p, i] = q[i][r[i]].pop(0)
+                left[i] -= 1
+            else:
+                out[p, i] = tile + (free[npad] if npad < len(free) else npad % 16)
+                npad += 1
+    return out
 
 
 @pytest.mark.parametrize("lb,core_rows,tile", [(0, 1024, 256), (0, 1700, 256), (300, 512, 64)])
 def test_dense_core_layout(lb, core_rows, tile):
     """The core x core block as index lists plus the remaining CSR, against numpy: ranks by degree (ties by id), every
-    core edge exactly once in the list of its (slice, tile) block at the right tile offset, the list in bank order
-    (windows of 64 entries; inside a window position p takes the next entry, in edge order, whose column is
-    (lane + p) mod 8 mod 8, or of the next residue that still has one), padding only behind the entries, everything else
-    left in the CSR in its order."""
+    core edge exactly once in the list of its (slice, tile) block at the right tile offset, the block in bank order (the
+    16 lanes of a group placed together, position by position: lanes without padding left to spend first, then the
+    others, each in lane order; a lane takes its first remaining entry, looking from residue (lane + p) mod 16 upwards,
+    whose residue mod 16 is not taken at this position, else spends a padding slot, else repeats a residue; padding
+    slots point at the zero columns tile + r for the residues r still free, in turn), everything else left in the CSR
+    in its order."""
     V = 4000
     ptr, col = host.gen_rmat(12, V, 120_000, seed=4)
     col = (col + lb).astype(np.int32)  # a share whose rows start at lb: ids are global
@@ -340,17 +369,20 @@ def test_dense_core_layout(lb, core_rows, tile):
     ntiles, off, idx = L["ntiles"], L["blk_off"].astype(np.int64), L["idx"]
     assert len(off) == core // 64 * ntiles + 1 and len(idx) == off[-1] * 256 and np.all(np.diff(off) >= 0)
     seen = 0
-    for i in (list(range(0, core, 37)) + [core - 1]):
-        v = order[i]
-        nb = rank[col[ptr[v]:ptr[v + 1]] - lb]
-        nb = nb[nb >= 0]
+    for grp in (list(range(0, core // 16, 5)) + [core // 16 - 1]):   # groups of 16 lanes: ranks 16 grp .. 16 grp + 15
+        nbs = []
+        for i in range(16 * grp, 16 * grp + 16):
+            v = order[i]
+            nb = rank[col[ptr[v]:ptr[v + 1]] - lb]
+            nbs.append(nb[nb >= 0])
+        g, l0 = grp // 4, 16 * (grp % 4)
         for t in range(ntiles):
-            want = nb[nb // tile == t] % tile
-            b0, b1 = off[(i // 64) * ntiles + t], off[(i // 64) * ntiles + t + 1]
-            got = idx[b0 * 256:b1 * 256].reshape(-1, 64, 4)[:, i % 64, :].reshape(-1)
-            assert len(want) <= len(got)
-            assert np.array_equal(got[:len(want)], _bank_order(want, i % 64)) and np.all(got[len(want):] == 0xFFFF)
-            seen += len(want)
+            want = [[int(x) for x in nb[nb // tile == t] % tile] for nb in nbs]
+            b0, b1 = off[g * ntiles + t], off[g * ntiles + t + 1]
+            got = idx[b0 * 256:b1 * 256].reshape(-1, 64, 4).transpose(0, 2, 1).reshape(-1, 64)[:, l0:l0 + 16]   # [position][lane]
+            assert max(len(w) for w in want) <= len(got)
+            assert np.array_equal(got, _bank_order(want, len(got), tile))
+            seen += sum(len(w) for w in want)
     assert seen > 0
     # every block is as long as its longest list, rounded up to 4
     cnt = np.zeros((core, ntiles), np.int64)
